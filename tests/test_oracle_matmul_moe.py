@@ -1,0 +1,209 @@
+"""Pins for the oracle's matmul, routing and MoE combine (no GPU)."""
+import numpy as np
+import pytest
+
+from gllm_amd.synth import random_activations, random_gate_logits, random_weight
+from oracle import npref
+
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+ALL = [Q8_0, Q4_K, Q5_K, Q6_K]
+
+
+def rel_l2(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
+
+
+# ------------------------------------------------------------------- matmul
+@pytest.mark.parametrize("dtype", ALL)
+def test_matmul_equals_dequant_then_float64_matmul(oracle, dtype):
+    m, n, k = 3, 17, 512
+    w, x = random_weight(dtype, n, k, seed=2), random_activations(m, k, seed=2)
+    want = npref.quantized_matmul(w, x, dtype, m, n, k)
+    got64 = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64)
+    got32 = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F32)
+    assert np.array_equal(got64, want.astype(np.float32))
+    assert rel_l2(got32, want) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_unit_vector_returns_a_weight_column_bit_exactly(oracle, dtype):
+    n, k = 9, 512
+    w = random_weight(dtype, n, k, seed=4)
+    deq = oracle.dequantize(w, dtype).reshape(n, k)
+    for col in (0, 31, 32, 255, 256, 300, 511):
+        x = np.zeros((1, k), np.float32)
+        x[0, col] = 1.0
+        for acc in (oracle.ACC_F32, oracle.ACC_F64):
+            y = oracle.quantized_matmul(w, x, dtype, 1, n, k, acc=acc)
+            assert np.array_equal(y[0].view(np.uint32), deq[:, col].view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q6_K])
+def test_linearity_and_row_permutation(oracle, dtype):
+    n, k = 12, 768
+    w = random_weight(dtype, n, k, seed=6)
+    x1, x2 = random_activations(1, k, seed=1), random_activations(1, k, seed=2)
+    y1 = oracle.quantized_matmul(w, x1, dtype, 1, n, k)
+    y2 = oracle.quantized_matmul(w, x2, dtype, 1, n, k)
+    y12 = oracle.quantized_matmul(w, 2.0 * x1 - 0.5 * x2, dtype, 1, n, k)
+    assert rel_l2(y12, 2.0 * y1.astype(np.float64) - 0.5 * y2) < 1e-6
+    rb = oracle.row_bytes(dtype, k)
+    perm = np.random.default_rng(0).permutation(n)
+    wp = w.reshape(n, rb)[perm].reshape(-1)
+    assert np.array_equal(oracle.quantized_matmul(wp, x1, dtype, 1, n, k), y1[:, perm])
+
+
+@pytest.mark.parametrize("dtype,k", [(Q4_K, 300), (Q6_K, 257), (Q8_0, 40), (Q5_K, 511)])
+def test_row_padding_is_dropped(oracle, dtype, k):
+    # src/compat/weight_helpers.rs:42-71: rows are whole blocks; elements past k are padding
+    n = 5
+    w = random_weight(dtype, n, k, seed=9)
+    bs = oracle.block_size(dtype)
+    kp = -(-k // bs) * bs
+    assert w.size == n * oracle.row_bytes(dtype, k)
+    x = random_activations(2, k, seed=9)
+    xp = np.zeros((2, kp), np.float32)
+    xp[:, :k] = x
+    a = oracle.quantized_matmul(w, x, dtype, 2, n, k)
+    b = oracle.quantized_matmul(w, xp, dtype, 2, n, kp)
+    assert np.array_equal(a, b)
+    assert np.array_equal(a, npref.quantized_matmul(w, x, dtype, 2, n, k).astype(np.float32))
+
+
+def test_threads_do_not_change_results(oracle):
+    m, n, k = 2, 64, 1024
+    w, x = random_weight(Q4_K, n, k, seed=3), random_activations(m, k, seed=3)
+    for acc in (oracle.ACC_F32, oracle.ACC_F64):
+        one = oracle.quantized_matmul(w, x, Q4_K, m, n, k, acc=acc, threads=1)
+        many = oracle.quantized_matmul(w, x, Q4_K, m, n, k, acc=acc, threads=5)
+        assert np.array_equal(one, many)
+
+
+def test_bf16_operand_variant(oracle):
+    m, n, k = 4, 16, 512
+    w, x = random_weight(Q4_K, n, k, seed=8), random_activations(m, k, seed=8)
+    wf = npref.bf16_rne(npref.dequantize(w, Q4_K)).reshape(n, k).astype(np.float64)
+    want = npref.bf16_rne(x).astype(np.float64) @ wf.T
+    got = oracle.quantized_matmul_bf16(w, x, Q4_K, m, n, k)
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+def test_baseline_config1_shape_runs_on_the_cpu_path(oracle):
+    # BASELINE config 0: Q4_K M=1 K=4096 N=4096, the reference's CPU-runnable case
+    n = k = 4096
+    w, x = random_weight(Q4_K, n, k, seed=0), random_activations(1, k, seed=0)
+    assert w.size == 9_437_184
+    y32 = oracle.quantized_matmul(w, x, Q4_K, 1, n, k, acc=oracle.ACC_F32, threads=8)
+    y64 = oracle.quantized_matmul(w, x, Q4_K, 1, n, k, acc=oracle.ACC_F64, threads=8)
+    assert rel_l2(y32, y64) < 1e-5
+    rows = [0, 1, 77, 4095]
+    rb = oracle.row_bytes(Q4_K, k)
+    sub = np.concatenate([w[r * rb:(r + 1) * rb] for r in rows])
+    assert np.array_equal(y64[0, rows], npref.quantized_matmul(sub, x, Q4_K, 1, len(rows), k)[0].astype(np.float32))
+
+
+# ------------------------------------------------------------------ routing
+def test_topk_indices_reference_vector(oracle):
+    # src/moe/routing.rs:462-466, :761-767, :1002-1012
+    assert oracle.topk_indices([0.1, 0.5, 0.3, 0.9, 0.2], 2).tolist() == [3, 1]
+    assert oracle.topk_indices([0.5, 0.3], 5).tolist() == [0, 1]
+    assert oracle.topk_indices([1.0, 2.0, 3.0], 0).size == 0
+    assert oracle.topk_indices([], 3).size == 0
+
+
+def test_topk_with_weights_reference_vectors(oracle):
+    # src/moe/routing.rs:469-478
+    idx, w = oracle.topk_with_weights([1.0, 2.0, 3.0], 2)
+    assert idx.tolist() == [2, 1] and abs(float(w.sum()) - 1.0) < 1e-6
+    e = np.exp(np.array([2.0, 3.0]) - 3.0)
+    assert np.allclose(w, (e / e.sum())[::-1], atol=1e-6)
+    # :770-779 equal logits: equal weights; stable sort keeps the lower index first
+    idx, w = oracle.topk_with_weights([1.0, 1.0, 1.0], 2)
+    assert idx.tolist() == [0, 1] and abs(w[0] - w[1]) < 1e-7 and abs(w.sum() - 1) < 1e-6
+    assert oracle.topk_with_weights([1.0, 2.0, 3.0], 0)[0].size == 0
+    assert oracle.topk_with_weights([], 3)[0].size == 0
+
+
+def test_softmax_reference_vectors(oracle):
+    # src/moe/routing.rs:481-489, :742-758
+    p = oracle.softmax([1.0, 2.0, 3.0])
+    assert abs(p.sum() - 1) < 1e-5 and p[2] > p[1] > p[0]
+    assert np.allclose(p, np.exp([1.0, 2.0, 3.0]) / np.exp([1.0, 2.0, 3.0]).sum(), atol=1e-7)
+    assert abs(oracle.softmax([5.0])[0] - 1.0) < 1e-6
+    assert np.allclose(oracle.softmax([0.0, 0.0, 0.0]), 1 / 3, atol=1e-6)
+    z = random_gate_logits(1, 128, seed=3)[0]
+    assert np.allclose(oracle.softmax(z), npref.softmax(z), rtol=1e-6, atol=1e-9)
+
+
+def test_expert_capacity_reference_vectors(oracle):
+    # src/moe/routing.rs:543-547, :724-739, :983-992
+    assert oracle.expert_capacity(1.25, 128, 8) == 20
+    assert oracle.expert_capacity(1.25, 100, 1) == 125
+    assert oracle.expert_capacity(1.25, 0, 8) == 0
+    assert oracle.expert_capacity(1.0, 10, 3) == 4
+    assert oracle.expert_capacity(-1.0, 10, 3) == 0
+    # 16 tokens over 128 experts at the default factor: one slot per expert
+    assert oracle.expert_capacity(1.25, 16, 128) == 1
+
+
+def test_route_table_capacity_and_fallback(oracle):
+    # src/moe/routing.rs:516-540: four tokens all prefer expert 0, capacity 1
+    r = oracle.route(np.array([[10.0, 0.0]] * 4, np.float32), top_k=1, capacity_factor=0.5)
+    assert r["overflow"] == 3 and r["len"].tolist() == [1, 1, 1, 1]
+    # the fallback takes the least-loaded expert (first minimum) and ignores capacity, :135-148
+    assert r["expert"][:, 0].tolist() == [0, 1, 0, 1]
+    assert r["weight"][:, 0].tolist() == [1.0, 1.0, 1.0, 1.0]
+    assert r["pos"][:, 0].tolist() == [0, 0, 1, 1] and r["counts"].tolist() == [2, 2]
+    # :550-568
+    lg = np.array([[0, 0, 100, 0], [0, 100, 0, 0], [0, 0, 100, 0]], np.float32)
+    r = oracle.route(lg, top_k=1, capacity_factor=8.0)
+    assert r["expert"][:, 0].tolist() == [2, 1, 2] and r["pos"][:, 0].tolist() == [0, 0, 1]
+
+
+def test_route_matches_numpy_topk_on_seeded_logits(oracle):
+    lg = random_gate_logits(16, 128, seed=0)
+    r = oracle.route(lg, top_k=8, capacity_factor=8.0)
+    assert r["overflow"] == 0 and np.all(r["len"] == 8)
+    for t in range(16):
+        idx, w = npref.topk_with_weights(lg[t], 8)
+        assert r["expert"][t].tolist() == idx.tolist()
+        assert np.allclose(r["weight"][t], w, rtol=1e-5)
+        assert abs(r["weight"][t].sum() - 1) < 1e-5
+
+
+# ---------------------------------------------------------------------- MoE
+def test_moe_dispatch_reference_vector(oracle):
+    # src/moe/routing.rs:646-659: outputs are constants per expert, so the combine is visible
+    idx, w = oracle.topk_with_weights([0.0, 1.0, 0.5], 2)
+    outs = np.array([[1.0, 1.0], [2.0, 2.0], [1.5, 1.5]])
+    mix = sum(w[i] * outs[idx[i]] for i in range(2))
+    assert idx.tolist() == [1, 2] and 1.5 < mix[0] < 2.0
+
+
+@pytest.mark.parametrize("relu_gate", [False, True])
+def test_moe_ffn_equals_dense_masked_evaluation(oracle, relu_gate):
+    # brute force: run every expert on every token and mask, which is what the reference
+    # graph does (build_graph.inc.rs:2119-2123)
+    tokens, hidden, ffn, experts, top_k = 3, 256, 512, 4, 2
+    gu = np.concatenate([random_weight(Q4_K, 2 * ffn, hidden, seed=10 + e) for e in range(experts)])
+    dn = np.concatenate([random_weight(Q6_K, hidden, ffn, seed=20 + e) for e in range(experts)])
+    x = random_activations(tokens, hidden, seed=1)
+    r = oracle.route(random_gate_logits(tokens, experts, seed=1), top_k, capacity_factor=8.0)
+    got = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"],
+                         relu_gate=relu_gate)
+    gu_f = npref.dequantize(gu, Q4_K).reshape(experts, 2 * ffn, hidden).astype(np.float64)
+    dn_f = npref.dequantize(dn, Q6_K).reshape(experts, hidden, ffn).astype(np.float64)
+    gate_w = np.zeros((tokens, experts))
+    for t in range(tokens):
+        for i in range(r["len"][t]):
+            gate_w[t, r["expert"][t, i]] = r["weight"][t, i]
+    want = np.zeros((tokens, hidden))
+    for e in range(experts):
+        g = x.astype(np.float64) @ gu_f[e, :ffn].T
+        u = x.astype(np.float64) @ gu_f[e, ffn:].T
+        if relu_gate:
+            g = np.maximum(g, 0)
+        h = (g / (1 + np.exp(-g))) * u
+        want += gate_w[:, e:e + 1] * (h @ dn_f[e].T)
+    assert rel_l2(got, want) < 2e-6
