@@ -163,7 +163,7 @@ def test_route_table_capacity_and_fallback(oracle):
 
 def test_route_matches_numpy_topk_on_seeded_logits(oracle):
     lg = random_gate_logits(16, 128, seed=0)
-    r = oracle.route(lg, top_k=8, capacity_factor=8.0)
+    r = oracle.route(lg, top_k=8, capacity_factor=128.0)
     assert r["overflow"] == 0 and np.all(r["len"] == 8)
     for t in range(16):
         idx, w = npref.topk_with_weights(lg[t], 8)
