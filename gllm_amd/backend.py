@@ -1,0 +1,243 @@
+"""Host-side mirror of the reference's backend interface for the quantized matmul path.
+
+``HipBackend.quantized_matmul`` / ``HipBackend.dequantize`` keep the names, argument
+order and error behaviour of ``Backend::quantized_matmul`` / ``Backend::dequantize``
+(reference: src/compat/mod.rs:233-256; CPU implementation src/compat/cpu_backend.rs:991-1159;
+error enum src/engine/executor_types.rs:322-329).  All arithmetic happens in
+``libgllm_hip_quant.so`` (hand-written gfx950 kernels behind a C ABI, see
+``include/gllm_hip_quant.h``); this module only moves pointers.  There is no CPU fallback:
+without the library or without a GPU every call raises.
+
+Buffers may be host slices (``bytes`` / numpy arrays, as in the reference's signature) or
+torch tensors that already live on the GPU.  torch is used for device memory and streams only.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+from .ggml import GgmlDType, QuantType, block_bytes, block_size, row_bytes, supported
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libgllm_hip_quant.so")
+
+OK, ERR_UNIMPLEMENTED, ERR_BAD_SHAPE, ERR_BAD_ALIGNMENT, ERR_HIP, ERR_INVALID = range(6)
+ACT_F32_SPLIT, ACT_BF16 = 0, 1
+
+
+class BackendError(Exception):
+    """``BackendError`` of the reference; subclasses are its variants."""
+
+
+class Unimplemented(BackendError):
+    pass
+
+
+class HipError(BackendError):
+    pass
+
+
+class OtherError(BackendError):
+    pass
+
+
+class MatmulDesc(C.Structure):
+    _fields_ = [("w_dev", C.c_void_p), ("w_bytes", C.c_size_t), ("x_dev", C.c_void_p),
+                ("y_dev", C.c_void_p), ("ggml_dtype", C.c_uint32), ("reserved", C.c_uint32),
+                ("m", C.c_size_t), ("n", C.c_size_t), ("k", C.c_size_t)]
+
+
+_lib = None
+
+
+def load_library() -> C.CDLL:
+    """dlopen the in-tree library and declare every prototype of the public header."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise HipError(f"{LIB_PATH} is missing: build it with `python -m gllm_amd.build`")
+    try:  # when torch is in the process, its HIP runtime must be the one the library binds to
+        import torch  # noqa: F401
+    except ImportError:  # the library runs without torch (host-pointer entry points)
+        pass
+    L = C.CDLL(LIB_PATH)
+    vp, sz, u32 = C.c_void_p, C.c_size_t, C.c_uint32
+    L.gllmq_init.restype = C.c_int
+    L.gllmq_init.argtypes = [C.POINTER(vp), C.c_int]
+    L.gllmq_destroy.restype = None
+    L.gllmq_destroy.argtypes = [vp]
+    L.gllmq_last_error.restype = C.c_char_p
+    L.gllmq_last_error.argtypes = [vp]
+    L.gllmq_status_string.restype = C.c_char_p
+    L.gllmq_status_string.argtypes = [C.c_int]
+    L.gllmq_version.restype = C.c_char_p
+    L.gllmq_version.argtypes = []
+    for name in ("gllmq_block_size", "gllmq_block_bytes"):
+        getattr(L, name).restype = sz
+        getattr(L, name).argtypes = [u32]
+    L.gllmq_row_bytes.restype = sz
+    L.gllmq_row_bytes.argtypes = [u32, sz]
+    L.gllmq_dequantize.restype = C.c_int
+    L.gllmq_dequantize.argtypes = [vp, vp, sz, vp, sz, u32, vp]
+    L.gllmq_quantized_matmul.restype = C.c_int
+    L.gllmq_quantized_matmul.argtypes = [vp, vp, sz, vp, vp, u32, sz, sz, sz, vp]
+    L.gllmq_quantized_matmul_ex.restype = C.c_int
+    L.gllmq_quantized_matmul_ex.argtypes = [vp, vp, sz, vp, vp, u32, sz, sz, sz, C.c_int, vp]
+    L.gllmq_quantized_matmul_batch.restype = C.c_int
+    L.gllmq_quantized_matmul_batch.argtypes = [vp, C.POINTER(MatmulDesc), sz, vp]
+    L.gllmq_moe_matvec.restype = C.c_int
+    L.gllmq_moe_matvec.argtypes = [vp, vp, u32, vp, u32, vp, vp, sz, sz, sz, sz, sz, vp, vp, vp, C.c_int, vp]
+    L.gllmq_dequantize_host.restype = C.c_int
+    L.gllmq_dequantize_host.argtypes = [vp, vp, sz, vp, sz, u32]
+    L.gllmq_quantized_matmul_host.restype = C.c_int
+    L.gllmq_quantized_matmul_host.argtypes = [vp, vp, sz, vp, vp, u32, sz, sz, sz]
+    _lib = L
+    return L
+
+
+EXPORTED_SYMBOLS = [
+    "gllmq_init", "gllmq_destroy", "gllmq_last_error", "gllmq_status_string", "gllmq_version",
+    "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
+    "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
+    "gllmq_moe_matvec", "gllmq_dequantize_host", "gllmq_quantized_matmul_host",
+]
+
+
+def _dtype_id(quant_type) -> int:
+    if isinstance(quant_type, QuantType):
+        return quant_type.ggml_dtype
+    return int(quant_type)
+
+
+def _is_torch(t) -> bool:
+    return type(t).__module__.startswith("torch")
+
+
+def _host_bytes(buf) -> np.ndarray:
+    if isinstance(buf, np.ndarray):
+        return np.ascontiguousarray(buf).reshape(-1).view(np.uint8)
+    return np.frombuffer(buf, dtype=np.uint8)
+
+
+class HipBackend:
+    """The MI355X backend for ``Op::QuantGemm``: quantized weights x f32 activations."""
+
+    def __init__(self, device: int = 0):
+        self._lib = load_library()
+        import torch
+        if not torch.cuda.is_available():
+            raise HipError("no HIP device is visible; this backend has no CPU path")
+        self._torch = torch
+        self.device = device
+        ctx = C.c_void_p()
+        rc = self._lib.gllmq_init(C.byref(ctx), device)
+        if rc != OK:
+            raise HipError(f"gllmq_init(device={device}): {self._lib.gllmq_status_string(rc).decode()}")
+        self._ctx = ctx
+
+    def close(self) -> None:
+        if getattr(self, "_ctx", None):
+            self._lib.gllmq_destroy(self._ctx)
+            self._ctx = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ------------------------------------------------------------------ helpers
+    def _raise(self, rc: int, what: str):
+        msg = self._lib.gllmq_last_error(self._ctx).decode(errors="replace") or what
+        if rc == ERR_UNIMPLEMENTED:
+            raise Unimplemented(msg)
+        if rc == ERR_HIP:
+            raise HipError(msg)
+        raise OtherError(f"{self._lib.gllmq_status_string(rc).decode()}: {msg}")
+
+    def _stream(self):
+        return C.c_void_p(self._torch.cuda.current_stream(self.device).cuda_stream)
+
+    def upload_weights(self, weight_blocks):
+        """Raw GGUF block bytes -> device buffer, untouched (the reference passes quantized
+        tensors through verbatim, src/engine/executor_compile.rs:207-211)."""
+        host = _host_bytes(weight_blocks)
+        return self._torch.from_numpy(host.copy()).to(f"cuda:{self.device}")
+
+    # ------------------------------------------------------------ trait methods
+    def quantized_matmul(self, weight_blocks, input, output, quant_type, m: int, n: int, k: int,
+                         act_mode: int = ACT_F32_SPLIT) -> None:
+        """output[m x n] = input[m x k] . W[n x k]^T, W given as raw GGUF blocks."""
+        dt = _dtype_id(quant_type)
+        if _is_torch(weight_blocks):
+            w, x, y = weight_blocks, input, output
+            if not (w.is_cuda and x.is_cuda and y.is_cuda):
+                raise OtherError("quantized_matmul: tensors must live on the GPU")
+            if x.dtype != self._torch.float32 or y.dtype != self._torch.float32:
+                raise Unimplemented("quantized_matmul: activations and outputs are f32 on this backend")
+            if not (w.is_contiguous() and x.is_contiguous() and y.is_contiguous()):
+                raise OtherError("quantized_matmul: tensors must be contiguous")
+            if x.numel() < m * k or y.numel() < m * n:
+                raise OtherError("quantized_matmul: input/output shorter than m*k / m*n")
+            rc = self._lib.gllmq_quantized_matmul_ex(
+                self._ctx, w.data_ptr(), w.numel() * w.element_size(), x.data_ptr(), y.data_ptr(),
+                dt, m, n, k, act_mode, self._stream())
+        else:
+            w = _host_bytes(weight_blocks)
+            x = np.ascontiguousarray(input, np.float32).reshape(-1)
+            if not (isinstance(output, np.ndarray) and output.dtype == np.float32 and output.flags.c_contiguous):
+                raise OtherError("quantized_matmul: output must be a contiguous float32 numpy array")
+            if x.size < m * k or output.size < m * n:
+                raise OtherError("quantized_matmul: input/output shorter than m*k / m*n")
+            rc = self._lib.gllmq_quantized_matmul_host(
+                self._ctx, w.ctypes.data, w.size, x.ctypes.data, output.ctypes.data, dt, m, n, k)
+        if rc != OK:
+            self._raise(rc, "quantized_matmul")
+
+    def dequantize(self, block_data, output, quant_type) -> None:
+        """Whole blocks of ``block_data`` -> f32 into ``output`` (chunks_exact on both sides)."""
+        dt = _dtype_id(quant_type)
+        if _is_torch(block_data):
+            b, o = block_data, output
+            if not (b.is_cuda and o.is_cuda and o.dtype == self._torch.float32):
+                raise OtherError("dequantize: tensors must live on the GPU, output f32")
+            rc = self._lib.gllmq_dequantize(self._ctx, b.data_ptr(), b.numel() * b.element_size(),
+                                            o.data_ptr(), o.numel(), dt, self._stream())
+        else:
+            b = _host_bytes(block_data)
+            if not (isinstance(output, np.ndarray) and output.dtype == np.float32 and output.flags.c_contiguous):
+                raise OtherError("dequantize: output must be a contiguous float32 numpy array")
+            rc = self._lib.gllmq_dequantize_host(self._ctx, b.ctypes.data, b.size, output.ctypes.data,
+                                                 output.size, dt)
+        if rc != OK:
+            self._raise(rc, "dequantize")
+
+    # --------------------------------------------------------------- extensions
+    def quantized_matmul_batch(self, descs) -> None:
+        """descs: iterable of (w, x, y, quant_type, m, n, k) device tensors; one C call."""
+        items = list(descs)
+        arr = (MatmulDesc * len(items))()
+        for i, (w, x, y, qt, m, n, k) in enumerate(items):
+            arr[i] = MatmulDesc(w.data_ptr(), w.numel() * w.element_size(), x.data_ptr(), y.data_ptr(),
+                                _dtype_id(qt), 0, m, n, k)
+        rc = self._lib.gllmq_quantized_matmul_batch(self._ctx, arr, len(items), self._stream())
+        if rc != OK:
+            self._raise(rc, "quantized_matmul_batch")
+
+    def moe_matvec(self, gate_up, dtype_gate_up, down, dtype_down, x, out, hidden: int, ffn: int,
+                   experts: int, route_expert, route_weight, route_len, relu_gate: bool = False) -> None:
+        tokens, top_k = route_expert.shape
+        rc = self._lib.gllmq_moe_matvec(
+            self._ctx, gate_up.data_ptr(), _dtype_id(dtype_gate_up), down.data_ptr(), _dtype_id(dtype_down),
+            x.data_ptr(), out.data_ptr(), tokens, hidden, ffn, experts, top_k, route_expert.data_ptr(),
+            route_weight.data_ptr(), route_len.data_ptr(), int(relu_gate), self._stream())
+        if rc != OK:
+            self._raise(rc, "moe_matvec")
+
+
+__all__ = ["HipBackend", "BackendError", "Unimplemented", "HipError", "OtherError", "QuantType",
+           "GgmlDType", "block_size", "block_bytes", "row_bytes", "supported", "load_library",
+           "EXPORTED_SYMBOLS", "ACT_F32_SPLIT", "ACT_BF16", "LIB_PATH"]

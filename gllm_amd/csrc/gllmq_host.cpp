@@ -1,0 +1,439 @@
+// Host side of libgllm_hip_quant.so: the C ABI of include/gllm_hip_quant.h over the
+// embedded gfx950 code object.  Kernels are launched with hipModuleLaunchKernel on the
+// caller's stream, the driver-style convention the reference's HIP backend uses
+// (src/compat/hip_backend.rs:211-238), except that the module is loaded and every
+// function resolved once per context instead of once per launch.
+#include "gllm_hip_quant.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+// The code object built from gllmq_kernels.hip, placed in .rodata by the assembler.
+__asm__(".section .rodata\n"
+        ".balign 4096\n"
+        ".global gllmq_code_object_begin\n"
+        "gllmq_code_object_begin:\n"
+        ".incbin \"" GLLMQ_HSACO_PATH "\"\n"
+        ".global gllmq_code_object_end\n"
+        "gllmq_code_object_end:\n"
+        ".byte 0\n"
+        ".previous\n");
+extern "C" const unsigned char gllmq_code_object_begin[];
+extern "C" const unsigned char gllmq_code_object_end[];
+
+namespace {
+
+constexpr uint32_t T_Q8_0 = GLLMQ_TYPE_Q8_0, T_Q4_K = GLLMQ_TYPE_Q4_K, T_Q5_K = GLLMQ_TYPE_Q5_K,
+                   T_Q6_K = GLLMQ_TYPE_Q6_K;
+
+struct Format {
+    uint32_t dtype;
+    size_t block_size, block_bytes;
+    size_t group_bytes; // bytes of 256 elements
+    size_t w_align;
+    const char *tag;
+};
+
+const Format kFormats[] = {
+    { T_Q8_0, 32, 34, 272, 2, "q8_0" },
+    { T_Q4_K, 256, 144, 144, 16, "q4k" },
+    { T_Q5_K, 256, 176, 176, 16, "q5k" },
+    { T_Q6_K, 256, 210, 210, 2, "q6k" },
+};
+constexpr int kNumFormats = 4;
+
+const Format *find_format(uint32_t dtype)
+{
+    for (const Format &f : kFormats)
+        if (f.dtype == dtype) return &f;
+    return nullptr;
+}
+
+int format_index(uint32_t dtype)
+{
+    for (int i = 0; i < kNumFormats; ++i)
+        if (kFormats[i].dtype == dtype) return i;
+    return -1;
+}
+
+// Mirror of gq::GemvParams in gemv.hip.inc.
+struct GemvParams {
+    const uint8_t *w;
+    const float *x;
+    float *y;
+    uint32_t n, k, groups, row_bytes, ks, rps, rows_per_wg, ldx, ldy, x_vec, accumulate;
+};
+
+} // namespace
+
+struct gllmq_ctx {
+    int device = 0;
+    hipModule_t module = nullptr;
+    hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
+    hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1]
+    int num_cus = 256;
+    uint32_t gemv_waves = 2048; // waves a GEMV launch aims to put on the device
+    std::mutex err_mutex;
+    std::string err;
+};
+
+namespace {
+
+int fail(gllmq_ctx *ctx, int code, const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (ctx) {
+        std::lock_guard<std::mutex> g(ctx->err_mutex);
+        ctx->err = buf;
+    }
+    return code;
+}
+
+#define GLLMQ_HIP(ctx, call)                                                                  \
+    do {                                                                                      \
+        hipError_t e_ = (call);                                                               \
+        if (e_ != hipSuccess)                                                                 \
+            return fail(ctx, GLLMQ_ERR_HIP, "%s failed: %s", #call, hipGetErrorString(e_));   \
+    } while (0)
+
+int get_function(gllmq_ctx *ctx, hipFunction_t *f, const char *name)
+{
+    hipError_t e = hipModuleGetFunction(f, ctx->module, name);
+    if (e != hipSuccess)
+        return fail(ctx, GLLMQ_ERR_HIP, "kernel %s missing from the code object: %s", name,
+                    hipGetErrorString(e));
+    return GLLMQ_OK;
+}
+
+int launch(gllmq_ctx *ctx, hipFunction_t f, uint32_t grid, uint32_t block, uint32_t lds, void *stream,
+           void *params, size_t params_size)
+{
+    void *config[] = { HIP_LAUNCH_PARAM_BUFFER_POINTER, params, HIP_LAUNCH_PARAM_BUFFER_SIZE,
+                       &params_size, HIP_LAUNCH_PARAM_END };
+    GLLMQ_HIP(ctx, hipModuleLaunchKernel(f, grid, 1, 1, block, 1, 1, lds, static_cast<hipStream_t>(stream),
+                                         nullptr, config));
+    return GLLMQ_OK;
+}
+
+bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// One GEMV launch over at most 64 groups (16384 elements) of K and m <= 2.
+int launch_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, size_t row_bytes, const float *x,
+                float *y, uint32_t m, uint32_t n, uint32_t k, uint32_t ldx, uint32_t ldy, bool accumulate,
+                void *stream)
+{
+    GemvParams P{};
+    P.w = w;
+    P.x = x;
+    P.y = y;
+    P.n = n;
+    P.k = k;
+    P.groups = (k + 255u) / 256u;
+    P.row_bytes = static_cast<uint32_t>(row_bytes);
+    const uint32_t parts = 4 * P.groups;
+    if (parts >= 64) {
+        P.ks = (parts + 63) / 64;
+        P.rps = 1;
+    } else {
+        P.ks = 1;
+        P.rps = 64 / parts;
+    }
+    const uint32_t rgs = std::max(1u, 4u / P.ks);
+    const uint32_t nwaves = P.ks * rgs;
+    const uint32_t row_steps = (n + P.rps - 1) / P.rps;
+    uint32_t wgs = std::max(1u, ctx->gemv_waves / nwaves);
+    wgs = std::min(wgs, (row_steps + rgs - 1) / rgs);
+    uint32_t steps_per_wg = (row_steps + wgs * rgs - 1) / (wgs * rgs);
+    P.rows_per_wg = steps_per_wg * rgs * P.rps;
+    // partial sums of a K-split row meet in LDS: keep them within 32 KiB
+    const uint32_t max_rows = 32768u / (4u * P.ks * m);
+    if (P.ks > 1 && P.rows_per_wg > max_rows) P.rows_per_wg = std::max(rgs, max_rows / rgs * rgs);
+    const uint32_t grid = (n + P.rows_per_wg - 1) / P.rows_per_wg;
+    const uint32_t lds = P.ks > 1 ? P.rows_per_wg * P.ks * m * 4u : 0u;
+    P.ldx = ldx;
+    P.ldy = ldy;
+    P.x_vec = aligned(x, 16) && (m == 1 || ldx % 4 == 0);
+    P.accumulate = accumulate ? 1u : 0u;
+    const int fi = format_index(f.dtype);
+    return launch(ctx, ctx->gemv[fi][m - 1], grid, 64 * nwaves, lds, stream, &P, sizeof P);
+}
+
+int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_bytes, const float *x,
+                      float *y, uint32_t dtype, size_t m, size_t n, size_t k)
+{
+    if (!f)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
+                    "quantized_matmul: ggml dtype %u is not covered (supported: Q8_0=8, Q4_K=12, Q5_K=13, Q6_K=14)",
+                    dtype);
+    if (m == 0 || n == 0) return GLLMQ_OK;
+    if (!w || !x || !y) return fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul: NULL device pointer");
+    if (k == 0) return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quantized_matmul: k = 0");
+    if (n > 0x7FFFFFFFu || k > 0x7FFFFFFFu || m > 0x7FFFFFFFu)
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quantized_matmul: dimension exceeds 2^31-1");
+    const size_t rb = gllmq_row_bytes(dtype, k);
+    if (w_bytes < n * rb)
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE,
+                    "quantized_matmul: weight buffer has %zu bytes, n=%zu rows of k=%zu need %zu", w_bytes, n, k,
+                    n * rb);
+    if (!aligned(w, f->w_align) || (rb % f->w_align) != 0)
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "quantized_matmul: weights of %s must be %zu-byte aligned",
+                    f->tag, f->w_align);
+    if (!aligned(x, 4) || !aligned(y, 4))
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "quantized_matmul: activations and outputs must be 4-byte aligned");
+    return -1; // go on
+}
+
+int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
+             size_t k, void *stream)
+{
+    const size_t rb = gllmq_row_bytes(f.dtype, k);
+    constexpr size_t kChunk = 16384; // elements of K one launch covers (four waves of 4096)
+    for (size_t m0 = 0; m0 < m; m0 += 2) {
+        const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(2, m - m0));
+        for (size_t k0 = 0; k0 < k; k0 += kChunk) {
+            const size_t kk = std::min(kChunk, k - k0);
+            int rc = launch_gemv(ctx, f, w + (k0 / 256) * f.group_bytes, rb, x + m0 * k + k0, y + m0 * n, mm,
+                                 static_cast<uint32_t>(n), static_cast<uint32_t>(kk), static_cast<uint32_t>(k),
+                                 static_cast<uint32_t>(n), k0 != 0, stream);
+            if (rc != GLLMQ_OK) return rc;
+        }
+    }
+    return GLLMQ_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+const char *gllmq_version(void) { return "gllm_hip_quant 0.1 (gfx950)"; }
+
+const char *gllmq_status_string(int status)
+{
+    switch (status) {
+    case GLLMQ_OK: return "ok";
+    case GLLMQ_ERR_UNIMPLEMENTED: return "unimplemented";
+    case GLLMQ_ERR_BAD_SHAPE: return "bad shape";
+    case GLLMQ_ERR_BAD_ALIGNMENT: return "bad alignment";
+    case GLLMQ_ERR_HIP: return "hip error";
+    case GLLMQ_ERR_INVALID: return "invalid argument";
+    default: return "unknown status";
+    }
+}
+
+size_t gllmq_block_size(uint32_t dtype)
+{
+    const Format *f = find_format(dtype);
+    return f ? f->block_size : 0;
+}
+
+size_t gllmq_block_bytes(uint32_t dtype)
+{
+    const Format *f = find_format(dtype);
+    return f ? f->block_bytes : 0;
+}
+
+size_t gllmq_row_bytes(uint32_t dtype, size_t k)
+{
+    const Format *f = find_format(dtype);
+    return f ? (k + f->block_size - 1) / f->block_size * f->block_bytes : 0;
+}
+
+int gllmq_init(gllmq_ctx **out, int device)
+{
+    if (!out) return GLLMQ_ERR_INVALID;
+    *out = nullptr;
+    gllmq_ctx *ctx = new gllmq_ctx;
+    ctx->device = device;
+    hipError_t e = hipSetDevice(device);
+    if (e == hipSuccess) e = hipFree(nullptr); // force context creation
+    if (e != hipSuccess) {
+        fprintf(stderr, "gllmq_init: device %d: %s\n", device, hipGetErrorString(e));
+        delete ctx;
+        return GLLMQ_ERR_HIP;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess) {
+        ctx->num_cus = prop.multiProcessorCount;
+        if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+            fprintf(stderr, "gllmq_init: device %d is %s; this library holds gfx950 code only\n", device,
+                    prop.gcnArchName);
+            delete ctx;
+            return GLLMQ_ERR_UNIMPLEMENTED;
+        }
+    }
+    e = hipModuleLoadData(&ctx->module, gllmq_code_object_begin);
+    if (e != hipSuccess) {
+        fprintf(stderr, "gllmq_init: hipModuleLoadData: %s\n", hipGetErrorString(e));
+        delete ctx;
+        return GLLMQ_ERR_HIP;
+    }
+    int rc = GLLMQ_OK;
+    char name[64];
+    for (int i = 0; i < kNumFormats && rc == GLLMQ_OK; ++i) {
+        snprintf(name, sizeof name, "gq_dequant_%s_v1", kFormats[i].tag);
+        rc = get_function(ctx, &ctx->dequant[i][0], name);
+        if (rc != GLLMQ_OK) break;
+        snprintf(name, sizeof name, "gq_dequant_%s_v4", kFormats[i].tag);
+        rc = get_function(ctx, &ctx->dequant[i][1], name);
+        for (int m = 1; m <= 2 && rc == GLLMQ_OK; ++m) {
+            snprintf(name, sizeof name, "gq_gemv_%s_m%d", kFormats[i].tag, m);
+            rc = get_function(ctx, &ctx->gemv[i][m - 1], name);
+        }
+    }
+    if (rc != GLLMQ_OK) {
+        fprintf(stderr, "gllmq_init: %s\n", ctx->err.c_str());
+        (void)hipModuleUnload(ctx->module);
+        delete ctx;
+        return rc;
+    }
+    ctx->gemv_waves = static_cast<uint32_t>(ctx->num_cus) * 8u;
+    if (const char *v = getenv("GLLMQ_GEMV_WAVES")) {
+        long w = strtol(v, nullptr, 10);
+        if (w >= 4 && w <= 65536) ctx->gemv_waves = static_cast<uint32_t>(w);
+    }
+    *out = ctx;
+    return GLLMQ_OK;
+}
+
+void gllmq_destroy(gllmq_ctx *ctx)
+{
+    if (!ctx) return;
+    if (ctx->module) (void)hipModuleUnload(ctx->module);
+    delete ctx;
+}
+
+const char *gllmq_last_error(const gllmq_ctx *ctx)
+{
+    if (!ctx) return "NULL context";
+    return ctx->err.c_str();
+}
+
+int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *out, size_t n_out,
+                     uint32_t dtype, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    const Format *f = find_format(dtype);
+    if (!f)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
+                    "dequantize: ggml dtype %u is not covered (supported: Q8_0=8, Q4_K=12, Q5_K=13, Q6_K=14)", dtype);
+    const size_t nb = std::min(n_bytes / f->block_bytes, n_out / f->block_size);
+    if (nb == 0) return GLLMQ_OK;
+    if (!blocks || !out) return fail(ctx, GLLMQ_ERR_INVALID, "dequantize: NULL device pointer");
+    if (!aligned(out, 4)) return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "dequantize: output must be 4-byte aligned");
+    uint64_t n_quads = static_cast<uint64_t>(nb) * (f->block_size / 4);
+    const int vec = aligned(out, 16) ? 1 : 0;
+    const uint64_t want = (n_quads + 255) / 256;
+    const uint32_t grid = static_cast<uint32_t>(std::min<uint64_t>(want, static_cast<uint64_t>(ctx->num_cus) * 64));
+    struct { const void *b; float *o; uint64_t n; } args = { blocks, out, n_quads };
+    return launch(ctx, ctx->dequant[format_index(dtype)][vec], grid, 256, 0, stream, &args, sizeof args);
+}
+
+int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y,
+                              uint32_t dtype, size_t m, size_t n, size_t k, int act_mode, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    const Format *f = find_format(dtype);
+    int rc = check_matmul_args(ctx, f, w, w_bytes, x, y, dtype, m, n, k);
+    if (rc >= 0) return rc;
+    (void)act_mode;
+    return run_gemv(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, stream);
+}
+
+int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y,
+                           uint32_t dtype, size_t m, size_t n, size_t k, void *stream)
+{
+    return gllmq_quantized_matmul_ex(ctx, w, w_bytes, x, y, dtype, m, n, k, GLLMQ_ACT_F32_SPLIT, stream);
+}
+
+int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs, size_t count, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    if (count && !descs) return fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul_batch: NULL descriptor list");
+    for (size_t i = 0; i < count; ++i) {
+        const gllmq_matmul_desc &d = descs[i];
+        int rc = gllmq_quantized_matmul(ctx, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k,
+                                        stream);
+        if (rc != GLLMQ_OK) return rc;
+    }
+    return GLLMQ_OK;
+}
+
+int gllmq_moe_matvec(gllmq_ctx *ctx, const void *, uint32_t, const void *, uint32_t, const float *, float *,
+                     size_t, size_t, size_t, size_t, size_t, const uint32_t *, const float *, const uint32_t *,
+                     int, void *)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "moe_matvec: not built yet");
+}
+
+int gllmq_dequantize_host(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *out, size_t n_out,
+                          uint32_t dtype)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    const Format *f = find_format(dtype);
+    if (!f) return gllmq_dequantize(ctx, blocks, n_bytes, out, n_out, dtype, nullptr);
+    const size_t nb = std::min(n_bytes / f->block_bytes, n_out / f->block_size);
+    if (nb == 0) return GLLMQ_OK;
+    void *d_in = nullptr, *d_out = nullptr;
+    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
+    GLLMQ_HIP(ctx, hipMalloc(&d_in, nb * f->block_bytes));
+    hipError_t e = hipMalloc(&d_out, nb * f->block_size * sizeof(float));
+    int rc = GLLMQ_OK;
+    if (e != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "hipMalloc: %s", hipGetErrorString(e));
+    if (rc == GLLMQ_OK && (e = hipMemcpy(d_in, blocks, nb * f->block_bytes, hipMemcpyHostToDevice)) != hipSuccess)
+        rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy H2D: %s", hipGetErrorString(e));
+    if (rc == GLLMQ_OK)
+        rc = gllmq_dequantize(ctx, d_in, nb * f->block_bytes, static_cast<float *>(d_out), nb * f->block_size,
+                              dtype, nullptr);
+    if (rc == GLLMQ_OK &&
+        (e = hipMemcpy(out, d_out, nb * f->block_size * sizeof(float), hipMemcpyDeviceToHost)) != hipSuccess)
+        rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy D2H: %s", hipGetErrorString(e));
+    (void)hipFree(d_in);
+    (void)hipFree(d_out);
+    return rc;
+}
+
+int gllmq_quantized_matmul_host(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y,
+                                uint32_t dtype, size_t m, size_t n, size_t k)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    const Format *f = find_format(dtype);
+    if (!f) return gllmq_quantized_matmul(ctx, w, w_bytes, x, y, dtype, m, n, k, nullptr);
+    if (m == 0 || n == 0) return GLLMQ_OK;
+    const size_t need = n * gllmq_row_bytes(dtype, k);
+    if (w_bytes < need)
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quantized_matmul: weight buffer has %zu bytes, need %zu", w_bytes, need);
+    void *d_w = nullptr, *d_x = nullptr, *d_y = nullptr;
+    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
+    int rc = GLLMQ_OK;
+    hipError_t e;
+    if ((e = hipMalloc(&d_w, need)) != hipSuccess || (e = hipMalloc(&d_x, m * k * sizeof(float))) != hipSuccess ||
+        (e = hipMalloc(&d_y, m * n * sizeof(float))) != hipSuccess)
+        rc = fail(ctx, GLLMQ_ERR_HIP, "hipMalloc: %s", hipGetErrorString(e));
+    if (rc == GLLMQ_OK && ((e = hipMemcpy(d_w, w, need, hipMemcpyHostToDevice)) != hipSuccess ||
+                           (e = hipMemcpy(d_x, x, m * k * sizeof(float), hipMemcpyHostToDevice)) != hipSuccess))
+        rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy H2D: %s", hipGetErrorString(e));
+    if (rc == GLLMQ_OK)
+        rc = gllmq_quantized_matmul(ctx, d_w, need, static_cast<const float *>(d_x), static_cast<float *>(d_y),
+                                    dtype, m, n, k, nullptr);
+    if (rc == GLLMQ_OK && (e = hipMemcpy(y, d_y, m * n * sizeof(float), hipMemcpyDeviceToHost)) != hipSuccess)
+        rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy D2H: %s", hipGetErrorString(e));
+    (void)hipFree(d_w);
+    (void)hipFree(d_x);
+    (void)hipFree(d_y);
+    return rc;
+}
+
+} // extern "C"

@@ -1,0 +1,10 @@
+// Single translation unit of every gfx950 kernel of the library.  It is compiled to a
+// code object (hipcc --genco) that the host library embeds and loads with
+// hipModuleLoadData; kernels are found by their extern "C" names.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "gq_device.h"
+
+#include "dequant.hip.inc"
+#include "gemv.hip.inc"

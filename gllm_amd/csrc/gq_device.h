@@ -1,0 +1,78 @@
+// Device-side helpers shared by the gfx950 kernels: block geometry, f16 decode,
+// the packed 6-bit scale/min fields of Q4_K/Q5_K and wave64 reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gq {
+
+constexpr int WAVE = 64;
+constexpr int QK_K = 256;
+
+// GgmlDType ids (reference: src/loader/gguf/types.rs:57-94)
+constexpr uint32_t T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14;
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h)
+{
+    // v_cvt_f32_f16 is IEEE for every class, subnormals included (f16 denormals are
+    // never flushed on this target).
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h & 0xFFFFu)));
+}
+
+// Loads of 2-byte aligned data as wider words.  gfx950 under the HSA ABI runs global
+// memory in unaligned-access mode, so one load instruction serves any byte address.
+template <typename T>
+__device__ __forceinline__ T load_unaligned(const void *p)
+{
+    T v;
+    __builtin_memcpy(&v, p, sizeof(T));
+    return v;
+}
+
+// (sc, m) pair j of the 12-byte field held as three little-endian dwords s0,s1,s2
+// (bytes 0-3, 4-7, 8-11).  Reference: quant-kquant-iq-proprietary.md:45-50.
+__device__ __forceinline__ void scale_min_k4(int j, uint32_t s0, uint32_t s1, uint32_t s2,
+                                             uint32_t &sc, uint32_t &mn)
+{
+    const int sh = 8 * (j & 3);
+    const uint32_t a = (s0 >> sh) & 0xFFu; // byte j&3 of scales[0..3]
+    const uint32_t b = (s1 >> sh) & 0xFFu; // byte j&3 of scales[4..7]
+    const uint32_t c = (s2 >> sh) & 0xFFu; // byte j&3 of scales[8..11]
+    if (j < 4) {
+        sc = a & 63u;
+        mn = b & 63u;
+    } else {
+        sc = (c & 0xFu) | ((a >> 6) << 4);
+        mn = (c >> 4) | ((b >> 6) << 4);
+    }
+}
+
+__device__ __forceinline__ float ubyte0(uint32_t v) { return static_cast<float>(v & 0xFFu); }
+__device__ __forceinline__ float ubyte1(uint32_t v) { return static_cast<float>((v >> 8) & 0xFFu); }
+__device__ __forceinline__ float ubyte2(uint32_t v) { return static_cast<float>((v >> 16) & 0xFFu); }
+__device__ __forceinline__ float ubyte3(uint32_t v) { return static_cast<float>(v >> 24); }
+
+// Sum over a segment of `len` consecutive lanes (len a multiple of 4, segment start a
+// multiple of 4, `pos` = lane's index inside its segment).  The total lands in the
+// lane with pos == 0; other lanes hold partial garbage.
+__device__ __forceinline__ float segment_sum(float v, int pos, int len)
+{
+    v += __shfl_xor(v, 1, WAVE);
+    v += __shfl_xor(v, 2, WAVE);
+#pragma unroll
+    for (int off = 32; off >= 4; off >>= 1) {
+        const float o = __shfl_down(v, off, WAVE);
+        if (pos + off < len) v += o;
+    }
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, WAVE);
+    return v;
+}
+
+} // namespace gq

@@ -1,0 +1,127 @@
+/*
+ * gllm_hip_quant: MI355X (gfx950) implementation of gllm's quantized-weight matmul path
+ * behind a C ABI.  Every entry point takes plain pointers and sizes; device pointers
+ * are HIP device addresses, `stream` is a hipStream_t passed as void* (NULL = the null
+ * stream).  All calls are asynchronous on `stream` unless the name ends in `_host`.
+ *
+ * Reference interfaces each entry point stands in for (paths inside putao520/gllm):
+ *   Backend::quantized_matmul  src/compat/mod.rs:233-246, CPU impl src/compat/cpu_backend.rs:991-1049
+ *   Backend::dequantize        src/compat/mod.rs:248-256, CPU impl src/compat/cpu_backend.rs:1051-1159
+ *   Op::QuantGemm contract     src/arch/auto_graph_fragments/build_graph.inc.rs:94-123
+ *   GgmlDType constants        src/loader/gguf/types.rs:57-94,152-236,443-472
+ *   MoE routing / combine      src/moe/routing.rs:100-173,263-327
+ *
+ * Shapes follow the reference: W is n rows (outputs) of k elements stored as GGUF
+ * blocks, K innermost, each row padded to whole blocks; x is [m x k], y is [m x n],
+ * row-major f32.  Supported ggml dtypes: Q8_0 (8), Q4_K (12), Q5_K (13), Q6_K (14);
+ * anything else returns GLLMQ_ERR_UNIMPLEMENTED, never a fallback
+ * (src/compat/cpu_backend.rs:1020-1046).
+ */
+#ifndef GLLM_HIP_QUANT_H
+#define GLLM_HIP_QUANT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GLLMQ_TYPE_Q8_0 8u
+#define GLLMQ_TYPE_Q4_K 12u
+#define GLLMQ_TYPE_Q5_K 13u
+#define GLLMQ_TYPE_Q6_K 14u
+
+/* Status codes.  BackendError::Unimplemented / ::Hip / ::Other of
+ * src/engine/executor_types.rs:322-329 map to UNIMPLEMENTED / HIP / the rest. */
+enum {
+    GLLMQ_OK = 0,
+    GLLMQ_ERR_UNIMPLEMENTED = 1, /* dtype or mode the library does not cover        */
+    GLLMQ_ERR_BAD_SHAPE = 2,     /* sizes inconsistent with dtype/m/n/k              */
+    GLLMQ_ERR_BAD_ALIGNMENT = 3, /* a device pointer misses the documented alignment */
+    GLLMQ_ERR_HIP = 4,           /* a HIP runtime call failed; see gllmq_last_error  */
+    GLLMQ_ERR_INVALID = 5        /* NULL context or pointer                          */
+};
+
+/* Activation rounding used by the m >= GLLMQ_GEMM_MIN_M tensor-core path. */
+enum {
+    GLLMQ_ACT_F32_SPLIT = 0, /* x carried as two f16 terms (22+ significant bits)  */
+    GLLMQ_ACT_BF16 = 1       /* x rounded to bf16 (round-to-nearest-even)          */
+};
+
+#define GLLMQ_GEMM_MIN_M 9
+
+typedef struct gllmq_ctx gllmq_ctx;
+
+/* ---- lifetime -------------------------------------------------------------------- */
+/* Loads the embedded gfx950 code object on `device` and resolves every kernel once
+ * (the reference reloads its module per launch, src/compat/hip_backend.rs:211-238). */
+int gllmq_init(gllmq_ctx **out_ctx, int device);
+void gllmq_destroy(gllmq_ctx *ctx);
+/* Message of the last failing call on this context ("" if none); valid until the next call. */
+const char *gllmq_last_error(const gllmq_ctx *ctx);
+const char *gllmq_status_string(int status);
+const char *gllmq_version(void);
+
+/* ---- format constants (GgmlDType::block_size / block_bytes / tensor_nbytes row rule) */
+size_t gllmq_block_size(uint32_t ggml_dtype);  /* 0 if unsupported */
+size_t gllmq_block_bytes(uint32_t ggml_dtype); /* 0 if unsupported */
+size_t gllmq_row_bytes(uint32_t ggml_dtype, size_t k);
+
+/* ---- Backend::dequantize ----------------------------------------------------------
+ * Decodes min(n_bytes / block_bytes, n_out / block_size) whole blocks; trailing
+ * partial chunks on either side are ignored (chunks_exact on both sides).
+ * Alignment: none required of `blocks_dev`; `out_dev` 4 bytes. */
+int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks_dev, size_t n_bytes, float *out_dev,
+                     size_t n_out, uint32_t ggml_dtype, void *stream);
+
+/* ---- Backend::quantized_matmul ----------------------------------------------------
+ * y[m x n] = x[m x k] . W[n x k]^T.  w_bytes must be at least n * gllmq_row_bytes(dtype,k).
+ * Alignment: w_dev 16 bytes for Q4_K/Q5_K, 2 bytes for Q6_K/Q8_0; x_dev 16, y_dev 4.
+ * m <= 8 runs the bandwidth (GEMV) kernels with f32 activations and f32 accumulation;
+ * larger m runs the MFMA kernels with GLLMQ_ACT_F32_SPLIT activations. */
+int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev,
+                           float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,
+                           void *stream);
+
+/* Same, with the activation mode of the MFMA path chosen by the caller (ignored for m <= 8). */
+int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes,
+                              const float *x_dev, float *y_dev, uint32_t ggml_dtype, size_t m,
+                              size_t n, size_t k, int act_mode, void *stream);
+
+/* A list of independent matmuls enqueued back to back on one stream from one call
+ * (one decode layer = QKV, O, gate/up, down: build_graph.inc.rs:1960-1999). */
+typedef struct gllmq_matmul_desc {
+    const void *w_dev;
+    size_t w_bytes;
+    const float *x_dev;
+    float *y_dev;
+    uint32_t ggml_dtype;
+    uint32_t reserved;
+    size_t m, n, k;
+} gllmq_matmul_desc;
+
+int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs, size_t count,
+                                 void *stream);
+
+/* ---- MoE expert matvec (ExpertRouteTable grouping, src/moe/routing.rs:163-173) -----
+ * out[t] = sum_i weight[t][i] * down_e( silu(gate_e x_t) * (up_e x_t) ), e = expert[t][i].
+ * gate_up_dev: per expert 2*ffn rows over `hidden` (gate rows, then up rows);
+ * down_dev: per expert `hidden` rows over `ffn`.  route_* are [tokens x top_k] device
+ * arrays, route_len[t] entries valid per token.  relu_gate != 0 applies max(g,0) first. */
+int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up_dev, uint32_t dtype_gate_up,
+                     const void *down_dev, uint32_t dtype_down, const float *x_dev, float *out_dev,
+                     size_t tokens, size_t hidden, size_t ffn, size_t experts, size_t top_k,
+                     const uint32_t *route_expert_dev, const float *route_weight_dev,
+                     const uint32_t *route_len_dev, int relu_gate, void *stream);
+
+/* ---- host-pointer convenience (upload, run, download, synchronise) ---------------- */
+int gllmq_dequantize_host(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *out,
+                          size_t n_out, uint32_t ggml_dtype);
+int gllmq_quantized_matmul_host(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x,
+                                float *y, uint32_t ggml_dtype, size_t m, size_t n, size_t k);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

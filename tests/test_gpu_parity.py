@@ -1,0 +1,187 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same inputs.
+
+Bars: dequantized weights bit-exact; matmul outputs rel-L2 <= 1e-4 and per-element
+|err| <= 1e-3 * max|y| against the oracle's float64 accumulation.
+"""
+import numpy as np
+import pytest
+
+from gllm_amd.synth import random_activations, random_blocks, random_weight
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+ALL = [Q8_0, Q4_K, Q5_K, Q6_K]
+REL_L2_TOL = 1e-4
+ELEM_TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from gllm_amd.backend import HipBackend
+    return HipBackend(0)
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+    return torch
+
+
+def check_close(got, want, what=""):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-300)
+    worst = np.abs(got - want).max() / max(np.abs(want).max(), 1e-300)
+    assert rel <= REL_L2_TOL and worst <= ELEM_TOL, f"{what}: rel_l2={rel:.3e} max_err/max|y|={worst:.3e}"
+    return rel
+
+
+def gpu_matmul(hip, torch, w, x, dtype, m, n, k):
+    wd = hip.upload_weights(w)
+    xd = torch.from_numpy(np.ascontiguousarray(x, np.float32)).cuda()
+    yd = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+    hip.quantized_matmul(wd, xd, yd, dtype, m, n, k)
+    torch.cuda.synchronize()
+    return yd.cpu().numpy()
+
+
+# ---------------------------------------------------------------- dequantize
+@pytest.mark.parametrize("dtype", ALL)
+def test_dequantize_bit_exact(hip, torch, oracle, dtype):
+    print(f"dequantize dtype={dtype}", flush=True)
+    nb = 1031
+    raw = random_blocks(dtype, nb, seed=100 + dtype)
+    blocks = raw.reshape(nb, -1)
+    off = {Q8_0: 0, Q4_K: 0, Q5_K: 0, Q6_K: 208}[dtype]
+    for i, pat in enumerate([0x0001, 0x03FF, 0x0000, 0x8000, 0xBC00, 0x7BFF, 0x0400, 0x8001]):
+        blocks[i, off:off + 2] = np.array([pat], np.uint16).view(np.uint8)
+    want = oracle.dequantize(raw, dtype)
+    bd = torch.from_numpy(raw).cuda()
+    od = torch.zeros(want.size, dtype=torch.float32, device="cuda")
+    hip.dequantize(bd, od, dtype)
+    torch.cuda.synchronize()
+    got = od.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # host-slice form of the same call (the reference's signature)
+    out = np.zeros(want.size, np.float32)
+    hip.dequantize(raw, out, dtype)
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_dequantize_partial_chunks_and_odd_alignment(hip, torch, oracle, dtype):
+    print(f"dequantize partial dtype={dtype}", flush=True)
+    bb, bs = oracle.block_bytes(dtype), oracle.block_size(dtype)
+    raw = random_blocks(dtype, 5, seed=7)
+    want = oracle.dequantize(raw, dtype)
+    # input one byte short of 5 blocks, output with room for 5: four blocks decoded
+    bd = torch.from_numpy(raw[: 5 * bb - 1].copy()).cuda()
+    od = torch.full((5 * bs,), -1.0, dtype=torch.float32, device="cuda")
+    hip.dequantize(bd, od, dtype)
+    got = od.cpu().numpy()
+    assert np.array_equal(got[: 4 * bs], want[: 4 * bs]) and np.all(got[4 * bs:] == -1.0)
+    # output short: three whole blocks fit; output pointer only 4-byte aligned; input at an odd address
+    shifted = torch.zeros(5 * bb + 1, dtype=torch.uint8, device="cuda")
+    shifted[1:] = torch.from_numpy(raw).cuda()
+    buf = torch.full((3 * bs + 9,), -1.0, dtype=torch.float32, device="cuda")
+    hip.dequantize(shifted[1:], buf[1:], dtype)
+    got = buf.cpu().numpy()
+    assert got[0] == -1.0 and np.array_equal(got[1: 1 + 3 * bs], want[: 3 * bs]) and np.all(got[1 + 3 * bs:] == -1.0)
+    # empty input is a no-op
+    hip.dequantize(bd[:0], od, dtype)
+
+
+# -------------------------------------------------------------------- GEMV
+SHAPES = [  # (n, k)
+    (33, 256), (7, 512), (64, 1536), (100, 4096), (40, 14336), (19, 8192), (5, 20480), (3, 11008),
+]
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("n,k", SHAPES)
+def test_gemv_m1_matches_oracle(hip, torch, oracle, dtype, n, k):
+    print(f"gemv dtype={dtype} n={n} k={k}", flush=True)
+    w, x = random_weight(dtype, n, k, seed=n + k), random_activations(1, k, seed=k)
+    want = oracle.quantized_matmul(w, x, dtype, 1, n, k, acc=oracle.ACC_F64, threads=4)
+    got = gpu_matmul(hip, torch, w, x, dtype, 1, n, k)
+    check_close(got, want, f"dtype={dtype} n={n} k={k}")
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("m", [2, 3, 5, 8])
+def test_small_m_matches_oracle(hip, torch, oracle, dtype, m):
+    n, k = 77, 4096
+    print(f"small-m dtype={dtype} m={m}", flush=True)
+    w, x = random_weight(dtype, n, k, seed=m), random_activations(m, k, seed=m)
+    want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+    got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+    check_close(got, want, f"dtype={dtype} m={m}")
+
+
+@pytest.mark.parametrize("dtype,k", [(Q4_K, 300), (Q5_K, 511), (Q6_K, 257), (Q8_0, 40), (Q8_0, 4000), (Q4_K, 4100)])
+def test_row_padding(hip, torch, oracle, dtype, k):
+    print(f"padding dtype={dtype} k={k}", flush=True)
+    n = 21
+    w, x = random_weight(dtype, n, k, seed=3), random_activations(2, k, seed=3)
+    want = oracle.quantized_matmul(w, x, dtype, 2, n, k, acc=oracle.ACC_F64)
+    got = gpu_matmul(hip, torch, w, x, dtype, 2, n, k)
+    check_close(got, want, f"dtype={dtype} k={k}")
+    got1 = gpu_matmul(hip, torch, w, x[:1], dtype, 1, n, k)
+    check_close(got1, want[:1], f"dtype={dtype} k={k} m=1")
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_unit_vector_returns_weight_column_bit_exactly(hip, torch, oracle, dtype):
+    print(f"unit vector dtype={dtype}", flush=True)
+    n, k = 50, 1024
+    w = random_weight(dtype, n, k, seed=12)
+    deq = oracle.dequantize(w, dtype).reshape(n, k)
+    for col in (0, 31, 32, 63, 64, 255, 256, 700, 1023):
+        x = np.zeros((1, k), np.float32)
+        x[0, col] = 1.0
+        got = gpu_matmul(hip, torch, w, x, dtype, 1, n, k)
+        assert np.array_equal(got[0].view(np.uint32), deq[:, col].view(np.uint32)), f"col {col}"
+
+
+def test_linearity_at_full_size(hip, torch):
+    # size-independent property at the headline shape: Q4_K 4096 -> 14336
+    n, k = 14336, 4096
+    print("linearity 14336x4096", flush=True)
+    w = random_weight(Q4_K, n, k, seed=0)
+    x1, x2 = random_activations(1, k, seed=1), random_activations(1, k, seed=2)
+    y1 = gpu_matmul(hip, torch, w, x1, Q4_K, 1, n, k).astype(np.float64)
+    y2 = gpu_matmul(hip, torch, w, x2, Q4_K, 1, n, k).astype(np.float64)
+    y12 = gpu_matmul(hip, torch, w, 3.0 * x1 - 2.0 * x2, Q4_K, 1, n, k)
+    check_close(y12, 3.0 * y1 - 2.0 * y2, "linearity")
+
+
+@pytest.mark.parametrize("dtype,n,k", [(Q4_K, 4096, 4096), (Q4_K, 14336, 4096), (Q6_K, 14336, 4096),
+                                       (Q6_K, 4096, 14336), (Q4_K, 6144, 4096)])
+def test_baseline_shapes_match_oracle(hip, torch, oracle, dtype, n, k):
+    print(f"baseline shape dtype={dtype} n={n} k={k}", flush=True)
+    w, x = random_weight(dtype, n, k, seed=0), random_activations(1, k, seed=0)
+    want = oracle.quantized_matmul(w, x, dtype, 1, n, k, acc=oracle.ACC_F64, threads=8)
+    got = gpu_matmul(hip, torch, w, x, dtype, 1, n, k)
+    rel = check_close(got, want, f"dtype={dtype} n={n} k={k}")
+    print(f"  rel_l2={rel:.3e}", flush=True)
+    # host-slice form of the call on the smallest of them
+    if n == 4096 and k == 4096:
+        out = np.zeros((1, n), np.float32)
+        hip.quantized_matmul(w, x, out, dtype, 1, n, k)
+        assert np.array_equal(out, got)
+
+
+# ------------------------------------------------------------------- errors
+def test_unsupported_formats_are_errors(hip, torch):
+    from gllm_amd.backend import OtherError, Unimplemented
+    w = torch.zeros(18 * 4, dtype=torch.uint8, device="cuda")
+    x = torch.zeros(32, dtype=torch.float32, device="cuda")
+    y = torch.zeros(4, dtype=torch.float32, device="cuda")
+    for dt in (0, 1, 2, 3, 6, 7, 10, 11, 15, 30, 39):  # F32, F16, Q4_0 ... Q8_K, BF16, MXFP4
+        with pytest.raises(Unimplemented):
+            hip.quantized_matmul(w, x, y, dt, 1, 4, 32)
+        with pytest.raises(Unimplemented):
+            hip.dequantize(w, y, dt)
+    with pytest.raises(OtherError):  # weight buffer shorter than n rows
+        hip.quantized_matmul(w, x, y, Q8_0, 1, 4, 64)
+    hip.quantized_matmul(w, x, y, Q8_0, 0, 4, 32)  # m = 0: nothing to do
