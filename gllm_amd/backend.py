@@ -90,6 +90,8 @@ def load_library() -> C.CDLL:
     L.gllmq_quantized_matmul_batch.argtypes = [vp, C.POINTER(MatmulDesc), sz, vp]
     L.gllmq_moe_matvec.restype = C.c_int
     L.gllmq_moe_matvec.argtypes = [vp, vp, u32, vp, u32, vp, vp, sz, sz, sz, sz, sz, vp, vp, vp, C.c_int, vp]
+    L.gllmq_stream_read.restype = C.c_int
+    L.gllmq_stream_read.argtypes = [vp, vp, sz, vp, vp]
     L.gllmq_dequantize_host.restype = C.c_int
     L.gllmq_dequantize_host.argtypes = [vp, vp, sz, vp, sz, u32]
     L.gllmq_quantized_matmul_host.restype = C.c_int
@@ -102,7 +104,7 @@ EXPORTED_SYMBOLS = [
     "gllmq_init", "gllmq_destroy", "gllmq_last_error", "gllmq_status_string", "gllmq_version",
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
-    "gllmq_moe_matvec", "gllmq_dequantize_host", "gllmq_quantized_matmul_host",
+    "gllmq_moe_matvec", "gllmq_stream_read", "gllmq_dequantize_host", "gllmq_quantized_matmul_host",
 ]
 
 
@@ -226,6 +228,13 @@ class HipBackend:
         rc = self._lib.gllmq_quantized_matmul_batch(self._ctx, arr, len(items), self._stream())
         if rc != OK:
             self._raise(rc, "quantized_matmul_batch")
+
+    def stream_read(self, buf, sink) -> None:
+        """Calibration: one streaming read of ``buf`` (device tensor, 16-byte multiple)."""
+        rc = self._lib.gllmq_stream_read(self._ctx, buf.data_ptr(), buf.numel() * buf.element_size(),
+                                         sink.data_ptr(), self._stream())
+        if rc != OK:
+            self._raise(rc, "stream_read")
 
     def moe_matvec(self, gate_up, dtype_gate_up, down, dtype_down, x, out, hidden: int, ffn: int,
                    experts: int, route_expert, route_weight, route_len, relu_gate: bool = False) -> None:

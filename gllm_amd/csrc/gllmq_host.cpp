@@ -69,8 +69,26 @@ struct GemvParams {
     const uint8_t *w;
     const float *x;
     float *y;
-    uint32_t n, k, groups, row_bytes, ks, rps, rows_per_wg, ldx, ldy, x_vec, accumulate;
+    uint32_t n, k, groups, row_bytes, ks, rps, rows_per_wg, ldx, ldy, x_vec, accumulate, prep_words;
 };
+
+// Mirror of gq::Mm8Params in mm8.hip.inc.
+struct Mm8Params {
+    const uint8_t *w;
+    const float *x;
+    float *y;
+    uint32_t n, k, groups, row_bytes, m, ldx, ldy, tiles, x_vec;
+};
+
+// Same carve-up as gq::mm8_lds_layout: bytes of LDS the int8 matrix-core kernel needs.
+uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs)
+{
+    const uint32_t plane_stride = groups * 256u + 16u;
+    const uint32_t sums = 3u * m * plane_stride;
+    const uint32_t scales = sums + m * groups * 8u * 4u;
+    const uint32_t red = (scales + m * groups * 4u + 15u) & ~15u;
+    return red + 2u * 8u * pairs * 64u * 4u + 8u * 5120u; // + one 5 KiB weight stage per wave
+}
 
 } // namespace
 
@@ -78,7 +96,12 @@ struct gllmq_ctx {
     int device = 0;
     hipModule_t module = nullptr;
     hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
-    hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1]
+    hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1], f32 multiply-add flavour
+    hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
+    bool gemv_f32 = false;                      // GLLMQ_GEMV_F32=1 selects the f32 flavour
+    hipFunction_t mm8_q4k[3] = {};              // int8 matrix-core kernels for 1, 2, 4 activation-row pairs
+    bool use_mm8 = true;                        // GLLMQ_MM8=0 falls back to the GEMV kernels
+    hipFunction_t stream_read = nullptr;
     int num_cus = 256;
     uint32_t gemv_waves = 2048; // waves a GEMV launch aims to put on the device
     std::mutex err_mutex;
@@ -157,17 +180,20 @@ int launch_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, size_t row_by
     wgs = std::min(wgs, (row_steps + rgs - 1) / rgs);
     uint32_t steps_per_wg = (row_steps + wgs * rgs - 1) / (wgs * rgs);
     P.rows_per_wg = steps_per_wg * rgs * P.rps;
-    // partial sums of a K-split row meet in LDS: keep them within 32 KiB
-    const uint32_t max_rows = 32768u / (4u * P.ks * m);
+    // partial sums of a K-split row meet in LDS: keep them within 8 KiB
+    const uint32_t max_rows = 8192u / (4u * P.ks * m);
     if (P.ks > 1 && P.rows_per_wg > max_rows) P.rows_per_wg = std::max(rgs, max_rows / rgs * rgs);
     const uint32_t grid = (n + P.rows_per_wg - 1) / P.rows_per_wg;
-    const uint32_t lds = P.ks > 1 ? P.rows_per_wg * P.ks * m * 4u : 0u;
+    // integer-dot flavour: per part and activation row 48 plane words + 1 scale + 4 sums
+    P.prep_words = ctx->gemv_f32 ? 0u : 53u * m * parts;
+    const uint32_t lds = P.prep_words * 4u + (P.ks > 1 ? P.rows_per_wg * P.ks * m * 4u : 0u);
     P.ldx = ldx;
     P.ldy = ldy;
     P.x_vec = aligned(x, 16) && (m == 1 || ldx % 4 == 0);
     P.accumulate = accumulate ? 1u : 0u;
     const int fi = format_index(f.dtype);
-    return launch(ctx, ctx->gemv[fi][m - 1], grid, 64 * nwaves, lds, stream, &P, sizeof P);
+    hipFunction_t fn = ctx->gemv_f32 ? ctx->gemv[fi][m - 1] : ctx->gemv_i8[fi][m - 1];
+    return launch(ctx, fn, grid, 64 * nwaves, lds, stream, &P, sizeof P);
 }
 
 int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_bytes, const float *x,
@@ -193,6 +219,35 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
     if (!aligned(x, 4) || !aligned(y, 4))
         return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "quantized_matmul: activations and outputs must be 4-byte aligned");
     return -1; // go on
+}
+
+// m <= 8 on the int8 matrix cores (Q4_K).  Returns -1 when the shape does not fit the
+// kernel (LDS for the prepared activations), so that the caller takes the GEMV kernels.
+int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
+            size_t k, void *stream)
+{
+    if (!ctx->use_mm8 || f.dtype != T_Q4_K || m > 8) return -1;
+    const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
+    const int pi = m <= 2 ? 0 : (m <= 4 ? 1 : 2);
+    const uint32_t pairs = 1u << pi;
+    const uint32_t lds = mm8_lds_bytes(groups, static_cast<uint32_t>(m), pairs);
+    if (lds > 152u * 1024u) return -1;
+    Mm8Params P{};
+    P.w = w;
+    P.x = x;
+    P.y = y;
+    P.n = static_cast<uint32_t>(n);
+    P.k = static_cast<uint32_t>(k);
+    P.groups = groups;
+    P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
+    P.m = static_cast<uint32_t>(m);
+    P.ldx = static_cast<uint32_t>(k);
+    P.ldy = static_cast<uint32_t>(n);
+    P.tiles = (P.n + 31u) / 32u;
+    P.x_vec = aligned(x, 16) && (m == 1 || k % 4 == 0);
+    uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
+    if (const char *v = getenv("GLLMQ_MM8_GRID")) grid = std::min<uint32_t>(grid, std::max(1, atoi(v)));
+    return launch(ctx, ctx->mm8_q4k[pi], grid, 512, lds, stream, &P, sizeof P);
 }
 
 int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
@@ -290,8 +345,15 @@ int gllmq_init(gllmq_ctx **out, int device)
         for (int m = 1; m <= 2 && rc == GLLMQ_OK; ++m) {
             snprintf(name, sizeof name, "gq_gemv_%s_m%d", kFormats[i].tag, m);
             rc = get_function(ctx, &ctx->gemv[i][m - 1], name);
+            if (rc != GLLMQ_OK) break;
+            snprintf(name, sizeof name, "gq_gemv_i8_%s_m%d", kFormats[i].tag, m);
+            rc = get_function(ctx, &ctx->gemv_i8[i][m - 1], name);
         }
     }
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->stream_read, "gq_stream_read");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_q4k[0], "gq_mm8_q4k_p1");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_q4k[1], "gq_mm8_q4k_p2");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_q4k[2], "gq_mm8_q4k_p4");
     if (rc != GLLMQ_OK) {
         fprintf(stderr, "gllmq_init: %s\n", ctx->err.c_str());
         (void)hipModuleUnload(ctx->module);
@@ -299,6 +361,8 @@ int gllmq_init(gllmq_ctx **out, int device)
         return rc;
     }
     ctx->gemv_waves = static_cast<uint32_t>(ctx->num_cus) * 8u;
+    if (const char *v = getenv("GLLMQ_GEMV_F32")) ctx->gemv_f32 = (v[0] == '1');
+    if (const char *v = getenv("GLLMQ_MM8")) ctx->use_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_GEMV_WAVES")) {
         long w = strtol(v, nullptr, 10);
         if (w >= 4 && w <= 65536) ctx->gemv_waves = static_cast<uint32_t>(w);
@@ -348,6 +412,8 @@ int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, con
     int rc = check_matmul_args(ctx, f, w, w_bytes, x, y, dtype, m, n, k);
     if (rc >= 0) return rc;
     (void)act_mode;
+    rc = run_mm8(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, stream);
+    if (rc >= 0) return rc;
     return run_gemv(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, stream);
 }
 
@@ -376,6 +442,16 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *, uint32_t, const void *, uint3
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
     return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "moe_matvec: not built yet");
+}
+
+int gllmq_stream_read(gllmq_ctx *ctx, const void *buf, size_t n_bytes, void *sink, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    if (!buf || !sink) return fail(ctx, GLLMQ_ERR_INVALID, "stream_read: NULL device pointer");
+    if (!aligned(buf, 16) || n_bytes % 16 != 0)
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "stream_read: buffer must be 16-byte aligned and sized");
+    struct { const void *b; uint64_t n; void *s; } args = { buf, n_bytes / 16, sink };
+    return launch(ctx, ctx->stream_read, static_cast<uint32_t>(ctx->num_cus) * 8u, 256, 0, stream, &args, sizeof args);
 }
 
 int gllmq_dequantize_host(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *out, size_t n_out,

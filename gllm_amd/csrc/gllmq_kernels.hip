@@ -8,3 +8,6 @@
 
 #include "dequant.hip.inc"
 #include "gemv.hip.inc"
+#include "gemv_i8.hip.inc"
+#include "mm8.hip.inc"
+#include "probe.hip.inc"

@@ -48,10 +48,33 @@ __device__ __forceinline__ void scale_min_k4(int j, uint32_t s0, uint32_t s1, ui
     }
 }
 
-__device__ __forceinline__ float ubyte0(uint32_t v) { return static_cast<float>(v & 0xFFu); }
-__device__ __forceinline__ float ubyte1(uint32_t v) { return static_cast<float>((v >> 8) & 0xFFu); }
-__device__ __forceinline__ float ubyte2(uint32_t v) { return static_cast<float>((v >> 16) & 0xFFu); }
-__device__ __forceinline__ float ubyte3(uint32_t v) { return static_cast<float>(v >> 24); }
+// Byte n of a dword as f32 in one instruction.  Written as asm because the optimiser
+// otherwise folds the caller's nibble mask into a bit-field extract per byte and spends
+// two instructions where one does.
+__device__ __forceinline__ float ubyte0(uint32_t v)
+{
+    float f;
+    asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v));
+    return f;
+}
+__device__ __forceinline__ float ubyte1(uint32_t v)
+{
+    float f;
+    asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v));
+    return f;
+}
+__device__ __forceinline__ float ubyte2(uint32_t v)
+{
+    float f;
+    asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v));
+    return f;
+}
+__device__ __forceinline__ float ubyte3(uint32_t v)
+{
+    float f;
+    asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v));
+    return f;
+}
 
 // Sum over a segment of `len` consecutive lanes (len a multiple of 4, segment start a
 // multiple of 4, `pos` = lane's index inside its segment).  The total lands in the
@@ -65,6 +88,24 @@ __device__ __forceinline__ float segment_sum(float v, int pos, int len)
         const float o = __shfl_down(v, off, WAVE);
         if (pos + off < len) v += o;
     }
+    return v;
+}
+
+// Sum over all 64 lanes with DPP only (no LDS traffic); the total lands in lane 63.
+template <int CTRL, int ROW_MASK, bool BOUND>
+__device__ __forceinline__ float dpp_f32(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, BOUND));
+}
+
+__device__ __forceinline__ float wave_sum_to_last_lane(float v)
+{
+    v += dpp_f32<0x111, 0xF, true>(v); // row_shr:1
+    v += dpp_f32<0x112, 0xF, true>(v); // row_shr:2
+    v += dpp_f32<0x114, 0xF, true>(v); // row_shr:4
+    v += dpp_f32<0x118, 0xF, true>(v); // row_shr:8  -> lane 15 of each row of 16 holds the row sum
+    v += dpp_f32<0x142, 0xA, false>(v); // row_bcast:15 into rows 1 and 3
+    v += dpp_f32<0x143, 0xC, false>(v); // row_bcast:31 into rows 2 and 3 -> lane 63 holds the total
     return v;
 }
 

@@ -115,6 +115,12 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up_dev, uint32_t dtype_gat
                      const uint32_t *route_expert_dev, const float *route_weight_dev,
                      const uint32_t *route_len_dev, int relu_gate, void *stream);
 
+/* ---- calibration ------------------------------------------------------------------
+ * No counterpart in the reference.  Reads `n_bytes` (multiple of 16, 16-byte aligned) of
+ * device memory once with a pure streaming kernel; timing it gives the read bandwidth a
+ * bandwidth-bound kernel can reach on this device.  `sink_dev` points at 4 writable bytes. */
+int gllmq_stream_read(gllmq_ctx *ctx, const void *buf_dev, size_t n_bytes, void *sink_dev, void *stream);
+
 /* ---- host-pointer convenience (upload, run, download, synchronise) ---------------- */
 int gllmq_dequantize_host(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *out,
                           size_t n_out, uint32_t ggml_dtype);
