@@ -99,7 +99,7 @@ struct gllmq_ctx {
     hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1], f32 multiply-add flavour
     hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
     bool gemv_f32 = false;                      // GLLMQ_GEMV_F32=1 selects the f32 flavour
-    hipFunction_t mm8_q4k[3] = {};              // int8 matrix-core kernels for 1, 2, 4 activation-row pairs
+    hipFunction_t mm8_q4k[3][3] = {};           // int8 matrix-core kernels [pairs 1,2,4][early steps 1,2,4]
     bool use_mm8 = true;                        // GLLMQ_MM8=0 falls back to the GEMV kernels
     hipFunction_t stream_read = nullptr;
     int num_cus = 256;
@@ -244,10 +244,15 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     P.ldx = static_cast<uint32_t>(k);
     P.ldy = static_cast<uint32_t>(n);
     P.tiles = (P.n + 31u) / 32u;
-    P.x_vec = aligned(x, 16) && (m == 1 || k % 4 == 0);
+    P.x_vec = 1;
+    if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
+    // preparation steps per wave: two 256-element blocks per step
+    const uint32_t ppt = (groups + 7u) / 8u, steps = ((ppt + 1u) / 2u) * static_cast<uint32_t>(m);
+    int ei = steps <= 1 ? 0 : (steps <= 2 ? 1 : 2);
+    while (ei < 2 && !ctx->mm8_q4k[pi][ei]) ++ei; // not every (pairs, early) pair is built
     uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
     if (const char *v = getenv("GLLMQ_MM8_GRID")) grid = std::min<uint32_t>(grid, std::max(1, atoi(v)));
-    return launch(ctx, ctx->mm8_q4k[pi], grid, 512, lds, stream, &P, sizeof P);
+    return launch(ctx, ctx->mm8_q4k[pi][ei], grid, 512, lds, stream, &P, sizeof P);
 }
 
 int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
@@ -351,9 +356,14 @@ int gllmq_init(gllmq_ctx **out, int device)
         }
     }
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->stream_read, "gq_stream_read");
-    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_q4k[0], "gq_mm8_q4k_p1");
-    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_q4k[1], "gq_mm8_q4k_p2");
-    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_q4k[2], "gq_mm8_q4k_p4");
+    {
+        static const struct { int pi, ei; const char *name; } kMm8[] = {
+            { 0, 0, "gq_mm8_q4k_p1_e1" }, { 0, 1, "gq_mm8_q4k_p1_e2" }, { 0, 2, "gq_mm8_q4k_p1_e4" },
+            { 1, 1, "gq_mm8_q4k_p2_e2" }, { 1, 2, "gq_mm8_q4k_p2_e4" }, { 2, 2, "gq_mm8_q4k_p4_e4" },
+        };
+        for (const auto &k : kMm8)
+            if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_q4k[k.pi][k.ei], k.name);
+    }
     if (rc != GLLMQ_OK) {
         fprintf(stderr, "gllmq_init: %s\n", ctx->err.c_str());
         (void)hipModuleUnload(ctx->module);
