@@ -76,6 +76,8 @@ def main():
     ap.add_argument("--steps", type=int, default=4000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-context", action="store_true",
+                    help="skip the cache-resident and streaming-read context runs (profiling: only the timed kernel launches)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU; the quantized matmul path has no multi-GPU part "
@@ -96,6 +98,7 @@ def main():
     g.manual_seed(1)
     x = torch.randn(M, K_DIM, device="cuda", generator=g)
     ys = [torch.empty(M, N, device="cuda") for _ in range(COPIES)]
+    nb = ws[0].numel()
     bytes_per_call = N * row_bytes(DTYPE, K_DIM) + M * K_DIM * 4 + M * N * 4  # 33,103,872
 
     def descs(count, single=False):
@@ -119,22 +122,26 @@ def main():
     gbs = bytes_per_call / (us_per_call * 1e-6) / 1e9
 
     # context figures (stderr): cache-resident weights, and the device's streaming-read rate
-    ms1 = timed(descs(min(args.steps, 1000), single=True))
-    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
-    nb = ws[0].numel()
-    for i in range(32):
-        hip.stream_read(ws[i % COPIES], sink)
-    torch.cuda.synchronize()
-    start.record()
-    for i in range(400):
-        hip.stream_read(ws[i % COPIES], sink)
-    stop.record()
-    torch.cuda.synchronize()
-    probe_us = start.elapsed_time(stop) * 1e3 / 400
+    context = None
+    if not args.no_context:
+        ms1 = timed(descs(min(args.steps, 1000), single=True))
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        for i in range(32):
+            hip.stream_read(ws[i % COPIES], sink)
+        torch.cuda.synchronize()
+        start.record()
+        for i in range(400):
+            hip.stream_read(ws[i % COPIES], sink)
+        stop.record()
+        torch.cuda.synchronize()
+        probe_us = start.elapsed_time(stop) * 1e3 / 400
+        context = {"cache_resident_us_per_call": round(ms1 * 1e3 / min(args.steps, 1000), 3),
+                   "stream_read_probe_gbs": round(nb / probe_us / 1e3, 1)}
     log(f"Q4_K GEMV 1x{K_DIM}x{N}: {us_per_call:.2f} us/call, {gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS * 100:.1f}% of 8 TB/s), "
         f"{2 * N * K_DIM / (us_per_call * 1e-6) / 1e12:.2f} TFLOP/s")
-    log(f"  same weights every call (cache resident): {ms1 * 1e3 / min(args.steps, 1000):.2f} us/call")
-    log(f"  streaming-read probe over the same 33 MB buffers: {probe_us:.2f} us/launch = {nb / probe_us / 1e3:.0f} GB/s")
+    if context:
+        log(f"  same weights every call (cache resident): {context['cache_resident_us_per_call']:.2f} us/call")
+        log(f"  streaming-read probe over the same 33 MB buffers: {context['stream_read_probe_gbs']:.0f} GB/s")
 
     result = {
         "metric": "Q4_K GEMV 1x4096x14336: achieved HBM GB/s",
@@ -160,9 +167,9 @@ def main():
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "note": "achieved = 33,103,872 algorithmic bytes / (event time over the timed region / steps); "
                              "the event time includes the gap between back-to-back launches"},
-        "context": {"cache_resident_us_per_call": round(ms1 * 1e3 / min(args.steps, 1000), 3),
-                    "stream_read_probe_gbs": round(nb / probe_us / 1e3, 1)},
     }
+    if context:
+        result["context"] = context
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
         log(f"  CPU baseline: {result['cpu_baseline']}")

@@ -77,7 +77,7 @@ struct Mm8Params {
     const uint8_t *w;
     const float *x;
     float *y;
-    uint32_t n, k, groups, row_bytes, m, ldx, ldy, tiles, x_vec;
+    uint32_t n, k, groups, row_bytes, m, ldx, ldy, tiles, grid;
 };
 
 // Same carve-up as gq::mm8_lds_layout: bytes of LDS the int8 matrix-core kernel needs.
@@ -244,7 +244,6 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     P.ldx = static_cast<uint32_t>(k);
     P.ldy = static_cast<uint32_t>(n);
     P.tiles = (P.n + 31u) / 32u;
-    P.x_vec = 1;
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
     // preparation steps per wave: two 256-element blocks per step
     const uint32_t ppt = (groups + 7u) / 8u, steps = ((ppt + 1u) / 2u) * static_cast<uint32_t>(m);
@@ -252,6 +251,7 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     while (ei < 2 && !ctx->mm8_q4k[pi][ei]) ++ei; // not every (pairs, early) pair is built
     uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
     if (const char *v = getenv("GLLMQ_MM8_GRID")) grid = std::min<uint32_t>(grid, std::max(1, atoi(v)));
+    P.grid = grid;
     return launch(ctx, ctx->mm8_q4k[pi][ei], grid, 512, lds, stream, &P, sizeof P);
 }
 
