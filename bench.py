@@ -26,6 +26,12 @@ COPIES = 16
 HBM_PEAK_GBS = 8000.0
 
 
+# HBM bytes per launch of the timed kernel on this workload, from two counter passes
+# (FETCH_SIZE 16,249.5 KiB and WRITE_SIZE 56.0 KiB per dispatch) scaled by what the same
+# counters read for a plain 32,256 KiB copy kernel (factors 1.9986 and 1.0000).
+TRAFFIC_BYTES_PER_LAUNCH = 33_312_900
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -78,6 +84,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-context", action="store_true",
                     help="skip the cache-resident and streaming-read context runs (profiling: only the timed kernel launches)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch plain device-to-device copies of one 33 MB weight buffer (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU; the quantized matmul path has no multi-GPU part "
@@ -115,6 +123,12 @@ def main():
         torch.cuda.synchronize()
         return start.elapsed_time(stop)  # ms
 
+    if args.copy_probe:
+        # A plain copy kernel of known size: 33,030,144 bytes read and as many written per launch.
+        dst = torch.empty_like(ws[0])
+        for i in range(8):
+            dst.copy_(ws[i % COPIES])
+        torch.cuda.synchronize()
     hip.quantized_matmul_batch(descs(args.warmup))
     torch.cuda.synchronize()
     ms = timed(descs(args.steps))
@@ -164,7 +178,7 @@ def main():
                                f"weights rotate over {COPIES} copies ({COPIES * nb >> 20} MiB) so every call reads HBM",
                    "bytes_per_call": bytes_per_call, "kernel": "gq_mm8_q4k_p1_e1"},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
                      "note": "achieved = 33,103,872 algorithmic bytes / (event time over the timed region / steps); "
                              "the event time includes the gap between back-to-back launches"},
     }
