@@ -80,6 +80,41 @@ struct Mm8Params {
     uint32_t n, k, groups, row_bytes, m, ldx, ldy, tiles, grid;
 };
 
+// Mirrors of the structs in moe.hip.inc.
+struct MoeJob {
+    uint32_t expert, p0, m, t0, t1;
+};
+struct MoePlanParams {
+    const uint32_t *route_expert;
+    const uint32_t *route_len;
+    uint32_t *pair_src;
+    uint32_t *pair_pos;
+    MoeJob *jobs;
+    uint32_t *counters;
+    uint32_t tokens, top_k, experts, pairs;
+};
+struct MoeGemvParams {
+    GemvParams g;
+    const MoeJob *jobs;
+    const uint32_t *counters;
+    uint64_t expert_stride;
+    uint32_t wgs_per_job, x_by_token, x_stride, y_stride;
+};
+struct MoeActParams {
+    const float *gu;
+    float *h;
+    const uint32_t *counters;
+    uint32_t ffn, relu_gate;
+};
+struct MoeCombineParams {
+    const float *o;
+    const float *route_weight;
+    const uint32_t *route_len;
+    const uint32_t *pair_pos;
+    float *out;
+    uint32_t tokens, top_k, hidden;
+};
+
 // Same carve-up as gq::mm8_lds_layout: bytes of LDS the int8 matrix-core kernel needs.
 uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs)
 {
@@ -102,6 +137,14 @@ struct gllmq_ctx {
     hipFunction_t mm8_q4k[3][3] = {};           // int8 matrix-core kernels [pairs 1,2,4][early steps 1,2,4]
     bool use_mm8 = true;                        // GLLMQ_MM8=0 falls back to the GEMV kernels
     hipFunction_t stream_read = nullptr;
+    hipFunction_t moe_plan = nullptr, moe_act = nullptr, moe_combine = nullptr;
+    hipFunction_t moe_gemv[kNumFormats] = {};
+    // Device workspace of the MoE path (pair tables, jobs, intermediate activations).  It
+    // grows on demand and is shared by all calls on this context: calls that use it must
+    // not overlap in time.
+    void *workspace = nullptr;
+    size_t workspace_bytes = 0;
+    std::mutex workspace_mutex;
     int num_cus = 256;
     uint32_t gemv_waves = 2048; // waves a GEMV launch aims to put on the device
     std::mutex err_mutex;
@@ -140,27 +183,36 @@ int get_function(gllmq_ctx *ctx, hipFunction_t *f, const char *name)
     return GLLMQ_OK;
 }
 
-int launch(gllmq_ctx *ctx, hipFunction_t f, uint32_t grid, uint32_t block, uint32_t lds, void *stream,
-           void *params, size_t params_size)
+int launch2d(gllmq_ctx *ctx, hipFunction_t f, uint32_t grid_x, uint32_t grid_y, uint32_t block, uint32_t lds,
+             void *stream, void *params, size_t params_size)
 {
     void *config[] = { HIP_LAUNCH_PARAM_BUFFER_POINTER, params, HIP_LAUNCH_PARAM_BUFFER_SIZE,
                        &params_size, HIP_LAUNCH_PARAM_END };
-    GLLMQ_HIP(ctx, hipModuleLaunchKernel(f, grid, 1, 1, block, 1, 1, lds, static_cast<hipStream_t>(stream),
+    GLLMQ_HIP(ctx, hipModuleLaunchKernel(f, grid_x, grid_y, 1, block, 1, 1, lds, static_cast<hipStream_t>(stream),
                                          nullptr, config));
     return GLLMQ_OK;
 }
 
+int launch(gllmq_ctx *ctx, hipFunction_t f, uint32_t grid, uint32_t block, uint32_t lds, void *stream,
+           void *params, size_t params_size)
+{
+    return launch2d(ctx, f, grid, 1, block, lds, stream, params, params_size);
+}
+
 bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
-// One GEMV launch over at most 64 groups (16384 elements) of K and m <= 2.
-int launch_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, size_t row_bytes, const float *x,
-                float *y, uint32_t m, uint32_t n, uint32_t k, uint32_t ldx, uint32_t ldy, bool accumulate,
-                void *stream)
+// Shape-dependent fields of a GEMV launch over at most 64 groups (16384 elements) of K and
+// m <= 2: how a row is split over lanes and waves, rows per workgroup, LDS.  `target_waves`
+// is the number of waves the launch aims to put on the device.
+struct GemvPlan {
+    GemvParams P;
+    uint32_t grid, threads, lds;
+};
+
+GemvPlan plan_gemv(const gllmq_ctx *ctx, uint32_t m, uint32_t n, uint32_t k, size_t row_bytes, uint32_t target_waves)
 {
-    GemvParams P{};
-    P.w = w;
-    P.x = x;
-    P.y = y;
+    GemvPlan L{};
+    GemvParams &P = L.P;
     P.n = n;
     P.k = k;
     P.groups = (k + 255u) / 256u;
@@ -176,24 +228,37 @@ int launch_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, size_t row_by
     const uint32_t rgs = std::max(1u, 4u / P.ks);
     const uint32_t nwaves = P.ks * rgs;
     const uint32_t row_steps = (n + P.rps - 1) / P.rps;
-    uint32_t wgs = std::max(1u, ctx->gemv_waves / nwaves);
+    uint32_t wgs = std::max(1u, target_waves / nwaves);
     wgs = std::min(wgs, (row_steps + rgs - 1) / rgs);
     uint32_t steps_per_wg = (row_steps + wgs * rgs - 1) / (wgs * rgs);
     P.rows_per_wg = steps_per_wg * rgs * P.rps;
     // partial sums of a K-split row meet in LDS: keep them within 8 KiB
     const uint32_t max_rows = 8192u / (4u * P.ks * m);
     if (P.ks > 1 && P.rows_per_wg > max_rows) P.rows_per_wg = std::max(rgs, max_rows / rgs * rgs);
-    const uint32_t grid = (n + P.rows_per_wg - 1) / P.rows_per_wg;
+    L.grid = (n + P.rows_per_wg - 1) / P.rows_per_wg;
+    L.threads = 64 * nwaves;
     // integer-dot flavour: per part and activation row 48 plane words + 1 scale + 4 sums
     P.prep_words = ctx->gemv_f32 ? 0u : 53u * m * parts;
-    const uint32_t lds = P.prep_words * 4u + (P.ks > 1 ? P.rows_per_wg * P.ks * m * 4u : 0u);
+    L.lds = P.prep_words * 4u + (P.ks > 1 ? P.rows_per_wg * P.ks * m * 4u : 0u);
+    return L;
+}
+
+int launch_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, size_t row_bytes, const float *x,
+                float *y, uint32_t m, uint32_t n, uint32_t k, uint32_t ldx, uint32_t ldy, bool accumulate,
+                void *stream)
+{
+    GemvPlan L = plan_gemv(ctx, m, n, k, row_bytes, ctx->gemv_waves);
+    GemvParams &P = L.P;
+    P.w = w;
+    P.x = x;
+    P.y = y;
     P.ldx = ldx;
     P.ldy = ldy;
     P.x_vec = aligned(x, 16) && (m == 1 || ldx % 4 == 0);
     P.accumulate = accumulate ? 1u : 0u;
     const int fi = format_index(f.dtype);
     hipFunction_t fn = ctx->gemv_f32 ? ctx->gemv[fi][m - 1] : ctx->gemv_i8[fi][m - 1];
-    return launch(ctx, fn, grid, 64 * nwaves, lds, stream, &P, sizeof P);
+    return launch(ctx, fn, L.grid, L.threads, L.lds, stream, &P, sizeof P);
 }
 
 int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_bytes, const float *x,
@@ -356,6 +421,13 @@ int gllmq_init(gllmq_ctx **out, int device)
         }
     }
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->stream_read, "gq_stream_read");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_plan, "gq_moe_plan");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_act, "gq_moe_act");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_combine, "gq_moe_combine");
+    for (int i = 0; i < kNumFormats && rc == GLLMQ_OK; ++i) {
+        snprintf(name, sizeof name, "gq_moe_gemv_%s", kFormats[i].tag);
+        rc = get_function(ctx, &ctx->moe_gemv[i], name);
+    }
     {
         static const struct { int pi, ei; const char *name; } kMm8[] = {
             { 0, 0, "gq_mm8_q4k_p1_e1" }, { 0, 1, "gq_mm8_q4k_p1_e2" }, { 0, 2, "gq_mm8_q4k_p1_e4" },
@@ -384,6 +456,7 @@ int gllmq_init(gllmq_ctx **out, int device)
 void gllmq_destroy(gllmq_ctx *ctx)
 {
     if (!ctx) return;
+    if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->module) (void)hipModuleUnload(ctx->module);
     delete ctx;
 }
@@ -446,12 +519,118 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
     return GLLMQ_OK;
 }
 
-int gllmq_moe_matvec(gllmq_ctx *ctx, const void *, uint32_t, const void *, uint32_t, const float *, float *,
-                     size_t, size_t, size_t, size_t, size_t, const uint32_t *, const float *, const uint32_t *,
-                     int, void *)
+int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, const void *down, uint32_t dtype_dn,
+                     const float *x, float *out, size_t tokens, size_t hidden, size_t ffn, size_t experts,
+                     size_t top_k, const uint32_t *route_expert, const float *route_weight,
+                     const uint32_t *route_len, int relu_gate, void *stream)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
-    return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "moe_matvec: not built yet");
+    const Format *fg = find_format(dtype_gu), *fd = find_format(dtype_dn);
+    if (!fg || !fd)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
+                    "moe_matvec: ggml dtype %u / %u is not covered (supported: Q8_0=8, Q4_K=12, Q5_K=13, Q6_K=14)",
+                    dtype_gu, dtype_dn);
+    if (tokens == 0 || hidden == 0) return GLLMQ_OK;
+    if (!gate_up || !down || !x || !out || !route_expert || !route_weight || !route_len)
+        return fail(ctx, GLLMQ_ERR_INVALID, "moe_matvec: NULL device pointer");
+    if (ffn == 0 || experts == 0 || top_k == 0)
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "moe_matvec: ffn, experts and top_k must be positive");
+    const size_t pairs = tokens * top_k;
+    // The plan kernel keeps the pair list and three words per expert in LDS, and a launch
+    // covers at most 16384 elements of K.
+    if (pairs > 16384 || experts > 4096)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
+                    "moe_matvec: tokens*top_k = %zu (max 16384) or experts = %zu (max 4096) is beyond this build", pairs,
+                    experts);
+    if (hidden > 16384 || ffn > 16384)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "moe_matvec: hidden = %zu / ffn = %zu beyond 16384 is not built",
+                    hidden, ffn);
+    if (hidden % 4 != 0 || ffn % 4 != 0)
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "moe_matvec: hidden and ffn must be multiples of 4");
+    const size_t rb_gu = gllmq_row_bytes(dtype_gu, hidden), rb_dn = gllmq_row_bytes(dtype_dn, ffn);
+    if (!aligned(gate_up, fg->w_align) || rb_gu % fg->w_align != 0 || !aligned(down, fd->w_align) ||
+        rb_dn % fd->w_align != 0)
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "moe_matvec: expert weights miss the alignment of their format");
+    if (!aligned(x, 16) || !aligned(out, 4))
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "moe_matvec: x must be 16-byte and out 4-byte aligned");
+
+    // workspace carve-up (256-byte aligned pieces)
+    auto up256 = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+    size_t off = 0;
+    const size_t o_src = off; off = up256(off + pairs * 4);
+    const size_t o_pos = off; off = up256(off + pairs * 4);
+    const size_t o_jobs = off; off = up256(off + pairs * sizeof(MoeJob));
+    const size_t o_cnt = off; off = up256(off + 2 * 4);
+    const size_t o_gu = off; off = up256(off + pairs * 2 * ffn * 4);
+    const size_t o_h = off; off = up256(off + pairs * ffn * 4);
+    const size_t o_o = off; off = up256(off + pairs * hidden * 4);
+    std::lock_guard<std::mutex> guard(ctx->workspace_mutex);
+    if (ctx->workspace_bytes < off) {
+        GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
+        if (ctx->workspace) {
+            GLLMQ_HIP(ctx, hipDeviceSynchronize()); // earlier calls may still be reading it
+            GLLMQ_HIP(ctx, hipFree(ctx->workspace));
+            ctx->workspace = nullptr;
+            ctx->workspace_bytes = 0;
+        }
+        GLLMQ_HIP(ctx, hipMalloc(&ctx->workspace, off));
+        ctx->workspace_bytes = off;
+    }
+    uint8_t *ws = static_cast<uint8_t *>(ctx->workspace);
+    uint32_t *pair_src = reinterpret_cast<uint32_t *>(ws + o_src);
+    uint32_t *pair_pos = reinterpret_cast<uint32_t *>(ws + o_pos);
+    MoeJob *jobs = reinterpret_cast<MoeJob *>(ws + o_jobs);
+    uint32_t *counters = reinterpret_cast<uint32_t *>(ws + o_cnt);
+    float *gu = reinterpret_cast<float *>(ws + o_gu);
+    float *h = reinterpret_cast<float *>(ws + o_h);
+    float *o = reinterpret_cast<float *>(ws + o_o);
+
+    {
+        MoePlanParams P{ route_expert, route_len, pair_src, pair_pos, jobs, counters, static_cast<uint32_t>(tokens),
+                         static_cast<uint32_t>(top_k), static_cast<uint32_t>(experts), static_cast<uint32_t>(pairs) };
+        const uint32_t lds = static_cast<uint32_t>((pairs + 3 * experts + 1024) * 4);
+        int rc = launch(ctx, ctx->moe_plan, 1, 1024, lds, stream, &P, sizeof P);
+        if (rc != GLLMQ_OK) return rc;
+    }
+    // Waves per job: the device takes about 8 waves per CU of these kernels; the jobs that
+    // exist (at most `pairs`, typically one per routed expert) share them.
+    const uint32_t job_waves = std::max<uint32_t>(16u, 4u * ctx->gemv_waves / static_cast<uint32_t>(pairs));
+    auto grouped = [&](const Format &f, const void *w, size_t rb, uint32_t n, uint32_t k, const float *xin,
+                       bool x_by_token, float *yout) -> int {
+        GemvPlan L = plan_gemv(ctx, 2, n, k, rb, job_waves);
+        MoeGemvParams Q{};
+        Q.g = L.P;
+        Q.g.w = static_cast<const uint8_t *>(w);
+        Q.g.x = xin;
+        Q.g.y = yout;
+        Q.g.x_vec = 1;
+        Q.g.accumulate = 0;
+        Q.jobs = jobs;
+        Q.counters = counters;
+        Q.expert_stride = static_cast<uint64_t>(n) * rb;
+        Q.wgs_per_job = L.grid;
+        Q.x_by_token = x_by_token ? 1u : 0u;
+        Q.x_stride = k;
+        Q.y_stride = n;
+        const uint64_t grid = static_cast<uint64_t>(L.grid) * pairs;
+        if (grid > 0x7FFFFFFFull) return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "moe_matvec: launch grid too large");
+        return launch(ctx, ctx->moe_gemv[format_index(f.dtype)], static_cast<uint32_t>(grid), L.threads, L.lds, stream,
+                      &Q, sizeof Q);
+    };
+    int rc = grouped(*fg, gate_up, rb_gu, static_cast<uint32_t>(2 * ffn), static_cast<uint32_t>(hidden), x, true, gu);
+    if (rc != GLLMQ_OK) return rc;
+    {
+        MoeActParams P{ gu, h, counters, static_cast<uint32_t>(ffn), relu_gate ? 1u : 0u };
+        rc = launch2d(ctx, ctx->moe_act, static_cast<uint32_t>((ffn + 255) / 256), static_cast<uint32_t>(pairs), 256, 0,
+                      stream, &P, sizeof P);
+        if (rc != GLLMQ_OK) return rc;
+    }
+    rc = grouped(*fd, down, rb_dn, static_cast<uint32_t>(hidden), static_cast<uint32_t>(ffn), h, false, o);
+    if (rc != GLLMQ_OK) return rc;
+    MoeCombineParams C{ o, route_weight, route_len, pair_pos, out, static_cast<uint32_t>(tokens),
+                        static_cast<uint32_t>(top_k), static_cast<uint32_t>(hidden) };
+    return launch2d(ctx, ctx->moe_combine, static_cast<uint32_t>((hidden + 255) / 256), static_cast<uint32_t>(tokens),
+                    256, 0, stream, &C, sizeof C);
 }
 
 int gllmq_stream_read(gllmq_ctx *ctx, const void *buf, size_t n_bytes, void *sink, void *stream)

@@ -105,10 +105,19 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
                                  void *stream);
 
 /* ---- MoE expert matvec (ExpertRouteTable grouping, src/moe/routing.rs:163-173) -----
- * out[t] = sum_i weight[t][i] * down_e( silu(gate_e x_t) * (up_e x_t) ), e = expert[t][i].
+ * out[t] = sum_i weight[t][i] * down_e( silu(gate_e x_t) * (up_e x_t) ), e = expert[t][i],
+ * summed in route order i = 0 .. route_len[t]-1 (src/moe/routing.rs:307-327); a token with
+ * no route gets zeros.  Only routed (token, expert) pairs are computed (the reference graph
+ * runs every expert on every token and masks, build_graph.inc.rs:2076-2123).
  * gate_up_dev: per expert 2*ffn rows over `hidden` (gate rows, then up rows);
  * down_dev: per expert `hidden` rows over `ffn`.  route_* are [tokens x top_k] device
- * arrays, route_len[t] entries valid per token.  relu_gate != 0 applies max(g,0) first. */
+ * arrays, route_len[t] entries valid per token; entries past route_len[t] are ignored and
+ * an expert index >= experts routes nowhere (device data is not validated on the host).
+ * relu_gate != 0 applies max(g,0) before silu.
+ * Limits of this build: tokens*top_k <= 16384, experts <= 4096, hidden and ffn <= 16384
+ * and multiples of 4 (else GLLMQ_ERR_UNIMPLEMENTED / BAD_SHAPE).  x_dev 16-byte aligned.
+ * Intermediate buffers live in a workspace owned by the context that grows on demand:
+ * calls of this function on one context must not overlap in time. */
 int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up_dev, uint32_t dtype_gate_up,
                      const void *down_dev, uint32_t dtype_down, const float *x_dev, float *out_dev,
                      size_t tokens, size_t hidden, size_t ffn, size_t experts, size_t top_k,
