@@ -69,7 +69,7 @@ struct GemvParams {
     const uint8_t *w;
     const float *x;
     float *y;
-    uint32_t n, k, groups, row_bytes, ks, rps, rows_per_wg, ldx, ldy, x_vec, accumulate, prep_words;
+    uint32_t n, k, groups, row_bytes, ks, rps, rows_per_wg, ldx, ldy, x_vec, accumulate, prep_words, act_bf16;
 };
 
 // Mirror of gq::Mm8Params in mm8.hip.inc.
@@ -77,7 +77,7 @@ struct Mm8Params {
     const uint8_t *w;
     const float *x;
     float *y;
-    uint32_t n, k, groups, row_bytes, m, ldx, ldy, tiles, grid;
+    uint32_t n, k, groups, row_bytes, m, ldx, ldy, tiles, grid, act_bf16;
 };
 
 // Mirrors of the structs in moe.hip.inc.
@@ -245,7 +245,7 @@ GemvPlan plan_gemv(const gllmq_ctx *ctx, uint32_t m, uint32_t n, uint32_t k, siz
 
 int launch_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, size_t row_bytes, const float *x,
                 float *y, uint32_t m, uint32_t n, uint32_t k, uint32_t ldx, uint32_t ldy, bool accumulate,
-                void *stream)
+                bool act_bf16, void *stream)
 {
     GemvPlan L = plan_gemv(ctx, m, n, k, row_bytes, ctx->gemv_waves);
     GemvParams &P = L.P;
@@ -256,6 +256,7 @@ int launch_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, size_t row_by
     P.ldy = ldy;
     P.x_vec = aligned(x, 16) && (m == 1 || ldx % 4 == 0);
     P.accumulate = accumulate ? 1u : 0u;
+    P.act_bf16 = act_bf16 ? 1u : 0u;
     const int fi = format_index(f.dtype);
     hipFunction_t fn = ctx->gemv_f32 ? ctx->gemv[fi][m - 1] : ctx->gemv_i8[fi][m - 1];
     return launch(ctx, fn, L.grid, L.threads, L.lds, stream, &P, sizeof P);
@@ -286,42 +287,52 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
     return -1; // go on
 }
 
-// m <= 8 on the int8 matrix cores (Q4_K).  Returns -1 when the shape does not fit the
-// kernel (LDS for the prepared activations), so that the caller takes the GEMV kernels.
+// Q4_K on the int8 matrix cores, activation rows in passes of at most 8 (a pass keeps its
+// rows' digit planes in LDS and reads the weights once).  Returns -1 when the shape does
+// not fit the kernel (LDS for the prepared activations, alignment), so that the caller
+// takes the GEMV kernels.
 int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
-            size_t k, void *stream)
+            size_t k, bool act_bf16, void *stream)
 {
-    if (!ctx->use_mm8 || f.dtype != T_Q4_K || m > 8) return -1;
-    const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
-    const int pi = m <= 2 ? 0 : (m <= 4 ? 1 : 2);
-    const uint32_t pairs = 1u << pi;
-    const uint32_t lds = mm8_lds_bytes(groups, static_cast<uint32_t>(m), pairs);
-    if (lds > 152u * 1024u) return -1;
-    Mm8Params P{};
-    P.w = w;
-    P.x = x;
-    P.y = y;
-    P.n = static_cast<uint32_t>(n);
-    P.k = static_cast<uint32_t>(k);
-    P.groups = groups;
-    P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
-    P.m = static_cast<uint32_t>(m);
-    P.ldx = static_cast<uint32_t>(k);
-    P.ldy = static_cast<uint32_t>(n);
-    P.tiles = (P.n + 31u) / 32u;
+    if (!ctx->use_mm8 || f.dtype != T_Q4_K) return -1;
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
-    // preparation steps per wave: two 256-element blocks per step
-    const uint32_t ppt = (groups + 7u) / 8u, steps = ((ppt + 1u) / 2u) * static_cast<uint32_t>(m);
-    int ei = steps <= 1 ? 0 : (steps <= 2 ? 1 : 2);
-    while (ei < 2 && !ctx->mm8_q4k[pi][ei]) ++ei; // not every (pairs, early) pair is built
-    uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
-    if (const char *v = getenv("GLLMQ_MM8_GRID")) grid = std::min<uint32_t>(grid, std::max(1, atoi(v)));
-    P.grid = grid;
-    return launch(ctx, ctx->mm8_q4k[pi][ei], grid, 512, lds, stream, &P, sizeof P);
+    const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
+    if (mm8_lds_bytes(groups, static_cast<uint32_t>(std::min<size_t>(m, 8)), m <= 2 ? 1u : (m <= 4 ? 2u : 4u)) >
+        152u * 1024u)
+        return -1;
+    for (size_t m0 = 0; m0 < m; m0 += 8) {
+        const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(8, m - m0));
+        const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
+        const uint32_t pairs = 1u << pi;
+        const uint32_t lds = mm8_lds_bytes(groups, mm, pairs);
+        Mm8Params P{};
+        P.w = w;
+        P.x = x + m0 * k;
+        P.y = y + m0 * n;
+        P.n = static_cast<uint32_t>(n);
+        P.k = static_cast<uint32_t>(k);
+        P.groups = groups;
+        P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
+        P.m = mm;
+        P.ldx = static_cast<uint32_t>(k);
+        P.ldy = static_cast<uint32_t>(n);
+        P.tiles = (P.n + 31u) / 32u;
+        P.act_bf16 = act_bf16 ? 1u : 0u;
+        // preparation steps per wave: two 256-element blocks per step
+        const uint32_t ppt = (groups + 7u) / 8u, steps = ((ppt + 1u) / 2u) * mm;
+        int ei = steps <= 1 ? 0 : (steps <= 2 ? 1 : 2);
+        while (ei < 2 && !ctx->mm8_q4k[pi][ei]) ++ei; // not every (pairs, early) pair is built
+        uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
+        if (const char *v = getenv("GLLMQ_MM8_GRID")) grid = std::min<uint32_t>(grid, std::max(1, atoi(v)));
+        P.grid = grid;
+        int rc = launch(ctx, ctx->mm8_q4k[pi][ei], grid, 512, lds, stream, &P, sizeof P);
+        if (rc != GLLMQ_OK) return rc;
+    }
+    return GLLMQ_OK;
 }
 
 int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
-             size_t k, void *stream)
+             size_t k, bool act_bf16, void *stream)
 {
     const size_t rb = gllmq_row_bytes(f.dtype, k);
     constexpr size_t kChunk = 16384; // elements of K one launch covers (four waves of 4096)
@@ -331,7 +342,7 @@ int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
             const size_t kk = std::min(kChunk, k - k0);
             int rc = launch_gemv(ctx, f, w + (k0 / 256) * f.group_bytes, rb, x + m0 * k + k0, y + m0 * n, mm,
                                  static_cast<uint32_t>(n), static_cast<uint32_t>(kk), static_cast<uint32_t>(k),
-                                 static_cast<uint32_t>(n), k0 != 0, stream);
+                                 static_cast<uint32_t>(n), k0 != 0, act_bf16, stream);
             if (rc != GLLMQ_OK) return rc;
         }
     }
@@ -494,10 +505,14 @@ int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, con
     const Format *f = find_format(dtype);
     int rc = check_matmul_args(ctx, f, w, w_bytes, x, y, dtype, m, n, k);
     if (rc >= 0) return rc;
-    (void)act_mode;
-    rc = run_mm8(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, stream);
+    if (act_mode != GLLMQ_ACT_F32_SPLIT && act_mode != GLLMQ_ACT_BF16)
+        return fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul: unknown activation mode %d", act_mode);
+    const bool bf16 = act_mode == GLLMQ_ACT_BF16;
+    if (bf16 && ctx->gemv_f32)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "quantized_matmul: bf16 activations are not built for GLLMQ_GEMV_F32=1");
+    rc = run_mm8(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
     if (rc >= 0) return rc;
-    return run_gemv(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, stream);
+    return run_gemv(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
 }
 
 int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y,

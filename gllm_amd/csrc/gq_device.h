@@ -20,6 +20,16 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h)
     return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(h & 0xFFFFu)));
 }
 
+// f32 -> nearest bf16 (ties to even) -> f32; NaN passes through.  Same rule as
+// half::bf16::from_f32, which the reference uses (src/compat/weight_helpers.rs:1202-1215).
+__device__ __forceinline__ float round_to_bf16(float v)
+{
+    uint32_t b = __builtin_bit_cast(uint32_t, v);
+    if ((b & 0x7FFFFFFFu) > 0x7F800000u) return v;
+    b += 0x7FFFu + ((b >> 16) & 1u);
+    return __builtin_bit_cast(float, b & 0xFFFF0000u);
+}
+
 // Loads of 2-byte aligned data as wider words.  gfx950 under the HSA ABI runs global
 // memory in unaligned-access mode, so one load instruction serves any byte address.
 template <typename T>

@@ -43,13 +43,19 @@ enum {
     GLLMQ_ERR_INVALID = 5        /* NULL context or pointer                          */
 };
 
-/* Activation rounding used by the m >= GLLMQ_GEMM_MIN_M tensor-core path. */
+/* Activation handling.  The reference passes f32 activations to its CPU kernels
+ * (build_graph.inc.rs:94); GLLMQ_ACT_F32_SPLIT keeps at least 22 significant bits of every
+ * activation relative to the largest magnitude of its 256-element block (64-element part
+ * in the GEMV kernels).  GLLMQ_ACT_BF16 rounds every activation to bf16 (nearest, ties to
+ * even, as half::bf16::from_f32 does) first and then runs the same kernels: the result is
+ * the exact-weight product with bf16 activations, accumulated as above. */
 enum {
-    GLLMQ_ACT_F32_SPLIT = 0, /* x carried as two f16 terms (22+ significant bits)  */
-    GLLMQ_ACT_BF16 = 1       /* x rounded to bf16 (round-to-nearest-even)          */
+    GLLMQ_ACT_F32_SPLIT = 0,
+    GLLMQ_ACT_BF16 = 1
 };
 
-#define GLLMQ_GEMM_MIN_M 9
+/* Rows of activations one pass over the weights serves (larger m runs several passes). */
+#define GLLMQ_ROWS_PER_PASS 8
 
 typedef struct gllmq_ctx gllmq_ctx;
 
@@ -78,13 +84,16 @@ int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks_dev, size_t n_bytes, flo
 /* ---- Backend::quantized_matmul ----------------------------------------------------
  * y[m x n] = x[m x k] . W[n x k]^T.  w_bytes must be at least n * gllmq_row_bytes(dtype,k).
  * Alignment: w_dev 16 bytes for Q4_K/Q5_K, 2 bytes for Q6_K/Q8_0; x_dev 16, y_dev 4.
- * m <= 8 runs the bandwidth (GEMV) kernels with f32 activations and f32 accumulation;
- * larger m runs the MFMA kernels with GLLMQ_ACT_F32_SPLIT activations. */
+ * Q4_K runs on the int8 matrix cores: activations become three signed base-256 digits of a
+ * per-block fixed-point value, digit products accumulate exactly in i32, scales and the
+ * final sum are f32; one pass over the weights serves up to 8 activation rows, larger m
+ * takes ceil(m / 8) passes.  Q5_K / Q6_K / Q8_0 run integer-dot GEMV kernels, two
+ * activation rows per pass. */
 int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev,
                            float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,
                            void *stream);
 
-/* Same, with the activation mode of the MFMA path chosen by the caller (ignored for m <= 8). */
+/* Same, with the activation mode chosen by the caller. */
 int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes,
                               const float *x_dev, float *y_dev, uint32_t ggml_dtype, size_t m,
                               size_t n, size_t k, int act_mode, void *stream);

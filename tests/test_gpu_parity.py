@@ -36,11 +36,11 @@ def check_close(got, want, what=""):
     return rel
 
 
-def gpu_matmul(hip, torch, w, x, dtype, m, n, k):
+def gpu_matmul(hip, torch, w, x, dtype, m, n, k, act_mode=0):
     wd = hip.upload_weights(w)
     xd = torch.from_numpy(np.ascontiguousarray(x, np.float32)).cuda()
     yd = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
-    hip.quantized_matmul(wd, xd, yd, dtype, m, n, k)
+    hip.quantized_matmul(wd, xd, yd, dtype, m, n, k, act_mode=act_mode)
     torch.cuda.synchronize()
     return yd.cpu().numpy()
 
@@ -170,6 +170,69 @@ def test_baseline_shapes_match_oracle(hip, torch, oracle, dtype, n, k):
         out = np.zeros((1, n), np.float32)
         hip.quantized_matmul(w, x, out, dtype, 1, n, k)
         assert np.array_equal(out, got)
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("m", [9, 16, 33])
+def test_batched_m_matches_oracle(hip, torch, oracle, dtype, m):
+    n, k = 203, 2048
+    print(f"batched-m dtype={dtype} m={m}", flush=True)
+    w, x = random_weight(dtype, n, k, seed=m), random_activations(m, k, seed=m + 1)
+    want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+    got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+    check_close(got, want, f"dtype={dtype} m={m}")
+
+
+@pytest.mark.parametrize("m", [16, 32, 64])
+def test_batched_decode_baseline_shape(hip, torch, oracle, m):
+    # Q4_K, K=4096, N=14336, M in {16, 32, 64}
+    n, k = 14336, 4096
+    print(f"batched decode m={m}", flush=True)
+    w, x = random_weight(Q4_K, n, k, seed=0), random_activations(m, k, seed=5)
+    want = oracle.quantized_matmul(w, x, Q4_K, m, n, k, acc=oracle.ACC_F64, threads=16)
+    got = gpu_matmul(hip, torch, w, x, Q4_K, m, n, k)
+    rel = check_close(got, want, f"m={m}")
+    print(f"  rel_l2={rel:.3e}", flush=True)
+
+
+def test_decode_layer_mix_batch(hip, torch, oracle):
+    """QKV 4096->6144 (Q4_K), O 4096->4096 (Q4_K), gate+up 4096->2x14336 (Q4_K), down 14336->4096
+    (Q6_K) enqueued by one batch call, each fed a fresh N(0,1) vector."""
+    print("layer mix", flush=True)
+    ops = [(Q4_K, 6144, 4096), (Q4_K, 4096, 4096), (Q4_K, 2 * 14336, 4096), (Q6_K, 4096, 14336)]
+    descs, wants, outs = [], [], []
+    for i, (dtype, n, k) in enumerate(ops):
+        w, x = random_weight(dtype, n, k, seed=20 + i), random_activations(1, k, seed=30 + i)
+        wants.append(oracle.quantized_matmul(w, x, dtype, 1, n, k, acc=oracle.ACC_F64, threads=16))
+        wd = hip.upload_weights(w)
+        xd = torch.from_numpy(x).cuda()
+        yd = torch.full((1, n), float("nan"), dtype=torch.float32, device="cuda")
+        descs.append((wd, xd, yd, dtype, 1, n, k))
+        outs.append(yd)
+    hip.quantized_matmul_batch(descs)
+    torch.cuda.synchronize()
+    for (dtype, n, k), yd, want in zip(ops, outs, wants):
+        check_close(yd.cpu().numpy(), want, f"layer mix dtype={dtype} n={n} k={k}")
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("m", [1, 16])
+def test_bf16_activation_mode(hip, torch, oracle, dtype, m):
+    """GLLMQ_ACT_BF16: exact weights times activations rounded to bf16 (ties to even)."""
+    from gllm_amd.backend import ACT_BF16
+    from oracle import npref
+    n, k = 301, 4096
+    print(f"bf16 activations dtype={dtype} m={m}", flush=True)
+    w, x = random_weight(dtype, n, k, seed=9), random_activations(m, k, seed=10)
+    assert npref.bf16_rne(np.array([1.0, -1.0], np.float32)).view(np.uint32).tolist() == [0x3F800000, 0xBF800000]
+    xb = npref.bf16_rne(x)
+    want = oracle.quantized_matmul(w, xb, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+    got = gpu_matmul(hip, torch, w, x, dtype, m, n, k, act_mode=ACT_BF16)
+    check_close(got, want, f"bf16 dtype={dtype} m={m}")
+    # and it is a different computation from the f32 one: the rounding shows
+    full = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+    rel = np.linalg.norm(got - full) / np.linalg.norm(full)
+    assert rel > 3e-4, rel
 
 
 # ------------------------------------------------------------------- errors
