@@ -1,0 +1,145 @@
+// C++ host mirror of the reference's backend interface for the quantized-weight matmul path,
+// on top of the C ABI in gllm_hip_quant.h.  Header-only; link with libgllm_hip_quant.so.
+//
+// Mirrors (paths inside putao520/gllm):
+//   trait Backend<E>::quantized_matmul / ::dequantize   src/compat/mod.rs:233-256
+//   enum BackendError                                   src/engine/executor_types.rs:322-329
+//   enum QuantType (kernel-side format names)           src/loader/adapter.rs:138-191
+//   GgmlDType::{block_size, block_bytes}                src/loader/gguf/types.rs:152-236
+//
+// The reference's methods take host slices (`&[u8]`, `&[E]`, `&mut [E]`) and return
+// `Result<(), BackendError>`; the methods below keep the names, argument order and meaning
+// and return a BackendError value whose kind is None on success.  Device-resident forms
+// (`*_device`) take HIP device pointers and a stream and are the ones a GPU executor uses:
+// weights are uploaded once (src/compat/hip_backend.rs:141-156) and stay put.
+#ifndef GLLM_HIP_QUANT_HPP
+#define GLLM_HIP_QUANT_HPP
+
+#include <cstddef>
+#include <cstdint>
+#include <string>
+
+#include "gllm_hip_quant.h"
+
+namespace gllm {
+
+// Names follow QuantType of the reference; values are the GGUF type ids.
+enum class QuantType : uint32_t {
+    Q4_0 = 2, Q4_1 = 3, Q5_0 = 6, Q5_1 = 7, Q8_0 = 8, Q8_1 = 9,
+    Q2K = 10, Q3K = 11, Q4K = 12, Q5K = 13, Q6K = 14, Q8K = 15,
+};
+
+struct BackendError {
+    enum class Kind { None, Hip, Unimplemented, Other };
+    Kind kind = Kind::None;
+    std::string message;
+    bool ok() const { return kind == Kind::None; }
+    explicit operator bool() const { return !ok(); } // true when an error is held
+};
+
+inline size_t block_size(QuantType t) { return gllmq_block_size(static_cast<uint32_t>(t)); }
+inline size_t block_bytes(QuantType t) { return gllmq_block_bytes(static_cast<uint32_t>(t)); }
+inline size_t row_bytes(QuantType t, size_t k) { return gllmq_row_bytes(static_cast<uint32_t>(t), k); }
+
+class HipBackend {
+public:
+    explicit HipBackend(int device = 0)
+    {
+        const int rc = gllmq_init(&ctx_, device);
+        if (rc != GLLMQ_OK) {
+            ctx_ = nullptr;
+            init_error_ = make(rc, "gllmq_init");
+        }
+    }
+    ~HipBackend() { gllmq_destroy(ctx_); }
+    HipBackend(const HipBackend &) = delete;
+    HipBackend &operator=(const HipBackend &) = delete;
+
+    const BackendError &init_error() const { return init_error_; }
+
+    // fn quantized_matmul(&self, weight_blocks, input, output, quant_type, m, n, k)
+    BackendError quantized_matmul(const uint8_t *weight_blocks, size_t weight_len, const float *input, size_t input_len,
+                                  float *output, size_t output_len, QuantType quant_type, size_t m, size_t n,
+                                  size_t k) const
+    {
+        if (!ctx_) return init_error_;
+        if (input_len < m * k || output_len < m * n)
+            return BackendError{ BackendError::Kind::Other, "quantized_matmul: input/output shorter than m*k / m*n" };
+        return make(gllmq_quantized_matmul_host(ctx_, weight_blocks, weight_len, input, output,
+                                                static_cast<uint32_t>(quant_type), m, n, k),
+                    "quantized_matmul");
+    }
+
+    // fn dequantize(&self, block_data, output, quant_type)
+    BackendError dequantize(const uint8_t *block_data, size_t block_len, float *output, size_t output_len,
+                            QuantType quant_type) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_dequantize_host(ctx_, block_data, block_len, output, output_len,
+                                          static_cast<uint32_t>(quant_type)),
+                    "dequantize");
+    }
+
+    // Device-resident forms: all pointers are HIP device addresses, `stream` a hipStream_t.
+    BackendError quantized_matmul_device(const void *w_dev, size_t w_bytes, const float *x_dev, float *y_dev,
+                                         QuantType quant_type, size_t m, size_t n, size_t k, void *stream = nullptr,
+                                         int act_mode = GLLMQ_ACT_F32_SPLIT) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_quantized_matmul_ex(ctx_, w_dev, w_bytes, x_dev, y_dev, static_cast<uint32_t>(quant_type), m,
+                                              n, k, act_mode, stream),
+                    "quantized_matmul");
+    }
+
+    BackendError dequantize_device(const void *blocks_dev, size_t n_bytes, float *out_dev, size_t n_out,
+                                   QuantType quant_type, void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_dequantize(ctx_, blocks_dev, n_bytes, out_dev, n_out, static_cast<uint32_t>(quant_type),
+                                     stream),
+                    "dequantize");
+    }
+
+    BackendError quantized_matmul_batch_device(const gllmq_matmul_desc *descs, size_t count,
+                                               void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_quantized_matmul_batch(ctx_, descs, count, stream), "quantized_matmul_batch");
+    }
+
+    // Expert FFN over a route table (ExpertRouteTable, src/moe/routing.rs:100-173).
+    BackendError moe_matvec_device(const void *gate_up_dev, QuantType t_gate_up, const void *down_dev, QuantType t_down,
+                                   const float *x_dev, float *out_dev, size_t tokens, size_t hidden, size_t ffn,
+                                   size_t experts, size_t top_k, const uint32_t *route_expert_dev,
+                                   const float *route_weight_dev, const uint32_t *route_len_dev, bool relu_gate = false,
+                                   void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_moe_matvec(ctx_, gate_up_dev, static_cast<uint32_t>(t_gate_up), down_dev,
+                                     static_cast<uint32_t>(t_down), x_dev, out_dev, tokens, hidden, ffn, experts, top_k,
+                                     route_expert_dev, route_weight_dev, route_len_dev, relu_gate ? 1 : 0, stream),
+                    "moe_matvec");
+    }
+
+    gllmq_ctx *raw() const { return ctx_; }
+
+private:
+    BackendError make(int rc, const char *what) const
+    {
+        if (rc == GLLMQ_OK) return BackendError{};
+        std::string msg = ctx_ ? gllmq_last_error(ctx_) : "";
+        if (msg.empty()) msg = std::string(what) + ": " + gllmq_status_string(rc);
+        switch (rc) {
+        case GLLMQ_ERR_UNIMPLEMENTED: return BackendError{ BackendError::Kind::Unimplemented, msg };
+        case GLLMQ_ERR_HIP: return BackendError{ BackendError::Kind::Hip, msg };
+        default: return BackendError{ BackendError::Kind::Other, msg };
+        }
+    }
+
+    gllmq_ctx *ctx_ = nullptr;
+    BackendError init_error_;
+};
+
+} // namespace gllm
+
+#endif

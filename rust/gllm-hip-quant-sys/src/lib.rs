@@ -1,0 +1,147 @@
+//! Raw bindings to `libgllm_hip_quant.so` (include/gllm_hip_quant.h) and the safe wrapper that
+//! plugs into gllm's `Backend` trait for the quantized-weight matmul path.
+//!
+//! Replaces the `Unimplemented` defaults of `Backend::quantized_matmul` / `Backend::dequantize`
+//! (src/compat/mod.rs:233-256) for the HIP backend (src/compat/hip_backend.rs).
+#![allow(non_camel_case_types)]
+
+use std::ffi::{c_char, c_int, c_void, CStr};
+
+#[repr(C)]
+pub struct gllmq_ctx {
+    _private: [u8; 0],
+}
+
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct gllmq_matmul_desc {
+    pub w_dev: *const c_void,
+    pub w_bytes: usize,
+    pub x_dev: *const f32,
+    pub y_dev: *mut f32,
+    pub ggml_dtype: u32,
+    pub reserved: u32,
+    pub m: usize,
+    pub n: usize,
+    pub k: usize,
+}
+
+pub const GLLMQ_OK: c_int = 0;
+pub const GLLMQ_ERR_UNIMPLEMENTED: c_int = 1;
+pub const GLLMQ_ERR_BAD_SHAPE: c_int = 2;
+pub const GLLMQ_ERR_BAD_ALIGNMENT: c_int = 3;
+pub const GLLMQ_ERR_HIP: c_int = 4;
+pub const GLLMQ_ERR_INVALID: c_int = 5;
+pub const GLLMQ_ACT_F32_SPLIT: c_int = 0;
+pub const GLLMQ_ACT_BF16: c_int = 1;
+
+extern "C" {
+    pub fn gllmq_init(out_ctx: *mut *mut gllmq_ctx, device: c_int) -> c_int;
+    pub fn gllmq_destroy(ctx: *mut gllmq_ctx);
+    pub fn gllmq_last_error(ctx: *const gllmq_ctx) -> *const c_char;
+    pub fn gllmq_status_string(status: c_int) -> *const c_char;
+    pub fn gllmq_version() -> *const c_char;
+    pub fn gllmq_block_size(ggml_dtype: u32) -> usize;
+    pub fn gllmq_block_bytes(ggml_dtype: u32) -> usize;
+    pub fn gllmq_row_bytes(ggml_dtype: u32, k: usize) -> usize;
+    pub fn gllmq_dequantize(ctx: *mut gllmq_ctx, blocks_dev: *const c_void, n_bytes: usize, out_dev: *mut f32,
+                            n_out: usize, ggml_dtype: u32, stream: *mut c_void) -> c_int;
+    pub fn gllmq_quantized_matmul(ctx: *mut gllmq_ctx, w_dev: *const c_void, w_bytes: usize, x_dev: *const f32,
+                                  y_dev: *mut f32, ggml_dtype: u32, m: usize, n: usize, k: usize,
+                                  stream: *mut c_void) -> c_int;
+    pub fn gllmq_quantized_matmul_ex(ctx: *mut gllmq_ctx, w_dev: *const c_void, w_bytes: usize, x_dev: *const f32,
+                                     y_dev: *mut f32, ggml_dtype: u32, m: usize, n: usize, k: usize,
+                                     act_mode: c_int, stream: *mut c_void) -> c_int;
+    pub fn gllmq_quantized_matmul_batch(ctx: *mut gllmq_ctx, descs: *const gllmq_matmul_desc, count: usize,
+                                        stream: *mut c_void) -> c_int;
+    pub fn gllmq_moe_matvec(ctx: *mut gllmq_ctx, gate_up_dev: *const c_void, dtype_gate_up: u32,
+                            down_dev: *const c_void, dtype_down: u32, x_dev: *const f32, out_dev: *mut f32,
+                            tokens: usize, hidden: usize, ffn: usize, experts: usize, top_k: usize,
+                            route_expert_dev: *const u32, route_weight_dev: *const f32,
+                            route_len_dev: *const u32, relu_gate: c_int, stream: *mut c_void) -> c_int;
+    pub fn gllmq_dequantize_host(ctx: *mut gllmq_ctx, blocks: *const c_void, n_bytes: usize, out: *mut f32,
+                                 n_out: usize, ggml_dtype: u32) -> c_int;
+    pub fn gllmq_quantized_matmul_host(ctx: *mut gllmq_ctx, w: *const c_void, w_bytes: usize, x: *const f32,
+                                       y: *mut f32, ggml_dtype: u32, m: usize, n: usize, k: usize) -> c_int;
+}
+
+/// Owner of one library context (one per device).  `Send + Sync` like the trait demands
+/// (src/compat/mod.rs:77): the library keeps no mutable state per call except the MoE
+/// workspace, which it guards itself.
+pub struct HipQuant {
+    ctx: *mut gllmq_ctx,
+}
+unsafe impl Send for HipQuant {}
+unsafe impl Sync for HipQuant {}
+
+/// Mirrors gllm's `BackendError` variants used on this path
+/// (src/engine/executor_types.rs:322-329).
+#[derive(Debug, Clone)]
+pub enum QuantError {
+    Hip(String),
+    Unimplemented(&'static str),
+    Other(String),
+}
+
+impl HipQuant {
+    pub fn new(device: i32) -> Result<Self, QuantError> {
+        let mut ctx = std::ptr::null_mut();
+        let rc = unsafe { gllmq_init(&mut ctx, device) };
+        if rc != GLLMQ_OK {
+            return Err(QuantError::Hip(format!("gllmq_init failed with status {rc}")));
+        }
+        Ok(Self { ctx })
+    }
+
+    fn check(&self, rc: c_int, what: &'static str) -> Result<(), QuantError> {
+        if rc == GLLMQ_OK {
+            return Ok(());
+        }
+        let msg = unsafe { CStr::from_ptr(gllmq_last_error(self.ctx)) }.to_string_lossy().into_owned();
+        Err(match rc {
+            GLLMQ_ERR_UNIMPLEMENTED => QuantError::Unimplemented(what),
+            GLLMQ_ERR_HIP => QuantError::Hip(msg),
+            _ => QuantError::Other(msg),
+        })
+    }
+
+    /// `Backend::quantized_matmul` with host slices (the trait's signature); `ggml_dtype` is
+    /// `quant_type_to_ggml_dtype(quant_type) as u32` (src/loader/adapter.rs:90-130).
+    pub fn quantized_matmul(&self, weight_blocks: &[u8], input: &[f32], output: &mut [f32], ggml_dtype: u32,
+                            m: usize, n: usize, k: usize) -> Result<(), QuantError> {
+        if input.len() < m * k || output.len() < m * n {
+            return Err(QuantError::Other("quantized_matmul: input/output shorter than m*k / m*n".into()));
+        }
+        let rc = unsafe {
+            gllmq_quantized_matmul_host(self.ctx, weight_blocks.as_ptr().cast(), weight_blocks.len(), input.as_ptr(),
+                                        output.as_mut_ptr(), ggml_dtype, m, n, k)
+        };
+        self.check(rc, "quantized_matmul")
+    }
+
+    /// `Backend::dequantize` with host slices.
+    pub fn dequantize(&self, block_data: &[u8], output: &mut [f32], ggml_dtype: u32) -> Result<(), QuantError> {
+        let rc = unsafe {
+            gllmq_dequantize_host(self.ctx, block_data.as_ptr().cast(), block_data.len(), output.as_mut_ptr(),
+                                  output.len(), ggml_dtype)
+        };
+        self.check(rc, "dequantize")
+    }
+
+    /// Device-resident form used by the executor: `w`, `x`, `y` are HIP device addresses of
+    /// tensors the HIP backend already owns (src/compat/hip_backend.rs:141-156).
+    ///
+    /// # Safety
+    /// The pointers must be valid device allocations of the stated sizes on this context's device.
+    pub unsafe fn quantized_matmul_device(&self, w: *const c_void, w_bytes: usize, x: *const f32, y: *mut f32,
+                                          ggml_dtype: u32, m: usize, n: usize, k: usize,
+                                          stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_quantized_matmul(self.ctx, w, w_bytes, x, y, ggml_dtype, m, n, k, stream), "quantized_matmul")
+    }
+}
+
+impl Drop for HipQuant {
+    fn drop(&mut self) {
+        unsafe { gllmq_destroy(self.ctx) }
+    }
+}
