@@ -297,11 +297,14 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     if (!ctx->use_mm8 || f.dtype != T_Q4_K) return -1;
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
-    if (mm8_lds_bytes(groups, static_cast<uint32_t>(std::min<size_t>(m, 8)), m <= 2 ? 1u : (m <= 4 ? 2u : 4u)) >
-        152u * 1024u)
-        return -1;
-    for (size_t m0 = 0; m0 < m; m0 += 8) {
-        const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(8, m - m0));
+    // Rows per pass: as many as the prepared activations leave room for in the 160 KiB of LDS.
+    auto pairs_for = [](uint32_t rows) { return rows <= 2 ? 1u : (rows <= 4 ? 2u : 4u); };
+    uint32_t rows_per_pass = static_cast<uint32_t>(std::min<size_t>(m, 8));
+    while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass)) > 160u * 1024u)
+        --rows_per_pass;
+    if (rows_per_pass == 0) return -1;
+    for (size_t m0 = 0; m0 < m; m0 += rows_per_pass) {
+        const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(rows_per_pass, m - m0));
         const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
         const uint32_t pairs = 1u << pi;
         const uint32_t lds = mm8_lds_bytes(groups, mm, pairs);
