@@ -80,6 +80,34 @@ struct Mm8Params {
     uint32_t n, k, groups, row_bytes, m, ldx, ldy, tiles, grid, act_bf16;
 };
 
+// Mirror of gq::MmfParams in mmf.hip.inc.
+struct MmfParams {
+    const uint8_t *w;
+    const float *x;
+    float *y;
+    uint8_t *ximg;
+    float *partial;
+    uint32_t *counters;
+    uint32_t n, k, groups, row_bytes, m, ldx, ldy, row_tiles, ksplit, blocks_per_split, act_bf16;
+};
+struct MmfPrepParams {
+    const float *x;
+    uint8_t *ximg;
+    uint32_t m, k, ldx, act_bf16;
+};
+
+// gq::MmfLds<MT>::image: bytes of one block's activation image (hi, sums, inverse scales, lo),
+// padded to whole rounds of 256 x 16 bytes.
+uint32_t mmf_image_bytes(uint32_t mt)
+{
+    const uint32_t rows = 32u * mt;
+    const uint32_t raw = rows * 528u * 2u + rows * 32u + rows * 4u;
+    return (raw + 4095u) / 4096u * 4096u;
+}
+
+// gq::MmfLds<MT>::total.
+uint32_t mmf_lds_bytes(uint32_t mt) { return mmf_image_bytes(mt) + 16u + 4u * 2u * 5120u; }
+
 // Mirrors of the structs in moe.hip.inc.
 struct MoeJob {
     uint32_t expert, p0, m, t0, t1;
@@ -137,6 +165,14 @@ struct gllmq_ctx {
     hipFunction_t mm8_q4k[3][3] = {};           // int8 matrix-core kernels [pairs 1,2,4][early steps 1,2,4]
     bool use_mm8 = true;                        // GLLMQ_MM8=0 falls back to the GEMV kernels
     hipFunction_t stream_read = nullptr;
+    hipFunction_t mmf_q4k[2][2] = {};           // f16 matrix-core GEMM [32-row activation tiles - 1][bf16 mode]
+    hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
+    bool use_mmf = true;                        // GLLMQ_MMF=0 keeps m > 8 on the 8-row passes
+    // Scratch of the GEMM: partial sums of K-split workgroups and their arrival counters
+    // (zero between launches).  Shared by all calls on this context, like `workspace`.
+    void *mmf_partial = nullptr;
+    size_t mmf_partial_bytes = 0;
+    uint32_t *mmf_counters = nullptr;
     hipFunction_t moe_plan = nullptr, moe_act = nullptr, moe_combine = nullptr;
     hipFunction_t moe_gemv[kNumFormats] = {};
     // Device workspace of the MoE path (pair tables, jobs, intermediate activations).  It
@@ -334,6 +370,74 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     return GLLMQ_OK;
 }
 
+// Q4_K with 9 or more activation rows: f16 matrix-core GEMM, 64 rows per pass, weights read
+// once per pass.  Returns -1 when the shape does not fit (alignment), like run_mm8.
+constexpr uint32_t kMmfMaxRowTiles = 16384;
+
+int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
+            size_t k, bool act_bf16, void *stream)
+{
+    if (!ctx->use_mmf || f.dtype != T_Q4_K || m < 9) return -1;
+    if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
+    const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
+    const uint32_t row_tiles = static_cast<uint32_t>((n + 255) / 256);
+    if (row_tiles > kMmfMaxRowTiles) return -1;
+    uint32_t ksplit = std::max(1u, static_cast<uint32_t>(ctx->num_cus) / row_tiles);
+    if (const char *v = getenv("GLLMQ_MMF_KSPLIT")) ksplit = static_cast<uint32_t>(std::max(1, atoi(v)));
+    ksplit = std::min(ksplit, groups);
+    const uint32_t bps = (groups + ksplit - 1) / ksplit;
+    ksplit = (groups + bps - 1) / bps; // every workgroup gets at least one block
+    std::lock_guard<std::mutex> guard(ctx->workspace_mutex);
+    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
+    if (!ctx->mmf_counters) {
+        GLLMQ_HIP(ctx, hipMalloc(reinterpret_cast<void **>(&ctx->mmf_counters), kMmfMaxRowTiles * 4));
+        GLLMQ_HIP(ctx, hipMemset(ctx->mmf_counters, 0, kMmfMaxRowTiles * 4));
+    }
+    const size_t rows_per_pass = 64;
+    // scratch: the activation images of one pass, then the partial sums
+    const size_t img_bytes = static_cast<size_t>(groups) * mmf_image_bytes(m <= 32 ? 1u : 2u);
+    const size_t need = img_bytes + (ksplit > 1 ? static_cast<size_t>(ksplit) * std::min(m, rows_per_pass) * n * 4 : 0);
+    if (ctx->mmf_partial_bytes < need) {
+        if (ctx->mmf_partial) {
+            GLLMQ_HIP(ctx, hipDeviceSynchronize()); // earlier calls may still be using it
+            GLLMQ_HIP(ctx, hipFree(ctx->mmf_partial));
+            ctx->mmf_partial = nullptr;
+            ctx->mmf_partial_bytes = 0;
+        }
+        GLLMQ_HIP(ctx, hipMalloc(&ctx->mmf_partial, need));
+        ctx->mmf_partial_bytes = need;
+    }
+    for (size_t m0 = 0; m0 < m; m0 += rows_per_pass) {
+        const uint32_t mm = static_cast<uint32_t>(std::min(rows_per_pass, m - m0));
+        const uint32_t mt = mm <= 32 ? 1u : 2u;
+        MmfParams P{};
+        P.w = w;
+        P.x = x + m0 * k;
+        P.y = y + m0 * n;
+        P.ximg = static_cast<uint8_t *>(ctx->mmf_partial);
+        P.partial = reinterpret_cast<float *>(static_cast<uint8_t *>(ctx->mmf_partial) + img_bytes);
+        P.counters = ctx->mmf_counters;
+        P.n = static_cast<uint32_t>(n);
+        P.k = static_cast<uint32_t>(k);
+        P.groups = groups;
+        P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
+        P.m = mm;
+        P.ldx = static_cast<uint32_t>(k);
+        P.ldy = static_cast<uint32_t>(n);
+        P.row_tiles = row_tiles;
+        P.ksplit = ksplit;
+        P.blocks_per_split = bps;
+        P.act_bf16 = act_bf16 ? 1u : 0u;
+        MmfPrepParams Q{ P.x, P.ximg, mm, P.k, P.ldx, P.act_bf16 };
+        int rc = launch(ctx, ctx->mmf_prep[mt - 1], groups, 256, 0, stream, &Q, sizeof Q);
+        if (rc != GLLMQ_OK) return rc;
+        rc = launch(ctx, ctx->mmf_q4k[mt - 1][act_bf16 ? 1 : 0], row_tiles * ksplit, 256, mmf_lds_bytes(mt), stream,
+                    &P, sizeof P);
+        if (rc != GLLMQ_OK) return rc;
+    }
+    return GLLMQ_OK;
+}
+
 int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
              size_t k, bool act_bf16, void *stream)
 {
@@ -435,6 +539,12 @@ int gllmq_init(gllmq_ctx **out, int device)
         }
     }
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->stream_read, "gq_stream_read");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[0], "gq_mmf_prep_t1");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[1], "gq_mmf_prep_t2");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_q4k[0][0], "gq_mmf_q4k_t1");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_q4k[1][0], "gq_mmf_q4k_t2");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_q4k[0][1], "gq_mmf_q4k_t1_bf16");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_q4k[1][1], "gq_mmf_q4k_t2_bf16");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_plan, "gq_moe_plan");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_act, "gq_moe_act");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_combine, "gq_moe_combine");
@@ -459,6 +569,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     ctx->gemv_waves = static_cast<uint32_t>(ctx->num_cus) * 8u;
     if (const char *v = getenv("GLLMQ_GEMV_F32")) ctx->gemv_f32 = (v[0] == '1');
     if (const char *v = getenv("GLLMQ_MM8")) ctx->use_mm8 = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_MMF")) ctx->use_mmf = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_GEMV_WAVES")) {
         long w = strtol(v, nullptr, 10);
         if (w >= 4 && w <= 65536) ctx->gemv_waves = static_cast<uint32_t>(w);
@@ -471,6 +582,8 @@ void gllmq_destroy(gllmq_ctx *ctx)
 {
     if (!ctx) return;
     if (ctx->workspace) (void)hipFree(ctx->workspace);
+    if (ctx->mmf_partial) (void)hipFree(ctx->mmf_partial);
+    if (ctx->mmf_counters) (void)hipFree(ctx->mmf_counters);
     if (ctx->module) (void)hipModuleUnload(ctx->module);
     delete ctx;
 }
@@ -513,6 +626,8 @@ int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, con
     const bool bf16 = act_mode == GLLMQ_ACT_BF16;
     if (bf16 && ctx->gemv_f32)
         return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "quantized_matmul: bf16 activations are not built for GLLMQ_GEMV_F32=1");
+    rc = run_mmf(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
+    if (rc >= 0) return rc;
     rc = run_mm8(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
     if (rc >= 0) return rc;
     return run_gemv(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);

@@ -10,5 +10,6 @@
 #include "gemv.hip.inc"
 #include "gemv_i8.hip.inc"
 #include "mm8.hip.inc"
+#include "mmf.hip.inc"
 #include "moe.hip.inc"
 #include "probe.hip.inc"
