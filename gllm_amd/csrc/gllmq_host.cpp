@@ -102,11 +102,11 @@ uint32_t mmf_image_bytes(uint32_t mt)
 {
     const uint32_t rows = 32u * mt;
     const uint32_t raw = rows * 528u * 2u + rows * 32u + rows * 4u;
-    return (raw + 4095u) / 4096u * 4096u;
+    return (raw + 8191u) / 8192u * 8192u; // whole rounds of 512 threads x 16 bytes
 }
 
-// gq::MmfLds<MT>::total.
-uint32_t mmf_lds_bytes(uint32_t mt) { return mmf_image_bytes(mt) + 16u + 4u * 2u * 5120u; }
+// gq::MmfLds<MT>::total: image, flag, one 5 KiB weight stage per wave.
+uint32_t mmf_lds_bytes(uint32_t mt) { return mmf_image_bytes(mt) + 16u + 8u * 5120u; }
 
 // Mirrors of the structs in moe.hip.inc.
 struct MoeJob {
@@ -370,14 +370,15 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     return GLLMQ_OK;
 }
 
-// Q4_K with 9 or more activation rows: f16 matrix-core GEMM, 64 rows per pass, weights read
+// Q4_K with more than 16 activation rows: f16 matrix-core GEMM, 64 rows per pass, weights read
 // once per pass.  Returns -1 when the shape does not fit (alignment), like run_mm8.
 constexpr uint32_t kMmfMaxRowTiles = 16384;
 
 int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
             size_t k, bool act_bf16, void *stream)
 {
-    if (!ctx->use_mmf || f.dtype != T_Q4_K || m < 9) return -1;
+    // up to 16 rows two 8-row passes of the int8 kernel are as fast
+    if (!ctx->use_mmf || f.dtype != T_Q4_K || m <= 16) return -1;
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
     const uint32_t row_tiles = static_cast<uint32_t>((n + 255) / 256);
@@ -431,7 +432,7 @@ int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         MmfPrepParams Q{ P.x, P.ximg, mm, P.k, P.ldx, P.act_bf16 };
         int rc = launch(ctx, ctx->mmf_prep[mt - 1], groups, 256, 0, stream, &Q, sizeof Q);
         if (rc != GLLMQ_OK) return rc;
-        rc = launch(ctx, ctx->mmf_q4k[mt - 1][act_bf16 ? 1 : 0], row_tiles * ksplit, 256, mmf_lds_bytes(mt), stream,
+        rc = launch(ctx, ctx->mmf_q4k[mt - 1][act_bf16 ? 1 : 0], row_tiles * ksplit, 512, mmf_lds_bytes(mt), stream,
                     &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }

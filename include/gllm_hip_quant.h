@@ -54,8 +54,6 @@ enum {
     GLLMQ_ACT_BF16 = 1
 };
 
-/* Rows of activations one pass over the weights serves (larger m runs several passes). */
-#define GLLMQ_ROWS_PER_PASS 8
 
 typedef struct gllmq_ctx gllmq_ctx;
 
@@ -86,9 +84,12 @@ int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks_dev, size_t n_bytes, flo
  * Alignment: w_dev 16 bytes for Q4_K/Q5_K, 2 bytes for Q6_K/Q8_0; x_dev 16, y_dev 4.
  * Q4_K runs on the int8 matrix cores: activations become three signed base-256 digits of a
  * per-block fixed-point value, digit products accumulate exactly in i32, scales and the
- * final sum are f32; one pass over the weights serves up to 8 activation rows, larger m
- * takes ceil(m / 8) passes.  Q5_K / Q6_K / Q8_0 run integer-dot GEMV kernels, two
- * activation rows per pass. */
+ * final sum are f32; one pass over the weights serves up to 8 activation rows.  More than
+ * 16 rows of Q4_K run a GEMM on the f16 matrix cores, 64 rows per pass: weights as the exact
+ * integers sc*q in f16, activations as two f16 terms (22 significant bits) of a per-block
+ * scaled value, f32 accumulation; its scratch (activation images, partial sums of the K
+ * split) lives in the context, so such calls on one context must not overlap in time.
+ * Q5_K / Q6_K / Q8_0 run integer-dot GEMV kernels, two activation rows per pass. */
 int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev,
                            float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,
                            void *stream);

@@ -173,7 +173,7 @@ def test_baseline_shapes_match_oracle(hip, torch, oracle, dtype, n, k):
 
 
 @pytest.mark.parametrize("dtype", ALL)
-@pytest.mark.parametrize("m", [9, 16, 33])
+@pytest.mark.parametrize("m", [9, 16, 17, 33, 70])
 def test_batched_m_matches_oracle(hip, torch, oracle, dtype, m):
     n, k = 203, 2048
     print(f"batched-m dtype={dtype} m={m}", flush=True)
@@ -216,7 +216,7 @@ def test_decode_layer_mix_batch(hip, torch, oracle):
 
 
 @pytest.mark.parametrize("dtype", ALL)
-@pytest.mark.parametrize("m", [1, 16])
+@pytest.mark.parametrize("m", [1, 16, 40])
 def test_bf16_activation_mode(hip, torch, oracle, dtype, m):
     """GLLMQ_ACT_BF16: exact weights times activations rounded to bf16 (ties to even)."""
     from gllm_amd.backend import ACT_BF16
