@@ -362,7 +362,7 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         int ei = steps <= 1 ? 0 : (steps <= 2 ? 1 : 2);
         while (ei < 2 && !ctx->mm8_q4k[pi][ei]) ++ei; // not every (pairs, early) pair is built
         uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
-        if (const char *v = getenv("GLLMQ_MM8_GRID")) grid = std::min<uint32_t>(grid, std::max(1, atoi(v)));
+        if (const char *v = getenv("GLLMQ_MM8_GRID")) grid = std::min<uint32_t>(P.tiles, std::max(1, atoi(v)));
         P.grid = grid;
         int rc = launch(ctx, ctx->mm8_q4k[pi][ei], grid, 512, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
