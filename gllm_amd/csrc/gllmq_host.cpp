@@ -722,13 +722,14 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
     {
         MoePlanParams P{ route_expert, route_len, pair_src, pair_pos, jobs, counters, static_cast<uint32_t>(tokens),
                          static_cast<uint32_t>(top_k), static_cast<uint32_t>(experts), static_cast<uint32_t>(pairs) };
-        const uint32_t lds = static_cast<uint32_t>((pairs + 3 * experts + 1024) * 4);
-        int rc = launch(ctx, ctx->moe_plan, 1, 1024, lds, stream, &P, sizeof P);
+        const uint32_t lds = static_cast<uint32_t>((pairs + 3 * experts + 4) * 4);
+        int rc = launch(ctx, ctx->moe_plan, 1, 256, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }
     // Waves per job: the device takes about 8 waves per CU of these kernels; the jobs that
     // exist (at most `pairs`, typically one per routed expert) share them.
-    const uint32_t job_waves = std::max<uint32_t>(16u, 4u * ctx->gemv_waves / static_cast<uint32_t>(pairs));
+    uint32_t job_waves = std::max<uint32_t>(16u, 4u * ctx->gemv_waves / static_cast<uint32_t>(pairs));
+    if (const char *v = getenv("GLLMQ_MOE_JOB_WAVES")) job_waves = static_cast<uint32_t>(std::max(4, atoi(v)));
     auto grouped = [&](const Format &f, const void *w, size_t rb, uint32_t n, uint32_t k, const float *xin,
                        bool x_by_token, float *yout) -> int {
         GemvPlan L = plan_gemv(ctx, 2, n, k, rb, job_waves);
