@@ -1,7 +1,11 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path: Q4_K dequantize-GEMV 1 x 4096 -> 14336 on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+Without --workload (or with gemv_q4k) it measures the headline configuration described
+below.  The other workloads are the remaining baseline configurations, timed the same way
+(one JSON line each): gemv_q4k_4096, gemv_q6k, layer_mix, gemm_m16, gemm_m32, gemm_m64, moe.
 
 A step is one call of the quantized matmul (m = 1) over one weight matrix.  The weights
 rotate over 16 distinct copies (528 MB) so that no cache level can serve them: every step
@@ -52,6 +56,154 @@ def device_weights(torch, n_rows: int, k: int, copies: int):
     return out
 
 
+BLOCK_BYTES = {8: 34, 12: 144, 13: 176, 14: 210}
+TAGS = {8: "Q8_0", 12: "Q4_K", 13: "Q5_K", 14: "Q6_K"}
+
+
+def device_weight_any(torch, g, dtype: int, rows: int, k: int):
+    """Random blocks of any of the four formats generated on the device (distributions of the
+    baseline configurations: uniform quants, f16 d / dmin in (0.001, 0.05), Q6_K d in
+    (0.001, 0.02) with int8 scales in -64..63)."""
+    from gllm_amd.ggml import row_bytes
+    w = torch.randint(0, 256, (rows * row_bytes(dtype, k),), dtype=torch.uint8, device="cuda", generator=g)
+    b = w.view(-1, BLOCK_BYTES[dtype])
+    nb = b.shape[0]
+    if dtype in (12, 13):
+        d = (torch.rand(nb, 2, device="cuda", generator=g) * 0.049 + 0.001).to(torch.float16)
+        b[:, 0:4] = d.view(torch.uint8).view(-1, 4)
+    elif dtype == 14:
+        d = (torch.rand(nb, 1, device="cuda", generator=g) * 0.019 + 0.001).to(torch.float16)
+        b[:, 208:210] = d.view(torch.uint8).view(-1, 2)
+        b[:, 192:208] = ((b[:, 192:208] & 0x7F).to(torch.int16) - 64).to(torch.int8).view(torch.uint8)
+    else:
+        d = (torch.rand(nb, 1, device="cuda", generator=g) * 0.049 + 0.001).to(torch.float16)
+        b[:, 0:2] = d.view(torch.uint8).view(-1, 2)
+    return w
+
+
+def run_other(args):
+    """The baseline configurations other than the headline one.  Same timing method: the timed
+    steps are enqueued back to back on one stream between two events, weights rotate over
+    enough copies to exceed the 256 MB Infinity Cache."""
+    import numpy as np
+    import torch
+
+    from gllm_amd.backend import HipBackend
+    from gllm_amd.ggml import row_bytes
+    from gllm_amd.synth import random_activations, random_gate_logits, random_weight
+    from oracle import cref
+
+    hip = HipBackend(0)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    threads = max(1, min(os.cpu_count() or 1, 16))
+    name = args.workload
+    steps = min(args.steps, 400)
+
+    def timed(fn, reps):
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(reps):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) * 1e3 / reps  # us
+
+    def cpu_time(fn, budget_s=8.0):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt > budget_s or reps >= 200:
+                return dt / reps, reps, dt
+
+    if name in ("gemv_q4k_4096", "gemv_q6k", "gemm_m16", "gemm_m32", "gemm_m64", "layer_mix"):
+        if name == "layer_mix":
+            ops = [(12, 6144, 4096, 1), (12, 4096, 4096, 1), (12, 2 * 14336, 4096, 1), (14, 4096, 14336, 1)]
+            copies = 3
+        else:
+            dtype, n, k, m = {"gemv_q4k_4096": (12, 4096, 4096, 1), "gemv_q6k": (14, 14336, 4096, 1),
+                              "gemm_m16": (12, 14336, 4096, 16), "gemm_m32": (12, 14336, 4096, 32),
+                              "gemm_m64": (12, 14336, 4096, 64)}[name]
+            ops = [(dtype, n, k, m)]
+            copies = max(2, (300 << 20) // (n * row_bytes(dtype, k)) + 1)
+        sets = []
+        for _ in range(copies):
+            sets.append([(device_weight_any(torch, g, dt, n, k), torch.randn(m, k, device="cuda", generator=g),
+                          torch.empty(m, n, device="cuda"), dt, m, n, k) for dt, n, k, m in ops])
+        flat = [d for st in sets for d in st]
+        hip.quantized_matmul_batch(flat)
+        reps = max(1, steps // copies)
+        us = timed(lambda: hip.quantized_matmul_batch(flat), reps) / copies
+        byts = sum(n * row_bytes(dt, k) + m * k * 4 + m * n * 4 for dt, n, k, m in ops)
+        flops = sum(2 * m * n * k for dt, n, k, m in ops)
+        desc = " + ".join(f"{TAGS[dt]} M={m} K={k} N={n}" for dt, n, k, m in ops)
+        # CPU: the oracle's reference-style path on the same shapes (bounded sample)
+        host = [(random_weight(dt, n, k, seed=i), random_activations(m, k, seed=i), dt, m, n, k)
+                for i, (dt, n, k, m) in enumerate(ops)]
+        sec, creps, cdt = cpu_time(lambda: [cref.quantized_matmul(w, x, dt, m, n, k, acc=cref.ACC_F32, threads=threads)
+                                            for w, x, dt, m, n, k in host])
+        sample = f"{creps} passes of the same shapes in {cdt:.1f} s"
+    elif name == "moe":
+        E, T, KK, H, F = 128, 16, 8, 4096, 1536
+        gu = device_weight_any(torch, g, 12, E * 2 * F, H)
+        dn = device_weight_any(torch, g, 14, E * H, F)
+        x = torch.randn(T, H, device="cuda", generator=g)
+        out = torch.empty(T, H, device="cuda")
+        tabs = []
+        for s_ in range(8):
+            # capacity factor = number of experts: nothing is dropped (the default 1.25 gives
+            # capacity 1 at 16 tokens over 128 experts and would drop most routes)
+            r = cref.route(random_gate_logits(T, E, seed=s_), KK, capacity_factor=float(E))
+            tabs.append((torch.from_numpy(r["expert"].view(np.int32)).cuda(), torch.from_numpy(r["weight"]).cuda(),
+                         torch.from_numpy(r["len"].view(np.int32)).cuda(), len(np.unique(r["expert"]))))
+        it = [0]
+
+        def run():
+            re_, rw, rl, _ = tabs[it[0] % len(tabs)]
+            it[0] += 1
+            hip.moe_matvec(gu, 12, dn, 14, x, out, H, F, E, re_, rw, rl)
+        run()
+        us = timed(run, max(8, steps // 4))
+        e_act = float(np.mean([t[3] for t in tabs]))
+        byts = int(e_act * (2 * F * row_bytes(12, H) + H * row_bytes(14, F)) + 128 * H * 4 + 128 * F * 8 + T * H * 4)
+        flops = 128 * 2 * (2 * F * H + H * F)
+        desc = (f"MoE expert matvec: {E} experts, top-{KK}, {T} tokens, gate/up Q4_K [{2 * F}x{H}], down Q6_K [{H}x{F}], "
+                f"{e_act:.1f} distinct experts hit per call on average, no capacity drop")
+        # CPU: 8 experts' worth of the same shapes (a sixteenth of the weights), 16 tokens top-2
+        Ec = 8
+        gu_h, dn_h = random_weight(12, Ec * 2 * F, H, seed=1), random_weight(14, Ec * H, F, seed=2)
+        rc_ = cref.route(random_gate_logits(T, Ec, seed=0), 2, capacity_factor=float(Ec))
+        xh = random_activations(T, H, seed=3)
+        pairs_c = int(rc_["len"].sum())
+        sec, creps, cdt = cpu_time(lambda: cref.moe_ffn(gu_h, 12, dn_h, 14, xh, H, F, Ec, rc_["expert"], rc_["weight"],
+                                                        rc_["len"], acc=cref.ACC_F32, threads=threads))
+        sec *= 128.0 / pairs_c  # the oracle works pair by pair: scale to the 128 pairs of the workload
+        sample = f"{creps} passes over {pairs_c} (token, expert) pairs of the same expert shapes in {cdt:.1f} s, scaled to 128 pairs"
+    else:
+        log(f"bench.py: unknown workload {name}")
+        sys.exit(2)
+
+    gbs = byts / us / 1e3
+    result = {
+        "metric": f"{name}: achieved HBM GB/s", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps,
+        "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6), "us_per_call": round(us, 3),
+        "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 2), "tflops": round(flops / us / 1e6, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "i8" if not name.startswith("gemm") else "f16", "data": "synthetic",
+        "config": {"workload": desc, "bytes_per_call": byts},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+        "cpu_baseline": {"value": round(byts / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+                         "us_per_call": round(sec * 1e6, 1), "sample": sample},
+    }
+    log(f"{name}: {us:.2f} us/call, {gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS * 100:.1f}% of 8 TB/s)")
+    print(json.dumps(result), flush=True)
+
+
 def cpu_baseline(budget_s: float = 12.0):
     """The oracle's reference-faithful matmul (per-block decode, f32 multiply-add) on the host
     cores, on the same shape with the same generator, repeated for about `budget_s` seconds."""
@@ -84,6 +236,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-context", action="store_true",
                     help="skip the cache-resident and streaming-read context runs (profiling: only the timed kernel launches)")
+    ap.add_argument("--workload", default="gemv_q4k",
+                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, gemm_m16, gemm_m32, gemm_m64, moe")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch plain device-to-device copies of one 33 MB weight buffer (counter calibration)")
     args = ap.parse_args()
@@ -100,6 +254,9 @@ def main():
     if not torch.cuda.is_available():
         log("bench.py: no GPU visible")
         sys.exit(1)
+    if args.workload != "gemv_q4k":
+        run_other(args)
+        return
     hip = HipBackend(0)
     ws = device_weights(torch, N, K_DIM, COPIES)
     g = torch.Generator(device="cuda")
