@@ -144,9 +144,12 @@ def run_other(args):
         # CPU: the oracle's reference-style path on the same shapes (bounded sample)
         host = [(random_weight(dt, n, k, seed=i), random_activations(m, k, seed=i), dt, m, n, k)
                 for i, (dt, n, k, m) in enumerate(ops)]
-        sec, creps, cdt = cpu_time(lambda: [cref.quantized_matmul(w, x, dt, m, n, k, acc=cref.ACC_F32, threads=threads)
-                                            for w, x, dt, m, n, k in host])
-        sample = f"{creps} passes of the same shapes in {cdt:.1f} s"
+        if args.no_cpu:
+            sec, sample = None, None
+        else:
+            sec, creps, cdt = cpu_time(lambda: [cref.quantized_matmul(w, x, dt, m, n, k, acc=cref.ACC_F32, threads=threads)
+                                                for w, x, dt, m, n, k in host])
+            sample = f"{creps} passes of the same shapes in {cdt:.1f} s"
     elif name == "moe":
         E, T, KK, H, F = 128, 16, 8, 4096, 1536
         gu = device_weight_any(torch, g, 12, E * 2 * F, H)
@@ -179,10 +182,14 @@ def run_other(args):
         rc_ = cref.route(random_gate_logits(T, Ec, seed=0), 2, capacity_factor=float(Ec))
         xh = random_activations(T, H, seed=3)
         pairs_c = int(rc_["len"].sum())
-        sec, creps, cdt = cpu_time(lambda: cref.moe_ffn(gu_h, 12, dn_h, 14, xh, H, F, Ec, rc_["expert"], rc_["weight"],
-                                                        rc_["len"], acc=cref.ACC_F32, threads=threads))
-        sec *= 128.0 / pairs_c  # the oracle works pair by pair: scale to the 128 pairs of the workload
-        sample = f"{creps} passes over {pairs_c} (token, expert) pairs of the same expert shapes in {cdt:.1f} s, scaled to 128 pairs"
+        if args.no_cpu:
+            sec, sample = None, None
+        else:
+            sec, creps, cdt = cpu_time(lambda: cref.moe_ffn(gu_h, 12, dn_h, 14, xh, H, F, Ec, rc_["expert"], rc_["weight"],
+                                                            rc_["len"], acc=cref.ACC_F32, threads=threads))
+            sec *= 128.0 / pairs_c  # the oracle works pair by pair: scale to the 128 pairs of the workload
+            sample = (f"{creps} passes over {pairs_c} (token, expert) pairs of the same expert shapes in {cdt:.1f} s, "
+                      f"scaled to 128 pairs")
     else:
         log(f"bench.py: unknown workload {name}")
         sys.exit(2)
@@ -197,9 +204,10 @@ def run_other(args):
         "config": {"workload": desc, "bytes_per_call": byts},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
-        "cpu_baseline": {"value": round(byts / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-                         "us_per_call": round(sec * 1e6, 1), "sample": sample},
     }
+    if sec is not None:
+        result["cpu_baseline"] = {"value": round(byts / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+                                  "us_per_call": round(sec * 1e6, 1), "sample": sample}
     log(f"{name}: {us:.2f} us/call, {gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS * 100:.1f}% of 8 TB/s)")
     print(json.dumps(result), flush=True)
 
