@@ -87,8 +87,12 @@ struct MmfParams {
     float *y;
     uint8_t *ximg;
     float *partial;
-    uint32_t *counters;
     uint32_t n, k, groups, row_bytes, m, ldx, ldy, row_tiles, ksplit, blocks_per_split, act_bf16;
+};
+struct MmfReduceParams {
+    const float *partial;
+    float *y;
+    uint32_t m, n, ldy, ksplit;
 };
 struct MmfPrepParams {
     const float *x;
@@ -105,8 +109,8 @@ uint32_t mmf_image_bytes(uint32_t mt)
     return (raw + 8191u) / 8192u * 8192u; // whole rounds of 512 threads x 16 bytes
 }
 
-// gq::MmfLds<MT>::total: image, flag, one 5 KiB weight stage per wave.
-uint32_t mmf_lds_bytes(uint32_t mt) { return mmf_image_bytes(mt) + 16u + 8u * 5120u; }
+// gq::MmfLds<MT>::total: image, one 5 KiB weight stage per wave.
+uint32_t mmf_lds_bytes(uint32_t mt) { return mmf_image_bytes(mt) + 8u * 5120u; }
 
 // Mirrors of the structs in moe.hip.inc.
 struct MoeJob {
@@ -167,12 +171,12 @@ struct gllmq_ctx {
     hipFunction_t stream_read = nullptr;
     hipFunction_t mmf_q4k[2][2] = {};           // f16 matrix-core GEMM [32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
+    hipFunction_t mmf_reduce = nullptr;         // and the in-order sum of its K-split partial results
     bool use_mmf = true;                        // GLLMQ_MMF=0 keeps m > 8 on the 8-row passes
-    // Scratch of the GEMM: partial sums of K-split workgroups and their arrival counters
-    // (zero between launches).  Shared by all calls on this context, like `workspace`.
+    // Scratch of the GEMM: activation images and partial sums of K-split workgroups.  Shared
+    // by all calls on this context, like `workspace`.
     void *mmf_partial = nullptr;
     size_t mmf_partial_bytes = 0;
-    uint32_t *mmf_counters = nullptr;
     hipFunction_t moe_plan = nullptr, moe_act = nullptr, moe_combine = nullptr;
     hipFunction_t moe_gemv[kNumFormats] = {};
     // Device workspace of the MoE path (pair tables, jobs, intermediate activations).  It
@@ -370,15 +374,14 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     return GLLMQ_OK;
 }
 
-// Q4_K with more than 16 activation rows: f16 matrix-core GEMM, 64 rows per pass, weights read
+// Q4_K with more than 8 activation rows: f16 matrix-core GEMM, 64 rows per pass, weights read
 // once per pass.  Returns -1 when the shape does not fit (alignment), like run_mm8.
 constexpr uint32_t kMmfMaxRowTiles = 16384;
 
 int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
             size_t k, bool act_bf16, void *stream)
 {
-    // up to 16 rows two 8-row passes of the int8 kernel are as fast
-    if (!ctx->use_mmf || f.dtype != T_Q4_K || m <= 16) return -1;
+    if (!ctx->use_mmf || f.dtype != T_Q4_K || m <= 8) return -1;
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
     const uint32_t row_tiles = static_cast<uint32_t>((n + 255) / 256);
@@ -390,10 +393,6 @@ int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     ksplit = (groups + bps - 1) / bps; // every workgroup gets at least one block
     std::lock_guard<std::mutex> guard(ctx->workspace_mutex);
     GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
-    if (!ctx->mmf_counters) {
-        GLLMQ_HIP(ctx, hipMalloc(reinterpret_cast<void **>(&ctx->mmf_counters), kMmfMaxRowTiles * 4));
-        GLLMQ_HIP(ctx, hipMemset(ctx->mmf_counters, 0, kMmfMaxRowTiles * 4));
-    }
     const size_t rows_per_pass = 64;
     // scratch: the activation images of one pass, then the partial sums
     const size_t img_bytes = static_cast<size_t>(groups) * mmf_image_bytes(m <= 32 ? 1u : 2u);
@@ -417,7 +416,6 @@ int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         P.y = y + m0 * n;
         P.ximg = static_cast<uint8_t *>(ctx->mmf_partial);
         P.partial = reinterpret_cast<float *>(static_cast<uint8_t *>(ctx->mmf_partial) + img_bytes);
-        P.counters = ctx->mmf_counters;
         P.n = static_cast<uint32_t>(n);
         P.k = static_cast<uint32_t>(k);
         P.groups = groups;
@@ -430,10 +428,15 @@ int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         P.blocks_per_split = bps;
         P.act_bf16 = act_bf16 ? 1u : 0u;
         MmfPrepParams Q{ P.x, P.ximg, mm, P.k, P.ldx, P.act_bf16 };
-        int rc = launch(ctx, ctx->mmf_prep[mt - 1], groups, 256, 0, stream, &Q, sizeof Q);
+        int rc = launch2d(ctx, ctx->mmf_prep[mt - 1], groups, 4, 64, 0, stream, &Q, sizeof Q);
         if (rc != GLLMQ_OK) return rc;
         rc = launch(ctx, ctx->mmf_q4k[mt - 1][act_bf16 ? 1 : 0], row_tiles * ksplit, 512, mmf_lds_bytes(mt), stream,
                     &P, sizeof P);
+        if (rc == GLLMQ_OK && ksplit > 1) {
+            MmfReduceParams R{ P.partial, P.y, mm, P.n, P.ldy, ksplit };
+            const uint64_t quads = (static_cast<uint64_t>(mm) * n + 3) / 4;
+            rc = launch(ctx, ctx->mmf_reduce, static_cast<uint32_t>((quads + 255) / 256), 256, 0, stream, &R, sizeof R);
+        }
         if (rc != GLLMQ_OK) return rc;
     }
     return GLLMQ_OK;
@@ -542,6 +545,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->stream_read, "gq_stream_read");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[0], "gq_mmf_prep_t1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[1], "gq_mmf_prep_t2");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_reduce, "gq_mmf_reduce");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_q4k[0][0], "gq_mmf_q4k_t1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_q4k[1][0], "gq_mmf_q4k_t2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_q4k[0][1], "gq_mmf_q4k_t1_bf16");
@@ -584,7 +588,6 @@ void gllmq_destroy(gllmq_ctx *ctx)
     if (!ctx) return;
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->mmf_partial) (void)hipFree(ctx->mmf_partial);
-    if (ctx->mmf_counters) (void)hipFree(ctx->mmf_counters);
     if (ctx->module) (void)hipModuleUnload(ctx->module);
     delete ctx;
 }
