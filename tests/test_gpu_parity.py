@@ -235,6 +235,25 @@ def test_bf16_activation_mode(hip, torch, oracle, dtype, m):
     assert rel > 3e-4, rel
 
 
+@pytest.mark.parametrize("env", [{"GLLMQ_MM8": "0", "GLLMQ_MMF": "0"}, {"GLLMQ_MMF": "0"},
+                                 {"GLLMQ_GEMV_F32": "1", "GLLMQ_MM8": "0", "GLLMQ_MMF": "0"}])
+def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
+    """The kernels the default dispatch does not pick: integer-dot GEMV for Q4_K, 8-row passes
+    for more than 8 rows, and the f32 multiply-add flavour; selected per context at init."""
+    from gllm_amd.backend import HipBackend
+    for k_, v_ in env.items():
+        monkeypatch.setenv(k_, v_)
+    hip2 = HipBackend(0)
+    print(f"alternative paths {env}", flush=True)
+    for dtype in ALL:
+        for m in (1, 2, 11):
+            n, k = 130, 2048
+            w, x = random_weight(dtype, n, k, seed=dtype + m), random_activations(m, k, seed=m)
+            want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+            got = gpu_matmul(hip2, torch, w, x, dtype, m, n, k)
+            check_close(got, want, f"env={env} dtype={dtype} m={m}")
+
+
 # ------------------------------------------------------------------- errors
 def test_unsupported_formats_are_errors(hip, torch):
     from gllm_amd.backend import OtherError, Unimplemented

@@ -90,7 +90,7 @@ def test_bf16_operand_variant(oracle):
 
 
 def test_baseline_config1_shape_runs_on_the_cpu_path(oracle):
-    # BASELINE config 0: Q4_K M=1 K=4096 N=4096, the reference's CPU-runnable case
+    # Q4_K M=1 K=4096 N=4096: the smallest baseline configuration, the one the reference runs on its CPU path
     n = k = 4096
     w, x = random_weight(Q4_K, n, k, seed=0), random_activations(1, k, seed=0)
     assert w.size == 9_437_184
