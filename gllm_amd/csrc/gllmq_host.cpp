@@ -167,7 +167,9 @@ struct gllmq_ctx {
     hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
     bool gemv_f32 = false;                      // GLLMQ_GEMV_F32=1 selects the f32 flavour
     hipFunction_t mm8_q4k[3][3] = {};           // int8 matrix-core kernels [pairs 1,2,4][early steps 1,2,4]
+    hipFunction_t mm8_q4k_areg[2][3][2] = {};   // same with register-resident activation operands [pairs 1,2][early][passes per tile - 1]
     bool use_mm8 = true;                        // GLLMQ_MM8=0 falls back to the GEMV kernels
+    bool mm8_areg = true;                       // GLLMQ_MM8_AREG=0 keeps the activation operands in LDS
     hipFunction_t stream_read = nullptr;
     hipFunction_t mmf_q4k[2][2] = {};           // f16 matrix-core GEMM [32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
@@ -368,7 +370,9 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
         if (const char *v = getenv("GLLMQ_MM8_GRID")) grid = std::min<uint32_t>(P.tiles, std::max(1, atoi(v)));
         P.grid = grid;
-        int rc = launch(ctx, ctx->mm8_q4k[pi][ei], grid, 512, lds, stream, &P, sizeof P);
+        hipFunction_t fn = ctx->mm8_q4k[pi][ei];
+        if (pi <= 1 && ppt <= 2 && ctx->mm8_areg) fn = ctx->mm8_q4k_areg[pi][ei][ppt - 1];
+        int rc = launch(ctx, fn, grid, 512, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }
     return GLLMQ_OK;
@@ -562,8 +566,13 @@ int gllmq_init(gllmq_ctx **out, int device)
             { 0, 0, "gq_mm8_q4k_p1_e1" }, { 0, 1, "gq_mm8_q4k_p1_e2" }, { 0, 2, "gq_mm8_q4k_p1_e4" },
             { 1, 1, "gq_mm8_q4k_p2_e2" }, { 1, 2, "gq_mm8_q4k_p2_e4" }, { 2, 2, "gq_mm8_q4k_p4_e4" },
         };
-        for (const auto &k : kMm8)
+        for (const auto &k : kMm8) {
             if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_q4k[k.pi][k.ei], k.name);
+            for (int a = 1; a <= 2 && k.pi <= 1 && rc == GLLMQ_OK; ++a) {
+                snprintf(name, sizeof name, "%s_a%d", k.name, a);
+                rc = get_function(ctx, &ctx->mm8_q4k_areg[k.pi][k.ei][a - 1], name);
+            }
+        }
     }
     if (rc != GLLMQ_OK) {
         fprintf(stderr, "gllmq_init: %s\n", ctx->err.c_str());
@@ -575,6 +584,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (const char *v = getenv("GLLMQ_GEMV_F32")) ctx->gemv_f32 = (v[0] == '1');
     if (const char *v = getenv("GLLMQ_MM8")) ctx->use_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MMF")) ctx->use_mmf = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_MM8_AREG")) ctx->mm8_areg = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_GEMV_WAVES")) {
         long w = strtol(v, nullptr, 10);
         if (w >= 4 && w <= 65536) ctx->gemv_waves = static_cast<uint32_t>(w);
