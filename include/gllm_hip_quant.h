@@ -3,6 +3,8 @@
  * behind a C ABI.  Every entry point takes plain pointers and sizes; device pointers
  * are HIP device addresses, `stream` is a hipStream_t passed as void* (NULL = the null
  * stream).  All calls are asynchronous on `stream` unless the name ends in `_host`.
+ * The context's device must be the calling thread's current HIP device, and `stream` a
+ * stream of that device.
  *
  * Reference interfaces each entry point stands in for (paths inside putao520/gllm):
  *   Backend::quantized_matmul  src/compat/mod.rs:233-246, CPU impl src/compat/cpu_backend.rs:991-1049

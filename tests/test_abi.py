@@ -54,3 +54,14 @@ def test_backend_refuses_to_run_without_a_gpu():
         pytest.skip("a GPU is present")
     with pytest.raises(backend.HipError):
         backend.HipBackend()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; any other --gpus value exits with a message, before touching a GPU."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, timeout=60)
+    assert r.returncode == 2
+    assert b"one GPU" in r.stderr
+    assert r.stdout.strip() == b""
