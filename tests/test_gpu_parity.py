@@ -254,6 +254,72 @@ def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
             check_close(got, want, f"env={env} dtype={dtype} m={m}")
 
 
+def test_empty_shapes_are_no_ops(hip, torch):
+    print("empty shapes", flush=True)
+    w = torch.zeros(144 * 16, dtype=torch.uint8, device="cuda")
+    x = torch.zeros(4096, dtype=torch.float32, device="cuda")
+    y = torch.full((8,), 7.0, dtype=torch.float32, device="cuda")
+    hip.quantized_matmul(w, x, y, Q4_K, 0, 1, 4096)  # m = 0
+    hip.quantized_matmul(w, x, y, Q4_K, 1, 0, 4096)  # n = 0
+    out = torch.full((8,), 7.0, dtype=torch.float32, device="cuda")
+    hip.dequantize(w[:100], out, Q4_K)               # less than one block in
+    hip.dequantize(w, out[:100], Q4_K)               # room for less than one block out
+    torch.cuda.synchronize()
+    assert torch.all(y == 7.0) and torch.all(out == 7.0)
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_rows_longer_than_one_launch_covers(hip, torch, oracle, dtype):
+    # K = 20480: the GEMV kernels take 16384 elements per launch and accumulate the rest
+    n, k = 67, 20480
+    print(f"long rows dtype={dtype}", flush=True)
+    for m in (1, 2, 3):
+        w, x = random_weight(dtype, n, k, seed=77 + m), random_activations(m, k, seed=78)
+        want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+        got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+        check_close(got, want, f"dtype={dtype} m={m} k={k}")
+
+
+def test_vocabulary_sized_output(hip, torch, oracle):
+    # lm_head shape: Q6_K, 151936 rows over 4096 (the largest matvec of a decode step)
+    n, k = 151936, 4096
+    print("lm_head 151936x4096 Q6_K", flush=True)
+    w, x = random_weight(Q6_K, n, k, seed=5), random_activations(1, k, seed=6)
+    want = oracle.quantized_matmul(w, x, Q6_K, 1, n, k, acc=oracle.ACC_F64, threads=16)
+    got = gpu_matmul(hip, torch, w, x, Q6_K, 1, n, k)
+    check_close(got, want, "lm_head")
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_activations_that_are_only_4_byte_aligned(hip, torch, oracle, dtype):
+    n, k, m = 45, 1024, 2
+    print(f"unaligned activations dtype={dtype}", flush=True)
+    w, x = random_weight(dtype, n, k, seed=31), random_activations(m, k, seed=32)
+    want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64)
+    wd = hip.upload_weights(w)
+    buf = torch.zeros(m * k + 1, dtype=torch.float32, device="cuda")
+    buf[1:] = torch.from_numpy(x.reshape(-1)).cuda()
+    yd = torch.zeros(m * n + 1, dtype=torch.float32, device="cuda")
+    hip.quantized_matmul(wd, buf[1:], yd[1:], dtype, m, n, k)
+    torch.cuda.synchronize()
+    check_close(yd[1:].cpu().numpy().reshape(m, n), want, f"unaligned dtype={dtype}")
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_non_finite_activations_give_non_finite_outputs(hip, torch, oracle, dtype):
+    """An Inf or NaN activation makes every output that depends on it non-finite (the exact
+    non-finite value is not pinned: the oracle may say Inf where the GPU says NaN)."""
+    n, k = 40, 1024
+    print(f"non-finite dtype={dtype}", flush=True)
+    w = random_weight(dtype, n, k, seed=41)
+    for bad in (np.inf, -np.inf, np.nan):
+        x = random_activations(1, k, seed=42)
+        x[0, 300] = bad
+        want = oracle.quantized_matmul(w, x, dtype, 1, n, k, acc=oracle.ACC_F64)
+        got = gpu_matmul(hip, torch, w, x, dtype, 1, n, k)
+        assert not np.isfinite(got[~np.isfinite(want)]).any()
+
+
 # ------------------------------------------------------------------- errors
 def test_unsupported_formats_are_errors(hip, torch):
     from gllm_amd.backend import OtherError, Unimplemented
