@@ -123,7 +123,7 @@ struct MoePlanParams {
     uint32_t *pair_pos;
     MoeJob *jobs;
     uint32_t *counters;
-    uint32_t tokens, top_k, experts, pairs;
+    uint32_t tokens, top_k, experts, pairs, fast;
 };
 struct MoeGemvParams {
     GemvParams g;
@@ -733,9 +733,10 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
     float *o = reinterpret_cast<float *>(ws + o_o);
 
     {
+        const uint32_t fast = pairs <= 4096 ? 1u : 0u; // quadratic in the pairs, but without serial LDS walks
         MoePlanParams P{ route_expert, route_len, pair_src, pair_pos, jobs, counters, static_cast<uint32_t>(tokens),
-                         static_cast<uint32_t>(top_k), static_cast<uint32_t>(experts), static_cast<uint32_t>(pairs) };
-        const uint32_t lds = static_cast<uint32_t>((pairs + 3 * experts + 4) * 4);
+                         static_cast<uint32_t>(top_k), static_cast<uint32_t>(experts), static_cast<uint32_t>(pairs), fast };
+        const uint32_t lds = static_cast<uint32_t>((pairs + 3 * experts + 4 + (fast ? 2 * pairs : 0)) * 4);
         int rc = launch(ctx, ctx->moe_plan, 1, 256, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }

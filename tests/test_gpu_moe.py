@@ -148,6 +148,20 @@ def test_moe_baseline_shape_reduced_expert_count(hip, torch, oracle):
     check_close(got2, want2, "moe baseline shape, default capacity")
 
 
+def test_moe_many_pairs(hip, torch, oracle):
+    """More (token, expert) pairs than the plan kernel's per-pair placement takes (4096): the
+    per-expert walk is used; experts get hundreds of tokens each."""
+    print("moe many pairs", flush=True)
+    experts, tokens, top_k, hidden, ffn = 16, 640, 8, 256, 256
+    gu, dn = expert_weights(Q4_K, Q6_K, experts, hidden, ffn, seed=80)
+    x = random_activations(tokens, hidden, seed=81)
+    r = oracle.route(random_gate_logits(tokens, experts, seed=82), top_k, capacity_factor=float(experts))
+    assert int(r["len"].sum()) == tokens * top_k > 4096
+    want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=16)
+    got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
+    check_close(got, want, "moe many pairs")
+
+
 def test_moe_error_behaviour(hip, torch):
     from gllm_amd.backend import Unimplemented
     print("moe errors", flush=True)
