@@ -78,6 +78,7 @@ struct Mm8Params {
     const float *x;
     float *y;
     uint32_t n, k, groups, row_bytes, m, ldx, ldy, tiles, grid, act_bf16;
+    const uint32_t *xrows;
 };
 
 // Mirror of gq::MmfParams in mmf.hip.inc.
@@ -116,12 +117,16 @@ uint32_t mmf_lds_bytes(uint32_t mt) { return mmf_image_bytes(mt) + 8u * 5120u; }
 struct MoeJob {
     uint32_t expert, p0, m, t0, t1;
 };
+struct MoeJob8 {
+    uint32_t expert, p0, m, pad, tok[8];
+};
 struct MoePlanParams {
     const uint32_t *route_expert;
     const uint32_t *route_len;
     uint32_t *pair_src;
     uint32_t *pair_pos;
     MoeJob *jobs;
+    MoeJob8 *jobs8;
     uint32_t *counters;
     uint32_t tokens, top_k, experts, pairs, fast;
 };
@@ -131,6 +136,13 @@ struct MoeGemvParams {
     const uint32_t *counters;
     uint64_t expert_stride;
     uint32_t wgs_per_job, x_by_token, x_stride, y_stride;
+};
+struct MoeMm8Params {
+    Mm8Params g;
+    const MoeJob8 *jobs;
+    const uint32_t *counters;
+    uint64_t expert_stride;
+    uint32_t slices, y_stride;
 };
 struct MoeActParams {
     const float *gu;
@@ -170,6 +182,7 @@ struct gllmq_ctx {
     hipFunction_t mm8_q4k_areg[2][3][2] = {};   // same with register-resident activation operands [pairs 1,2][early][passes per tile - 1]
     bool use_mm8 = true;                        // GLLMQ_MM8=0 falls back to the GEMV kernels
     bool mm8_areg = true;                       // GLLMQ_MM8_AREG=0 keeps the activation operands in LDS
+    bool moe_mm8 = true;                        // GLLMQ_MOE_MM8=0 keeps the MoE gate/up rows on the GEMV kernels
     hipFunction_t stream_read = nullptr;
     hipFunction_t mmf_q4k[2][2] = {};           // f16 matrix-core GEMM [32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
@@ -181,6 +194,8 @@ struct gllmq_ctx {
     size_t mmf_partial_bytes = 0;
     hipFunction_t moe_plan = nullptr, moe_act = nullptr, moe_combine = nullptr;
     hipFunction_t moe_gemv[kNumFormats] = {};
+    hipFunction_t moe_mm8_q4k[2] = {};          // grouped int8 matrix-core kernel [passes per tile - 1]
+    uint32_t *identity_rows = nullptr;          // device: 0..7, the activation rows of an ungathered matmul
     // Device workspace of the MoE path (pair tables, jobs, intermediate activations).  It
     // grows on demand and is shared by all calls on this context: calls that use it must
     // not overlap in time.
@@ -363,6 +378,7 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         P.ldy = static_cast<uint32_t>(n);
         P.tiles = (P.n + 31u) / 32u;
         P.act_bf16 = act_bf16 ? 1u : 0u;
+        P.xrows = ctx->identity_rows;
         // preparation steps per wave: two 256-element blocks per step
         const uint32_t ppt = (groups + 7u) / 8u, steps = ((ppt + 1u) / 2u) * mm;
         int ei = steps <= 1 ? 0 : (steps <= 2 ? 1 : 2);
@@ -561,6 +577,14 @@ int gllmq_init(gllmq_ctx **out, int device)
         snprintf(name, sizeof name, "gq_moe_gemv_%s", kFormats[i].tag);
         rc = get_function(ctx, &ctx->moe_gemv[i], name);
     }
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_q4k[0], "gq_moe_mm8_q4k_a1");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_q4k[1], "gq_moe_mm8_q4k_a2");
+    if (rc == GLLMQ_OK) {
+        static const uint32_t kRows[8] = { 0, 1, 2, 3, 4, 5, 6, 7 };
+        hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->identity_rows), sizeof kRows);
+        if (he == hipSuccess) he = hipMemcpy(ctx->identity_rows, kRows, sizeof kRows, hipMemcpyHostToDevice);
+        if (he != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "row table: %s", hipGetErrorString(he));
+    }
     {
         static const struct { int pi, ei; const char *name; } kMm8[] = {
             { 0, 0, "gq_mm8_q4k_p1_e1" }, { 0, 1, "gq_mm8_q4k_p1_e2" }, { 0, 2, "gq_mm8_q4k_p1_e4" },
@@ -585,6 +609,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (const char *v = getenv("GLLMQ_MM8")) ctx->use_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MMF")) ctx->use_mmf = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MM8_AREG")) ctx->mm8_areg = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_MOE_MM8")) ctx->moe_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_GEMV_WAVES")) {
         long w = strtol(v, nullptr, 10);
         if (w >= 4 && w <= 65536) ctx->gemv_waves = static_cast<uint32_t>(w);
@@ -597,6 +622,7 @@ void gllmq_destroy(gllmq_ctx *ctx)
 {
     if (!ctx) return;
     if (ctx->workspace) (void)hipFree(ctx->workspace);
+    if (ctx->identity_rows) (void)hipFree(ctx->identity_rows);
     if (ctx->mmf_partial) (void)hipFree(ctx->mmf_partial);
     if (ctx->module) (void)hipModuleUnload(ctx->module);
     delete ctx;
@@ -707,7 +733,8 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
     const size_t o_src = off; off = up256(off + pairs * 4);
     const size_t o_pos = off; off = up256(off + pairs * 4);
     const size_t o_jobs = off; off = up256(off + pairs * sizeof(MoeJob));
-    const size_t o_cnt = off; off = up256(off + 2 * 4);
+    const size_t o_jobs8 = off; off = up256(off + pairs * sizeof(MoeJob8));
+    const size_t o_cnt = off; off = up256(off + 4 * 4);
     const size_t o_gu = off; off = up256(off + pairs * 2 * ffn * 4);
     const size_t o_h = off; off = up256(off + pairs * ffn * 4);
     const size_t o_o = off; off = up256(off + pairs * hidden * 4);
@@ -727,16 +754,17 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
     uint32_t *pair_src = reinterpret_cast<uint32_t *>(ws + o_src);
     uint32_t *pair_pos = reinterpret_cast<uint32_t *>(ws + o_pos);
     MoeJob *jobs = reinterpret_cast<MoeJob *>(ws + o_jobs);
+    MoeJob8 *jobs8 = reinterpret_cast<MoeJob8 *>(ws + o_jobs8);
     uint32_t *counters = reinterpret_cast<uint32_t *>(ws + o_cnt);
     float *gu = reinterpret_cast<float *>(ws + o_gu);
     float *h = reinterpret_cast<float *>(ws + o_h);
     float *o = reinterpret_cast<float *>(ws + o_o);
 
+    const uint32_t fast = pairs <= 4096 ? 1u : 0u; // per-pair placement: quadratic in the pairs, but without serial LDS walks
     {
-        const uint32_t fast = pairs <= 4096 ? 1u : 0u; // quadratic in the pairs, but without serial LDS walks
-        MoePlanParams P{ route_expert, route_len, pair_src, pair_pos, jobs, counters, static_cast<uint32_t>(tokens),
+        MoePlanParams P{ route_expert, route_len, pair_src, pair_pos, jobs, jobs8, counters, static_cast<uint32_t>(tokens),
                          static_cast<uint32_t>(top_k), static_cast<uint32_t>(experts), static_cast<uint32_t>(pairs), fast };
-        const uint32_t lds = static_cast<uint32_t>((pairs + 3 * experts + 4 + (fast ? 2 * pairs : 0)) * 4);
+        const uint32_t lds = static_cast<uint32_t>((pairs + 4 * experts + 4 + (fast ? 2 * pairs : 0)) * 4);
         int rc = launch(ctx, ctx->moe_plan, 1, 256, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }
@@ -766,7 +794,39 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         return launch(ctx, ctx->moe_gemv[format_index(f.dtype)], static_cast<uint32_t>(grid), L.threads, L.lds, stream,
                       &Q, sizeof Q);
     };
-    int rc = grouped(*fg, gate_up, rb_gu, static_cast<uint32_t>(2 * ffn), static_cast<uint32_t>(hidden), x, true, gu);
+    // gate/up: Q4_K with rows of at most 16 blocks goes to the int8 matrix cores, every token
+    // of an expert (up to eight per job) in one pass over its weights
+    int rc = GLLMQ_OK;
+    const uint32_t groups_gu = static_cast<uint32_t>((hidden + 255) / 256);
+    const bool gu_mm8 = fast && ctx->use_mm8 && ctx->moe_mm8 && fg->dtype == T_Q4_K && groups_gu <= 16 && hidden % 8 == 0 &&
+                        mm8_lds_bytes(groups_gu, 8, 4) <= 160u * 1024u;
+    if (gu_mm8) {
+        MoeMm8Params Q{};
+        Q.g.w = static_cast<const uint8_t *>(gate_up);
+        Q.g.x = x;
+        Q.g.y = gu;
+        Q.g.n = static_cast<uint32_t>(2 * ffn);
+        Q.g.k = static_cast<uint32_t>(hidden);
+        Q.g.groups = groups_gu;
+        Q.g.row_bytes = static_cast<uint32_t>(rb_gu);
+        Q.g.ldx = static_cast<uint32_t>(hidden);
+        Q.g.tiles = (Q.g.n + 31u) / 32u;
+        Q.jobs = jobs8;
+        Q.counters = counters;
+        Q.expert_stride = static_cast<uint64_t>(2 * ffn) * rb_gu;
+        Q.y_stride = static_cast<uint32_t>(2 * ffn);
+        // upper bound of the jobs: one per expert hit, plus one per eight further pairs
+        const uint64_t max_jobs = std::min<uint64_t>(pairs, experts + pairs / 8);
+        uint32_t slices = std::max<uint32_t>(1u, (3u * static_cast<uint32_t>(ctx->num_cus)) / (2u * static_cast<uint32_t>(std::min<uint64_t>(pairs, experts))));
+        if (const char *v = getenv("GLLMQ_MOE_SLICES")) slices = static_cast<uint32_t>(std::max(1, atoi(v)));
+        slices = std::min(slices, Q.g.tiles);
+        Q.slices = slices;
+        const uint32_t ppt = (groups_gu + 7u) / 8u;
+        rc = launch(ctx, ctx->moe_mm8_q4k[ppt - 1], static_cast<uint32_t>(max_jobs * slices), 512,
+                    mm8_lds_bytes(groups_gu, 8, 4), stream, &Q, sizeof Q);
+    } else {
+        rc = grouped(*fg, gate_up, rb_gu, static_cast<uint32_t>(2 * ffn), static_cast<uint32_t>(hidden), x, true, gu);
+    }
     if (rc != GLLMQ_OK) return rc;
     {
         MoeActParams P{ gu, h, counters, static_cast<uint32_t>(ffn), relu_gate ? 1u : 0u };

@@ -120,7 +120,10 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
  * out[t] = sum_i weight[t][i] * down_e( silu(gate_e x_t) * (up_e x_t) ), e = expert[t][i],
  * summed in route order i = 0 .. route_len[t]-1 (src/moe/routing.rs:307-327); a token with
  * no route gets zeros.  Only routed (token, expert) pairs are computed (the reference graph
- * runs every expert on every token and masks, build_graph.inc.rs:2076-2123).
+ * runs every expert on every token and masks, build_graph.inc.rs:2076-2123).  Q4_K gate/up
+ * rows of at most 4096 elements run on the int8 matrix cores, all tokens of an expert (eight
+ * per pass) against one read of its weights; other formats and the down rows run the
+ * integer-dot GEMV, two tokens per pass.
  * gate_up_dev: per expert 2*ffn rows over `hidden` (gate rows, then up rows);
  * down_dev: per expert `hidden` rows over `ffn`.  route_* are [tokens x top_k] device
  * arrays, route_len[t] entries valid per token; entries past route_len[t] are ignored and
