@@ -110,8 +110,12 @@ uint32_t mmf_image_bytes(uint32_t mt)
     return (raw + 8191u) / 8192u * 8192u; // whole rounds of 512 threads x 16 bytes
 }
 
-// gq::MmfLds<MT>::total: image, one 5 KiB weight stage per wave.
-uint32_t mmf_lds_bytes(uint32_t mt) { return mmf_image_bytes(mt) + 8u * 5120u; }
+// gq::MmfLds<MT>::total: image and one 5 KiB weight stage per wave, twice where that fits.
+uint32_t mmf_lds_bytes(uint32_t mt)
+{
+    const uint32_t once = mmf_image_bytes(mt) + 8u * 5120u;
+    return 2u * once <= 160u * 1024u ? 2u * once : once; // two sets that take turns, where they fit
+}
 
 // Mirrors of the structs in moe.hip.inc.
 struct MoeJob {
@@ -413,9 +417,10 @@ int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     ksplit = (groups + bps - 1) / bps; // every workgroup gets at least one block
     std::lock_guard<std::mutex> guard(ctx->workspace_mutex);
     GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
-    const size_t rows_per_pass = 64;
+    size_t rows_per_pass = 64;
+    if (const char *v = getenv("GLLMQ_MMF_ROWS")) rows_per_pass = atoi(v) <= 32 ? 32 : 64;
     // scratch: the activation images of one pass, then the partial sums
-    const size_t img_bytes = static_cast<size_t>(groups) * mmf_image_bytes(m <= 32 ? 1u : 2u);
+    const size_t img_bytes = static_cast<size_t>(groups) * mmf_image_bytes(std::min(m, rows_per_pass) <= 32 ? 1u : 2u);
     const size_t need = img_bytes + (ksplit > 1 ? static_cast<size_t>(ksplit) * std::min(m, rows_per_pass) * n * 4 : 0);
     if (ctx->mmf_partial_bytes < need) {
         if (ctx->mmf_partial) {
@@ -448,7 +453,7 @@ int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         P.blocks_per_split = bps;
         P.act_bf16 = act_bf16 ? 1u : 0u;
         MmfPrepParams Q{ P.x, P.ximg, mm, P.k, P.ldx, P.act_bf16 };
-        int rc = launch2d(ctx, ctx->mmf_prep[mt - 1], groups, 4, 64, 0, stream, &Q, sizeof Q);
+        int rc = launch2d(ctx, ctx->mmf_prep[mt - 1], groups, 16, 64, 0, stream, &Q, sizeof Q);
         if (rc != GLLMQ_OK) return rc;
         rc = launch(ctx, ctx->mmf_q4k[mt - 1][act_bf16 ? 1 : 0], row_tiles * ksplit, 512, mmf_lds_bytes(mt), stream,
                     &P, sizeof P);
