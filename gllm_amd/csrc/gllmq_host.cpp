@@ -163,14 +163,15 @@ struct MoeCombineParams {
     uint32_t tokens, top_k, hidden;
 };
 
-// Same carve-up as gq::mm8_lds_layout: bytes of LDS the int8 matrix-core kernel needs.
-uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs)
+// Same carve-up as gq::mm8_lds_layout: bytes of LDS the int8 matrix-core kernels need.
+// q6k: 16 sub-block sums per block and a 7.5 KiB weight stage per wave instead of 8 and 5 KiB.
+uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs, bool q6k = false)
 {
     const uint32_t plane_stride = groups * 256u + 16u;
     const uint32_t sums = 3u * m * plane_stride;
-    const uint32_t scales = sums + m * groups * 8u * 4u;
+    const uint32_t scales = sums + m * groups * (q6k ? 16u : 8u) * 4u;
     const uint32_t red = (scales + m * groups * 4u + 15u) & ~15u;
-    return red + 2u * 8u * pairs * 64u * 4u + 8u * 5120u; // + one 5 KiB weight stage per wave
+    return red + 2u * 8u * pairs * 64u * 4u + 8u * (q6k ? 7680u : 5120u);
 }
 
 } // namespace
@@ -182,10 +183,15 @@ struct gllmq_ctx {
     hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1], f32 multiply-add flavour
     hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
     bool gemv_f32 = false;                      // GLLMQ_GEMV_F32=1 selects the f32 flavour
-    hipFunction_t mm8_q4k[3][3] = {};           // int8 matrix-core kernels [pairs 1,2,4][early steps 1,2,4]
-    hipFunction_t mm8_q4k_areg[2][3][2] = {};   // same with register-resident activation operands [pairs 1,2][early][passes per tile - 1]
+    // int8 matrix-core kernels [0 = Q4_K, 1 = Q6_K][pairs 1,2,4][early steps 1,2,4], and the same
+    // with register-resident activation operands [..][pairs 1,2][early][passes per tile - 1]
+    hipFunction_t mm8[2][3][3] = {};
+    hipFunction_t mm8_areg[2][2][3][2] = {};
     bool use_mm8 = true;                        // GLLMQ_MM8=0 falls back to the GEMV kernels
-    bool mm8_areg = true;                       // GLLMQ_MM8_AREG=0 keeps the activation operands in LDS
+    bool mm8_areg_on = true;                    // GLLMQ_MM8_AREG=0 keeps the activation operands in LDS
+    // Fewest activation rows that send Q6_K to the matrix-core kernel: up to two rows the GEMV
+    // kernels are as fast or faster.  GLLMQ_MM8_Q6K_MIN_M overrides (1 = always, 0 = never).
+    uint32_t mm8_q6k_min_m = 3;
     bool moe_mm8 = true;                        // GLLMQ_MOE_MM8=0 keeps the MoE gate/up rows on the GEMV kernels
     hipFunction_t stream_read = nullptr;
     hipFunction_t mmf_q4k[2][2] = {};           // f16 matrix-core GEMM [32-row activation tiles - 1][bf16 mode]
@@ -348,27 +354,29 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
     return -1; // go on
 }
 
-// Q4_K on the int8 matrix cores, activation rows in passes of at most 8 (a pass keeps its
-// rows' digit planes in LDS and reads the weights once).  Returns -1 when the shape does
+// Q4_K and Q6_K on the int8 matrix cores, activation rows in passes of at most 8 (a pass keeps
+// its rows' digit planes in LDS and reads the weights once).  Returns -1 when the shape does
 // not fit the kernel (LDS for the prepared activations, alignment), so that the caller
 // takes the GEMV kernels.
 int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
             size_t k, bool act_bf16, void *stream)
 {
-    if (!ctx->use_mm8 || f.dtype != T_Q4_K) return -1;
+    if (!ctx->use_mm8 || (f.dtype != T_Q4_K && f.dtype != T_Q6_K)) return -1;
+    const bool q6k = f.dtype == T_Q6_K;
+    if (q6k && (ctx->mm8_q6k_min_m == 0 || m < ctx->mm8_q6k_min_m)) return -1;
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
     // Rows per pass: as many as the prepared activations leave room for in the 160 KiB of LDS.
     auto pairs_for = [](uint32_t rows) { return rows <= 2 ? 1u : (rows <= 4 ? 2u : 4u); };
     uint32_t rows_per_pass = static_cast<uint32_t>(std::min<size_t>(m, 8));
-    while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass)) > 160u * 1024u)
+    while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass), q6k) > 160u * 1024u)
         --rows_per_pass;
     if (rows_per_pass == 0) return -1;
     for (size_t m0 = 0; m0 < m; m0 += rows_per_pass) {
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(rows_per_pass, m - m0));
         const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
         const uint32_t pairs = 1u << pi;
-        const uint32_t lds = mm8_lds_bytes(groups, mm, pairs);
+        const uint32_t lds = mm8_lds_bytes(groups, mm, pairs, q6k);
         Mm8Params P{};
         P.w = w;
         P.x = x + m0 * k;
@@ -386,20 +394,18 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         // preparation steps per wave: two 256-element blocks per step
         const uint32_t ppt = (groups + 7u) / 8u, steps = ((ppt + 1u) / 2u) * mm;
         int ei = steps <= 1 ? 0 : (steps <= 2 ? 1 : 2);
-        while (ei < 2 && !ctx->mm8_q4k[pi][ei]) ++ei; // not every (pairs, early) pair is built
+        while (ei < 2 && !ctx->mm8[q6k][pi][ei]) ++ei; // not every (pairs, early) pair is built
         uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
         if (const char *v = getenv("GLLMQ_MM8_GRID")) grid = std::min<uint32_t>(P.tiles, std::max(1, atoi(v)));
         P.grid = grid;
-        hipFunction_t fn = ctx->mm8_q4k[pi][ei];
-        if (pi <= 1 && ppt <= 2 && ctx->mm8_areg) fn = ctx->mm8_q4k_areg[pi][ei][ppt - 1];
+        hipFunction_t fn = ctx->mm8[q6k][pi][ei];
+        if (pi <= 1 && ppt <= 2 && ctx->mm8_areg_on) fn = ctx->mm8_areg[q6k][pi][ei][ppt - 1];
         int rc = launch(ctx, fn, grid, 512, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }
     return GLLMQ_OK;
 }
 
-// Q4_K with more than 8 activation rows: f16 matrix-core GEMM, 64 rows per pass, weights read
-// once per pass.  Returns -1 when the shape does not fit (alignment), like run_mm8.
 constexpr uint32_t kMmfMaxRowTiles = 16384;
 
 int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
@@ -591,17 +597,19 @@ int gllmq_init(gllmq_ctx **out, int device)
         if (he != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "row table: %s", hipGetErrorString(he));
     }
     {
-        static const struct { int pi, ei; const char *name; } kMm8[] = {
-            { 0, 0, "gq_mm8_q4k_p1_e1" }, { 0, 1, "gq_mm8_q4k_p1_e2" }, { 0, 2, "gq_mm8_q4k_p1_e4" },
-            { 1, 1, "gq_mm8_q4k_p2_e2" }, { 1, 2, "gq_mm8_q4k_p2_e4" }, { 2, 2, "gq_mm8_q4k_p4_e4" },
+        static const struct { int pi, ei; const char *tag; } kMm8[] = {
+            { 0, 0, "p1_e1" }, { 0, 1, "p1_e2" }, { 0, 2, "p1_e4" }, { 1, 1, "p2_e2" }, { 1, 2, "p2_e4" }, { 2, 2, "p4_e4" },
         };
-        for (const auto &k : kMm8) {
-            if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_q4k[k.pi][k.ei], k.name);
-            for (int a = 1; a <= 2 && k.pi <= 1 && rc == GLLMQ_OK; ++a) {
-                snprintf(name, sizeof name, "%s_a%d", k.name, a);
-                rc = get_function(ctx, &ctx->mm8_q4k_areg[k.pi][k.ei][a - 1], name);
+        static const char *const kMm8Format[2] = { "q4k", "q6k" };
+        for (int q = 0; q < 2; ++q)
+            for (const auto &k : kMm8) {
+                snprintf(name, sizeof name, "gq_mm8_%s_%s", kMm8Format[q], k.tag);
+                if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8[q][k.pi][k.ei], name);
+                for (int a = 1; a <= 2 && k.pi <= 1 && rc == GLLMQ_OK; ++a) {
+                    snprintf(name, sizeof name, "gq_mm8_%s_%s_a%d", kMm8Format[q], k.tag, a);
+                    rc = get_function(ctx, &ctx->mm8_areg[q][k.pi][k.ei][a - 1], name);
+                }
             }
-        }
     }
     if (rc != GLLMQ_OK) {
         fprintf(stderr, "gllmq_init: %s\n", ctx->err.c_str());
@@ -613,7 +621,8 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (const char *v = getenv("GLLMQ_GEMV_F32")) ctx->gemv_f32 = (v[0] == '1');
     if (const char *v = getenv("GLLMQ_MM8")) ctx->use_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MMF")) ctx->use_mmf = (v[0] != '0');
-    if (const char *v = getenv("GLLMQ_MM8_AREG")) ctx->mm8_areg = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_MM8_AREG")) ctx->mm8_areg_on = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_MM8_Q6K_MIN_M")) ctx->mm8_q6k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
     if (const char *v = getenv("GLLMQ_MOE_MM8")) ctx->moe_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_GEMV_WAVES")) {
         long w = strtol(v, nullptr, 10);

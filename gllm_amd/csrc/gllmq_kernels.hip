@@ -10,6 +10,7 @@
 #include "gemv.hip.inc"
 #include "gemv_i8.hip.inc"
 #include "mm8.hip.inc"
+#include "mm8_q6k.hip.inc"
 #include "mmf.hip.inc"
 #include "moe.hip.inc"
 #include "probe.hip.inc"

@@ -118,6 +118,18 @@ def test_small_m_matches_oracle(hip, torch, oracle, dtype, m):
     check_close(got, want, f"dtype={dtype} m={m}")
 
 
+@pytest.mark.parametrize("dtype", [Q4_K, Q6_K])
+@pytest.mark.parametrize("m", [3, 8])
+def test_small_m_down_projection_shape(hip, torch, oracle, dtype, m):
+    # K = 14336: seven passes per tile on the matrix-core kernels, activation operands read from LDS
+    n, k = 70, 14336
+    print(f"small-m long rows dtype={dtype} m={m}", flush=True)
+    w, x = random_weight(dtype, n, k, seed=40 + m), random_activations(m, k, seed=41)
+    want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+    got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+    check_close(got, want, f"dtype={dtype} m={m} k={k}")
+
+
 @pytest.mark.parametrize("dtype,k", [(Q4_K, 300), (Q5_K, 511), (Q6_K, 257), (Q8_0, 40), (Q8_0, 4000), (Q4_K, 4100)])
 def test_row_padding(hip, torch, oracle, dtype, k):
     print(f"padding dtype={dtype} k={k}", flush=True)
@@ -236,17 +248,19 @@ def test_bf16_activation_mode(hip, torch, oracle, dtype, m):
 
 
 @pytest.mark.parametrize("env", [{"GLLMQ_MM8": "0", "GLLMQ_MMF": "0"}, {"GLLMQ_MMF": "0"},
-                                 {"GLLMQ_GEMV_F32": "1", "GLLMQ_MM8": "0", "GLLMQ_MMF": "0"}])
+                                 {"GLLMQ_GEMV_F32": "1", "GLLMQ_MM8": "0", "GLLMQ_MMF": "0"},
+                                 {"GLLMQ_MM8_Q6K_MIN_M": "1"}, {"GLLMQ_MM8_Q6K_MIN_M": "0"}])
 def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
     """The kernels the default dispatch does not pick: integer-dot GEMV for Q4_K, 8-row passes
-    for more than 8 rows, and the f32 multiply-add flavour; selected per context at init."""
+    for more than 8 rows, the f32 multiply-add flavour, Q6_K on the matrix cores for one and two
+    rows and on the GEMV kernels for more; selected per context at init."""
     from gllm_amd.backend import HipBackend
     for k_, v_ in env.items():
         monkeypatch.setenv(k_, v_)
     hip2 = HipBackend(0)
     print(f"alternative paths {env}", flush=True)
     for dtype in ALL:
-        for m in (1, 2, 11):
+        for m in (1, 2, 5, 11):
             n, k = 130, 2048
             w, x = random_weight(dtype, n, k, seed=dtype + m), random_activations(m, k, seed=m)
             want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
