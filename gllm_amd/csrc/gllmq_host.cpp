@@ -147,6 +147,7 @@ struct MoeMm8Params {
     const uint32_t *counters;
     uint64_t expert_stride;
     uint32_t slices, y_stride;
+    const uint32_t *rows;
 };
 struct MoeActParams {
     const float *gu;
@@ -192,7 +193,9 @@ struct gllmq_ctx {
     // Fewest activation rows that send Q6_K to the matrix-core kernel: up to two rows the GEMV
     // kernels are as fast or faster.  GLLMQ_MM8_Q6K_MIN_M overrides (1 = always, 0 = never).
     uint32_t mm8_q6k_min_m = 3;
-    bool moe_mm8 = true;                        // GLLMQ_MOE_MM8=0 keeps the MoE gate/up rows on the GEMV kernels
+    bool moe_mm8 = true;                        // GLLMQ_MOE_MM8=0 keeps the MoE expert rows on the GEMV kernels
+    bool moe_mm8_q6k = true;                    // GLLMQ_MOE_MM8_Q6K=0 keeps Q6_K expert rows there
+    bool moe_mm8_rows = true;                   // GLLMQ_MOE_MM8_ROWS=0: no wave-per-tile kernel for short Q6_K rows
     hipFunction_t stream_read = nullptr;
     hipFunction_t mmf_q4k[2][2] = {};           // f16 matrix-core GEMM [32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
@@ -204,7 +207,8 @@ struct gllmq_ctx {
     size_t mmf_partial_bytes = 0;
     hipFunction_t moe_plan = nullptr, moe_act = nullptr, moe_combine = nullptr;
     hipFunction_t moe_gemv[kNumFormats] = {};
-    hipFunction_t moe_mm8_q4k[2] = {};          // grouped int8 matrix-core kernel [passes per tile - 1]
+    hipFunction_t moe_mm8_fn[2][2] = {};        // grouped int8 matrix-core kernels [0 = Q4_K, 1 = Q6_K][passes per tile - 1]
+    hipFunction_t moe_mm8_q6k_rows = nullptr;   // Q6_K rows of at most 8 blocks: a wave per 32-row tile
     uint32_t *identity_rows = nullptr;          // device: 0..7, the activation rows of an ungathered matmul
     // Device workspace of the MoE path (pair tables, jobs, intermediate activations).  It
     // grows on demand and is shared by all calls on this context: calls that use it must
@@ -588,8 +592,11 @@ int gllmq_init(gllmq_ctx **out, int device)
         snprintf(name, sizeof name, "gq_moe_gemv_%s", kFormats[i].tag);
         rc = get_function(ctx, &ctx->moe_gemv[i], name);
     }
-    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_q4k[0], "gq_moe_mm8_q4k_a1");
-    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_q4k[1], "gq_moe_mm8_q4k_a2");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[0][0], "gq_moe_mm8_q4k_a1");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[0][1], "gq_moe_mm8_q4k_a2");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[1][0], "gq_moe_mm8_q6k_a1");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[1][1], "gq_moe_mm8_q6k_a2");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_q6k_rows, "gq_moe_mm8_q6k_rows");
     if (rc == GLLMQ_OK) {
         static const uint32_t kRows[8] = { 0, 1, 2, 3, 4, 5, 6, 7 };
         hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->identity_rows), sizeof kRows);
@@ -624,6 +631,8 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (const char *v = getenv("GLLMQ_MM8_AREG")) ctx->mm8_areg_on = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MM8_Q6K_MIN_M")) ctx->mm8_q6k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
     if (const char *v = getenv("GLLMQ_MOE_MM8")) ctx->moe_mm8 = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_MOE_MM8_Q6K")) ctx->moe_mm8_q6k = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_MOE_MM8_ROWS")) ctx->moe_mm8_rows = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_GEMV_WAVES")) {
         long w = strtol(v, nullptr, 10);
         if (w >= 4 && w <= 65536) ctx->gemv_waves = static_cast<uint32_t>(w);
@@ -808,39 +817,56 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         return launch(ctx, ctx->moe_gemv[format_index(f.dtype)], static_cast<uint32_t>(grid), L.threads, L.lds, stream,
                       &Q, sizeof Q);
     };
-    // gate/up: Q4_K with rows of at most 16 blocks goes to the int8 matrix cores, every token
-    // of an expert (up to eight per job) in one pass over its weights
-    int rc = GLLMQ_OK;
-    const uint32_t groups_gu = static_cast<uint32_t>((hidden + 255) / 256);
-    const bool gu_mm8 = fast && ctx->use_mm8 && ctx->moe_mm8 && fg->dtype == T_Q4_K && groups_gu <= 16 && hidden % 8 == 0 &&
-                        mm8_lds_bytes(groups_gu, 8, 4) <= 160u * 1024u;
-    if (gu_mm8) {
+    // Q4_K and Q6_K with rows of at most 16 blocks go to the int8 matrix cores, every token of
+    // an expert (up to eight per job) in one pass over its weights.  `by_token`: the activation
+    // rows are x[token] (gate/up), else rows by sorted position (down).
+    auto grouped_mm8 = [&](const Format &f, const void *wbase, size_t rb, uint32_t n, uint32_t k, const float *xin,
+                           bool by_token, float *yout) -> int {
+        const bool q6k = f.dtype == T_Q6_K;
+        const uint32_t groups = (k + 255u) / 256u;
         MoeMm8Params Q{};
-        Q.g.w = static_cast<const uint8_t *>(gate_up);
-        Q.g.x = x;
-        Q.g.y = gu;
-        Q.g.n = static_cast<uint32_t>(2 * ffn);
-        Q.g.k = static_cast<uint32_t>(hidden);
-        Q.g.groups = groups_gu;
-        Q.g.row_bytes = static_cast<uint32_t>(rb_gu);
-        Q.g.ldx = static_cast<uint32_t>(hidden);
-        Q.g.tiles = (Q.g.n + 31u) / 32u;
+        Q.g.w = static_cast<const uint8_t *>(wbase);
+        Q.g.x = xin;
+        Q.g.y = yout;
+        Q.g.n = n;
+        Q.g.k = k;
+        Q.g.groups = groups;
+        Q.g.row_bytes = static_cast<uint32_t>(rb);
+        Q.g.ldx = k;
+        Q.g.tiles = (n + 31u) / 32u;
         Q.jobs = jobs8;
         Q.counters = counters;
-        Q.expert_stride = static_cast<uint64_t>(2 * ffn) * rb_gu;
-        Q.y_stride = static_cast<uint32_t>(2 * ffn);
+        Q.expert_stride = static_cast<uint64_t>(n) * rb;
+        Q.y_stride = n;
+        Q.rows = by_token ? nullptr : ctx->identity_rows;
         // upper bound of the jobs: one per expert hit, plus one per eight further pairs
         const uint64_t max_jobs = std::min<uint64_t>(pairs, experts + pairs / 8);
         uint32_t slices = std::max<uint32_t>(1u, (3u * static_cast<uint32_t>(ctx->num_cus)) / (2u * static_cast<uint32_t>(std::min<uint64_t>(pairs, experts))));
         if (const char *v = getenv("GLLMQ_MOE_SLICES")) slices = static_cast<uint32_t>(std::max(1, atoi(v)));
-        slices = std::min(slices, Q.g.tiles);
+        const uint32_t ppt = (groups + 7u) / 8u;
+        hipFunction_t fn = ctx->moe_mm8_fn[q6k][ppt - 1];
+        uint32_t units = Q.g.tiles; // what the slices of a job share: tiles, or groups of eight tiles
+        if (q6k && groups <= 8 && ctx->moe_mm8_rows) {
+            fn = ctx->moe_mm8_q6k_rows;
+            units = (Q.g.tiles + 7u) / 8u;
+        }
+        slices = std::min(slices, units);
         Q.slices = slices;
-        const uint32_t ppt = (groups_gu + 7u) / 8u;
-        rc = launch(ctx, ctx->moe_mm8_q4k[ppt - 1], static_cast<uint32_t>(max_jobs * slices), 512,
-                    mm8_lds_bytes(groups_gu, 8, 4), stream, &Q, sizeof Q);
-    } else {
+        return launch(ctx, fn, static_cast<uint32_t>(max_jobs * slices), 512, mm8_lds_bytes(groups, 8, 4, q6k), stream,
+                      &Q, sizeof Q);
+    };
+    auto fits_mm8 = [&](const Format &f, size_t k) {
+        const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
+        const bool q6k = f.dtype == T_Q6_K;
+        if (!(fast && ctx->use_mm8 && ctx->moe_mm8) || groups > 16 || k % 8 != 0) return false;
+        if (f.dtype != T_Q4_K && !(q6k && ctx->moe_mm8_q6k)) return false;
+        return mm8_lds_bytes(groups, 8, 4, q6k) <= 160u * 1024u;
+    };
+    int rc = GLLMQ_OK;
+    if (fits_mm8(*fg, hidden))
+        rc = grouped_mm8(*fg, gate_up, rb_gu, static_cast<uint32_t>(2 * ffn), static_cast<uint32_t>(hidden), x, true, gu);
+    else
         rc = grouped(*fg, gate_up, rb_gu, static_cast<uint32_t>(2 * ffn), static_cast<uint32_t>(hidden), x, true, gu);
-    }
     if (rc != GLLMQ_OK) return rc;
     {
         MoeActParams P{ gu, h, counters, static_cast<uint32_t>(ffn), relu_gate ? 1u : 0u };
@@ -848,7 +874,10 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
                       stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }
-    rc = grouped(*fd, down, rb_dn, static_cast<uint32_t>(hidden), static_cast<uint32_t>(ffn), h, false, o);
+    if (fits_mm8(*fd, ffn))
+        rc = grouped_mm8(*fd, down, rb_dn, static_cast<uint32_t>(hidden), static_cast<uint32_t>(ffn), h, false, o);
+    else
+        rc = grouped(*fd, down, rb_dn, static_cast<uint32_t>(hidden), static_cast<uint32_t>(ffn), h, false, o);
     if (rc != GLLMQ_OK) return rc;
     MoeCombineParams C{ o, route_weight, route_len, pair_pos, out, static_cast<uint32_t>(tokens),
                         static_cast<uint32_t>(top_k), static_cast<uint32_t>(hidden) };
