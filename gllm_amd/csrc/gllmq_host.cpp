@@ -196,6 +196,9 @@ struct gllmq_ctx {
     bool moe_mm8 = true;                        // GLLMQ_MOE_MM8=0 keeps the MoE expert rows on the GEMV kernels
     bool moe_mm8_q6k = true;                    // GLLMQ_MOE_MM8_Q6K=0 keeps Q6_K expert rows there
     bool moe_mm8_rows = true;                   // GLLMQ_MOE_MM8_ROWS=0: no wave-per-tile kernel for short Q6_K rows
+    // development overrides of launch shapes, read once at init (0 = the library's own choice):
+    // GLLMQ_MM8_GRID, GLLMQ_MMF_KSPLIT, GLLMQ_MMF_ROWS, GLLMQ_MOE_JOB_WAVES, GLLMQ_MOE_SLICES
+    uint32_t tune_mm8_grid = 0, tune_mmf_ksplit = 0, tune_mmf_rows = 0, tune_moe_job_waves = 0, tune_moe_slices = 0;
     hipFunction_t stream_read = nullptr;
     hipFunction_t mmf_q4k[2][2] = {};           // f16 matrix-core GEMM [32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
@@ -400,7 +403,7 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         int ei = steps <= 1 ? 0 : (steps <= 2 ? 1 : 2);
         while (ei < 2 && !ctx->mm8[q6k][pi][ei]) ++ei; // not every (pairs, early) pair is built
         uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
-        if (const char *v = getenv("GLLMQ_MM8_GRID")) grid = std::min<uint32_t>(P.tiles, std::max(1, atoi(v)));
+        if (ctx->tune_mm8_grid) grid = std::min<uint32_t>(P.tiles, ctx->tune_mm8_grid);
         P.grid = grid;
         hipFunction_t fn = ctx->mm8[q6k][pi][ei];
         if (pi <= 1 && ppt <= 2 && ctx->mm8_areg_on) fn = ctx->mm8_areg[q6k][pi][ei][ppt - 1];
@@ -421,14 +424,14 @@ int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     const uint32_t row_tiles = static_cast<uint32_t>((n + 255) / 256);
     if (row_tiles > kMmfMaxRowTiles) return -1;
     uint32_t ksplit = std::max(1u, static_cast<uint32_t>(ctx->num_cus) / row_tiles);
-    if (const char *v = getenv("GLLMQ_MMF_KSPLIT")) ksplit = static_cast<uint32_t>(std::max(1, atoi(v)));
+    if (ctx->tune_mmf_ksplit) ksplit = ctx->tune_mmf_ksplit;
     ksplit = std::min(ksplit, groups);
     const uint32_t bps = (groups + ksplit - 1) / ksplit;
     ksplit = (groups + bps - 1) / bps; // every workgroup gets at least one block
     std::lock_guard<std::mutex> guard(ctx->workspace_mutex);
     GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
     size_t rows_per_pass = 64;
-    if (const char *v = getenv("GLLMQ_MMF_ROWS")) rows_per_pass = atoi(v) <= 32 ? 32 : 64;
+    if (ctx->tune_mmf_rows) rows_per_pass = ctx->tune_mmf_rows <= 32 ? 32 : 64;
     // scratch: the activation images of one pass, then the partial sums
     const size_t img_bytes = static_cast<size_t>(groups) * mmf_image_bytes(std::min(m, rows_per_pass) <= 32 ? 1u : 2u);
     const size_t need = img_bytes + (ksplit > 1 ? static_cast<size_t>(ksplit) * std::min(m, rows_per_pass) * n * 4 : 0);
@@ -628,6 +631,12 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (const char *v = getenv("GLLMQ_GEMV_F32")) ctx->gemv_f32 = (v[0] == '1');
     if (const char *v = getenv("GLLMQ_MM8")) ctx->use_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MMF")) ctx->use_mmf = (v[0] != '0');
+    auto tune = [](const char *name) { const char *v = getenv(name); return v ? static_cast<uint32_t>(std::max(0, atoi(v))) : 0u; };
+    ctx->tune_mm8_grid = tune("GLLMQ_MM8_GRID");
+    ctx->tune_mmf_ksplit = tune("GLLMQ_MMF_KSPLIT");
+    ctx->tune_mmf_rows = tune("GLLMQ_MMF_ROWS");
+    ctx->tune_moe_job_waves = tune("GLLMQ_MOE_JOB_WAVES");
+    ctx->tune_moe_slices = tune("GLLMQ_MOE_SLICES");
     if (const char *v = getenv("GLLMQ_MM8_AREG")) ctx->mm8_areg_on = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MM8_Q6K_MIN_M")) ctx->mm8_q6k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
     if (const char *v = getenv("GLLMQ_MOE_MM8")) ctx->moe_mm8 = (v[0] != '0');
@@ -794,7 +803,7 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
     // Waves per job: the device takes about 8 waves per CU of these kernels; the jobs that
     // exist (at most `pairs`, typically one per routed expert) share them.
     uint32_t job_waves = std::max<uint32_t>(16u, 4u * ctx->gemv_waves / static_cast<uint32_t>(pairs));
-    if (const char *v = getenv("GLLMQ_MOE_JOB_WAVES")) job_waves = static_cast<uint32_t>(std::max(4, atoi(v)));
+    if (ctx->tune_moe_job_waves) job_waves = std::max(4u, ctx->tune_moe_job_waves);
     auto grouped = [&](const Format &f, const void *w, size_t rb, uint32_t n, uint32_t k, const float *xin,
                        bool x_by_token, float *yout) -> int {
         GemvPlan L = plan_gemv(ctx, 2, n, k, rb, job_waves);
@@ -842,7 +851,7 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         // upper bound of the jobs: one per expert hit, plus one per eight further pairs
         const uint64_t max_jobs = std::min<uint64_t>(pairs, experts + pairs / 8);
         uint32_t slices = std::max<uint32_t>(1u, (3u * static_cast<uint32_t>(ctx->num_cus)) / (2u * static_cast<uint32_t>(std::min<uint64_t>(pairs, experts))));
-        if (const char *v = getenv("GLLMQ_MOE_SLICES")) slices = static_cast<uint32_t>(std::max(1, atoi(v)));
+        if (ctx->tune_moe_slices) slices = ctx->tune_moe_slices;
         const uint32_t ppt = (groups + 7u) / 8u;
         hipFunction_t fn = ctx->moe_mm8_fn[q6k][ppt - 1];
         uint32_t units = Q.g.tiles; // what the slices of a job share: tiles, or groups of eight tiles

@@ -148,6 +148,42 @@ def test_moe_baseline_shape_reduced_expert_count(hip, torch, oracle):
     check_close(got2, want2, "moe baseline shape, default capacity")
 
 
+@pytest.mark.parametrize("hidden,ffn", [(256, 768), (512, 2304), (4352, 256)])
+def test_moe_more_than_eight_tokens_per_expert(hip, torch, oracle, hidden, ffn):
+    """Experts with around twenty tokens each: jobs of eight tokens plus a remainder.  ffn = 768
+    takes the wave-per-tile Q6_K kernel, ffn = 2304 (9 blocks per row) the tile-split one with two
+    passes per tile, hidden = 4352 (17 blocks) leaves the matrix-core kernels for the GEMV."""
+    print(f"moe >8 tokens per expert hidden={hidden} ffn={ffn}", flush=True)
+    experts, tokens, top_k = 4, 40, 2
+    gu, dn = expert_weights(Q4_K, Q6_K, experts, hidden, ffn, seed=90)
+    x = random_activations(tokens, hidden, seed=91)
+    r = oracle.route(random_gate_logits(tokens, experts, seed=92), top_k, capacity_factor=float(experts))
+    counts = np.bincount(r["expert"][:, :top_k].reshape(-1), minlength=experts)
+    assert counts.max() > 8
+    want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
+    got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
+    check_close(got, want, f"moe hidden={hidden} ffn={ffn}")
+
+
+def test_moe_grouped_kernel_alternatives(torch, oracle, monkeypatch):
+    """The grouped kernels the default dispatch does not pick for this shape: Q6_K down rows on
+    the tile-split matrix-core kernel and on the integer-dot GEMV."""
+    from gllm_amd.backend import HipBackend
+    experts, tokens, top_k, hidden, ffn = 6, 20, 3, 512, 1024
+    gu, dn = expert_weights(Q4_K, Q6_K, experts, hidden, ffn, seed=95)
+    x = random_activations(tokens, hidden, seed=96)
+    r = oracle.route(random_gate_logits(tokens, experts, seed=97), top_k, capacity_factor=float(experts))
+    want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
+    for env in ({"GLLMQ_MOE_MM8_ROWS": "0"}, {"GLLMQ_MOE_MM8_Q6K": "0"}, {"GLLMQ_MOE_MM8": "0"}):
+        print(f"moe alternatives {env}", flush=True)
+        with monkeypatch.context() as mp:
+            for k_, v_ in env.items():
+                mp.setenv(k_, v_)
+            hip2 = HipBackend(0)
+        got = run_gpu(hip2, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
+        check_close(got, want, f"moe {env}")
+
+
 def test_moe_many_pairs(hip, torch, oracle):
     """More (token, expert) pairs than the plan kernel's per-pair placement takes (4096): the
     per-expert walk is used; experts get hundreds of tokens each."""
