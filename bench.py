@@ -190,6 +190,35 @@ def run_other(args):
             sec *= 128.0 / pairs_c  # the oracle works pair by pair: scale to the 128 pairs of the workload
             sample = (f"{creps} passes over {pairs_c} (token, expert) pairs of the same expert shapes in {cdt:.1f} s, "
                       f"scaled to 128 pairs")
+    elif name.startswith("dequant_"):
+        # Backend::dequantize of one 14336 x 4096 weight matrix: block bytes in, 4 bytes per element out
+        dtype = {"dequant_q4k": 12, "dequant_q5k": 13, "dequant_q6k": 14, "dequant_q8_0": 8}.get(name)
+        if dtype is None:
+            log(f"bench.py: unknown workload {name}")
+            sys.exit(2)
+        n, k = 14336, 4096
+        copies = 3
+        ws = [device_weight_any(torch, g, dtype, n, k) for _ in range(copies)]
+        outs = [torch.empty(n * k, device="cuda") for _ in range(copies)]
+        it = [0]
+
+        def run():
+            i = it[0] % copies
+            it[0] += 1
+            hip.dequantize(ws[i], outs[i], dtype)
+        run()
+        us = timed(run, max(8, steps // 4))
+        byts = n * row_bytes(dtype, k) + n * k * 4
+        flops = 0
+        desc = f"Backend::dequantize {TAGS[dtype]} {n} x {k} (block bytes in, f32 out), rotating over {copies} matrices"
+        host_w = random_weight(dtype, n // 8, k, seed=0)
+        if args.no_cpu:
+            sec, sample = None, None
+        else:
+            sec, creps, cdt = cpu_time(lambda: cref.dequantize(host_w, dtype))
+            sec *= 8.0
+            sample = f"{creps} decodes of an eighth of the matrix ({n // 8} x {k}) on one thread in {cdt:.1f} s, scaled by 8"
+            threads = 1
     else:
         log(f"bench.py: unknown workload {name}")
         sys.exit(2)
@@ -200,7 +229,7 @@ def run_other(args):
         "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6), "us_per_call": round(us, 3),
         "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 2), "tflops": round(flops / us / 1e6, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "i8" if not name.startswith("gemm") else "f16", "data": "synthetic",
+        "dtype": "f16" if name.startswith("gemm") else ("f32" if name.startswith("dequant") else "i8"), "data": "synthetic",
         "config": {"workload": desc, "bytes_per_call": byts},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
@@ -245,7 +274,8 @@ def main():
     ap.add_argument("--no-context", action="store_true",
                     help="skip the cache-resident and streaming-read context runs (profiling: only the timed kernel launches)")
     ap.add_argument("--workload", default="gemv_q4k",
-                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, gemm_m16, gemm_m32, gemm_m64, moe")
+                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, gemm_m16, gemm_m32, gemm_m64, moe, "
+                         "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch plain device-to-device copies of one 33 MB weight buffer (counter calibration)")
     args = ap.parse_args()
