@@ -164,15 +164,24 @@ struct MoeCombineParams {
     uint32_t tokens, top_k, hidden;
 };
 
+// Formats of the int8 matrix-core kernels, in the order of the kernel tables below.
+enum Mm8Kind { MM8_Q4K = 0, MM8_Q6K = 1, MM8_Q5K = 2, MM8_KINDS = 3 };
+int mm8_kind(uint32_t dtype)
+{
+    return dtype == T_Q4_K ? MM8_Q4K : dtype == T_Q6_K ? MM8_Q6K : dtype == T_Q5_K ? MM8_Q5K : -1;
+}
+
 // Same carve-up as gq::mm8_lds_layout: bytes of LDS the int8 matrix-core kernels need.
-// q6k: 16 sub-block sums per block and a 7.5 KiB weight stage per wave instead of 8 and 5 KiB.
-uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs, bool q6k = false)
+// Q6_K keeps 16 sub-block sums per block instead of 8; the weight stage of a wave is 5, 7.5 and
+// 6 KiB for Q4_K, Q6_K and Q5_K.
+uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs, int kind = MM8_Q4K)
 {
     const uint32_t plane_stride = groups * 256u + 16u;
     const uint32_t sums = 3u * m * plane_stride;
-    const uint32_t scales = sums + m * groups * (q6k ? 16u : 8u) * 4u;
+    const uint32_t scales = sums + m * groups * (kind == MM8_Q6K ? 16u : 8u) * 4u;
     const uint32_t red = (scales + m * groups * 4u + 15u) & ~15u;
-    return red + 2u * 8u * pairs * 64u * 4u + 8u * (q6k ? 7680u : 5120u);
+    const uint32_t stage = kind == MM8_Q6K ? 7680u : kind == MM8_Q5K ? 6144u : 5120u;
+    return red + 2u * 8u * pairs * 64u * 4u + 8u * stage;
 }
 
 } // namespace
@@ -185,15 +194,16 @@ struct gllmq_ctx {
     hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1], f32 multiply-add flavour
     hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
     bool gemv_f32 = false;                      // GLLMQ_GEMV_F32=1 selects the f32 flavour
-    // int8 matrix-core kernels [0 = Q4_K, 1 = Q6_K][pairs 1,2,4][early steps 1,2,4], and the same
-    // with register-resident activation operands [..][pairs 1,2][early][passes per tile - 1]
-    hipFunction_t mm8[2][3][3] = {};
-    hipFunction_t mm8_areg[2][2][3][2] = {};
+    // int8 matrix-core kernels [Mm8Kind][pairs 1,2,4][early steps 1,2,4], and the same with
+    // register-resident activation operands [Mm8Kind][pairs 1,2][early][passes per tile - 1]
+    hipFunction_t mm8[MM8_KINDS][3][3] = {};
+    hipFunction_t mm8_areg[MM8_KINDS][2][3][2] = {};
     bool use_mm8 = true;                        // GLLMQ_MM8=0 falls back to the GEMV kernels
     bool mm8_areg_on = true;                    // GLLMQ_MM8_AREG=0 keeps the activation operands in LDS
     // Fewest activation rows that send Q6_K to the matrix-core kernel: up to two rows the GEMV
     // kernels are as fast or faster.  GLLMQ_MM8_Q6K_MIN_M overrides (1 = always, 0 = never).
     uint32_t mm8_q6k_min_m = 3;
+    uint32_t mm8_q5k_min_m = 2;                 // the same for Q5_K (GLLMQ_MM8_Q5K_MIN_M): one row is as fast on the GEMV
     bool moe_mm8 = true;                        // GLLMQ_MOE_MM8=0 keeps the MoE expert rows on the GEMV kernels
     bool moe_mm8_q6k = true;                    // GLLMQ_MOE_MM8_Q6K=0 keeps Q6_K expert rows there
     bool moe_mm8_rows = true;                   // GLLMQ_MOE_MM8_ROWS=0: no wave-per-tile kernel for short Q6_K rows
@@ -211,7 +221,7 @@ struct gllmq_ctx {
     size_t mmf_partial_bytes = 0;
     hipFunction_t moe_plan = nullptr, moe_act = nullptr, moe_combine = nullptr;
     hipFunction_t moe_gemv[kNumFormats] = {};
-    hipFunction_t moe_mm8_fn[2][2] = {};        // grouped int8 matrix-core kernels [0 = Q4_K, 1 = Q6_K][passes per tile - 1]
+    hipFunction_t moe_mm8_fn[MM8_KINDS][2] = {}; // grouped int8 matrix-core kernels [Mm8Kind][passes per tile - 1]
     hipFunction_t moe_mm8_q6k_rows = nullptr;   // Q6_K rows of at most 8 blocks: a wave per 32-row tile
     uint32_t *identity_rows = nullptr;          // device: 0..7, the activation rows of an ungathered matmul
     // Device workspace of the MoE path (pair tables, jobs, intermediate activations).  It
@@ -362,29 +372,30 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
     return -1; // go on
 }
 
-// Q4_K and Q6_K on the int8 matrix cores, activation rows in passes of at most 8 (a pass keeps
+// Q4_K, Q5_K and Q6_K on the int8 matrix cores, activation rows in passes of at most 8 (a pass keeps
 // its rows' digit planes in LDS and reads the weights once).  Returns -1 when the shape does
 // not fit the kernel (LDS for the prepared activations, alignment), so that the caller
 // takes the GEMV kernels.
 int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
             size_t k, bool act_bf16, void *stream)
 {
-    if (!ctx->use_mm8 || (f.dtype != T_Q4_K && f.dtype != T_Q6_K)) return -1;
-    const bool q6k = f.dtype == T_Q6_K;
-    if (q6k && (ctx->mm8_q6k_min_m == 0 || m < ctx->mm8_q6k_min_m)) return -1;
+    const int kind = mm8_kind(f.dtype);
+    if (!ctx->use_mm8 || kind < 0) return -1;
+    if (kind == MM8_Q6K && (ctx->mm8_q6k_min_m == 0 || m < ctx->mm8_q6k_min_m)) return -1;
+    if (kind == MM8_Q5K && (ctx->mm8_q5k_min_m == 0 || m < ctx->mm8_q5k_min_m)) return -1;
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
     // Rows per pass: as many as the prepared activations leave room for in the 160 KiB of LDS.
     auto pairs_for = [](uint32_t rows) { return rows <= 2 ? 1u : (rows <= 4 ? 2u : 4u); };
     uint32_t rows_per_pass = static_cast<uint32_t>(std::min<size_t>(m, 8));
-    while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass), q6k) > 160u * 1024u)
+    while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass), kind) > 160u * 1024u)
         --rows_per_pass;
     if (rows_per_pass == 0) return -1;
     for (size_t m0 = 0; m0 < m; m0 += rows_per_pass) {
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(rows_per_pass, m - m0));
         const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
         const uint32_t pairs = 1u << pi;
-        const uint32_t lds = mm8_lds_bytes(groups, mm, pairs, q6k);
+        const uint32_t lds = mm8_lds_bytes(groups, mm, pairs, kind);
         Mm8Params P{};
         P.w = w;
         P.x = x + m0 * k;
@@ -402,12 +413,12 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         // preparation steps per wave: two 256-element blocks per step
         const uint32_t ppt = (groups + 7u) / 8u, steps = ((ppt + 1u) / 2u) * mm;
         int ei = steps <= 1 ? 0 : (steps <= 2 ? 1 : 2);
-        while (ei < 2 && !ctx->mm8[q6k][pi][ei]) ++ei; // not every (pairs, early) pair is built
+        while (ei < 2 && !ctx->mm8[kind][pi][ei]) ++ei; // not every (pairs, early) pair is built
         uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
         if (ctx->tune_mm8_grid) grid = std::min<uint32_t>(P.tiles, ctx->tune_mm8_grid);
         P.grid = grid;
-        hipFunction_t fn = ctx->mm8[q6k][pi][ei];
-        if (pi <= 1 && ppt <= 2 && ctx->mm8_areg_on) fn = ctx->mm8_areg[q6k][pi][ei][ppt - 1];
+        hipFunction_t fn = ctx->mm8[kind][pi][ei];
+        if (pi <= 1 && ppt <= 2 && ctx->mm8_areg_on) fn = ctx->mm8_areg[kind][pi][ei][ppt - 1];
         int rc = launch(ctx, fn, grid, 512, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }
@@ -600,6 +611,8 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[0][1], "gq_moe_mm8_q4k_a2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[1][0], "gq_moe_mm8_q6k_a1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[1][1], "gq_moe_mm8_q6k_a2");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[2][0], "gq_moe_mm8_q5k_a1");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[2][1], "gq_moe_mm8_q5k_a2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_q6k_rows, "gq_moe_mm8_q6k_rows");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->dequant_wave, "gq_dequant_q4k_wave");
     if (rc == GLLMQ_OK) {
@@ -612,8 +625,8 @@ int gllmq_init(gllmq_ctx **out, int device)
         static const struct { int pi, ei; const char *tag; } kMm8[] = {
             { 0, 0, "p1_e1" }, { 0, 1, "p1_e2" }, { 0, 2, "p1_e4" }, { 1, 1, "p2_e2" }, { 1, 2, "p2_e4" }, { 2, 2, "p4_e4" },
         };
-        static const char *const kMm8Format[2] = { "q4k", "q6k" };
-        for (int q = 0; q < 2; ++q)
+        static const char *const kMm8Format[MM8_KINDS] = { "q4k", "q6k", "q5k" };
+        for (int q = 0; q < MM8_KINDS; ++q)
             for (const auto &k : kMm8) {
                 snprintf(name, sizeof name, "gq_mm8_%s_%s", kMm8Format[q], k.tag);
                 if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8[q][k.pi][k.ei], name);
@@ -641,6 +654,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     ctx->tune_moe_slices = tune("GLLMQ_MOE_SLICES");
     if (const char *v = getenv("GLLMQ_MM8_AREG")) ctx->mm8_areg_on = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MM8_Q6K_MIN_M")) ctx->mm8_q6k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
+    if (const char *v = getenv("GLLMQ_MM8_Q5K_MIN_M")) ctx->mm8_q5k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
     if (const char *v = getenv("GLLMQ_MOE_MM8")) ctx->moe_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MOE_MM8_Q6K")) ctx->moe_mm8_q6k = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MOE_MM8_ROWS")) ctx->moe_mm8_rows = (v[0] != '0');
@@ -836,7 +850,8 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
     // rows are x[token] (gate/up), else rows by sorted position (down).
     auto grouped_mm8 = [&](const Format &f, const void *wbase, size_t rb, uint32_t n, uint32_t k, const float *xin,
                            bool by_token, float *yout) -> int {
-        const bool q6k = f.dtype == T_Q6_K;
+        const int kind = mm8_kind(f.dtype);
+        const bool q6k = kind == MM8_Q6K;
         const uint32_t groups = (k + 255u) / 256u;
         MoeMm8Params Q{};
         Q.g.w = static_cast<const uint8_t *>(wbase);
@@ -858,7 +873,7 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         uint32_t slices = std::max<uint32_t>(1u, (3u * static_cast<uint32_t>(ctx->num_cus)) / (2u * static_cast<uint32_t>(std::min<uint64_t>(pairs, experts))));
         if (ctx->tune_moe_slices) slices = ctx->tune_moe_slices;
         const uint32_t ppt = (groups + 7u) / 8u;
-        hipFunction_t fn = ctx->moe_mm8_fn[q6k][ppt - 1];
+        hipFunction_t fn = ctx->moe_mm8_fn[kind][ppt - 1];
         uint32_t units = Q.g.tiles; // what the slices of a job share: tiles, or groups of eight tiles
         if (q6k && groups <= 8 && ctx->moe_mm8_rows) {
             fn = ctx->moe_mm8_q6k_rows;
@@ -866,15 +881,15 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         }
         slices = std::min(slices, units);
         Q.slices = slices;
-        return launch(ctx, fn, static_cast<uint32_t>(max_jobs * slices), 512, mm8_lds_bytes(groups, 8, 4, q6k), stream,
+        return launch(ctx, fn, static_cast<uint32_t>(max_jobs * slices), 512, mm8_lds_bytes(groups, 8, 4, kind), stream,
                       &Q, sizeof Q);
     };
     auto fits_mm8 = [&](const Format &f, size_t k) {
         const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
-        const bool q6k = f.dtype == T_Q6_K;
-        if (!(fast && ctx->use_mm8 && ctx->moe_mm8) || groups > 16 || k % 8 != 0) return false;
-        if (f.dtype != T_Q4_K && !(q6k && ctx->moe_mm8_q6k)) return false;
-        return mm8_lds_bytes(groups, 8, 4, q6k) <= 160u * 1024u;
+        const int kind = mm8_kind(f.dtype);
+        if (!(fast && ctx->use_mm8 && ctx->moe_mm8) || kind < 0 || groups > 16 || k % 8 != 0) return false;
+        if (kind == MM8_Q6K && !ctx->moe_mm8_q6k) return false;
+        return mm8_lds_bytes(groups, 8, 4, kind) <= 160u * 1024u;
     };
     int rc = GLLMQ_OK;
     if (fits_mm8(*fg, hidden))

@@ -91,9 +91,9 @@ int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks_dev, size_t n_bytes, flo
  * integers sc*q in f16, activations as two f16 terms (22 significant bits) of a per-block
  * scaled value, f32 accumulation; its scratch (activation images, partial sums of the K
  * split) lives in the context, so such calls on one context must not overlap in time.
- * Q6_K with 3 or more rows runs the same int8 matrix-core scheme, 8 rows per pass.
- * Q5_K, Q8_0, and Q6_K with one or two rows, run integer-dot GEMV kernels, two activation
- * rows per pass. */
+ * Q5_K with 2 or more rows and Q6_K with 3 or more run the same int8 matrix-core scheme,
+ * 8 rows per pass.  Q8_0, Q5_K with one row and Q6_K with one or two rows run integer-dot
+ * GEMV kernels, two activation rows per pass. */
 int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev,
                            float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,
                            void *stream);

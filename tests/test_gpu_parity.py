@@ -118,7 +118,7 @@ def test_small_m_matches_oracle(hip, torch, oracle, dtype, m):
     check_close(got, want, f"dtype={dtype} m={m}")
 
 
-@pytest.mark.parametrize("dtype", [Q4_K, Q6_K])
+@pytest.mark.parametrize("dtype", [Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("m", [3, 8])
 def test_small_m_down_projection_shape(hip, torch, oracle, dtype, m):
     # K = 14336: seven passes per tile on the matrix-core kernels, activation operands read from LDS
@@ -249,11 +249,12 @@ def test_bf16_activation_mode(hip, torch, oracle, dtype, m):
 
 @pytest.mark.parametrize("env", [{"GLLMQ_MM8": "0", "GLLMQ_MMF": "0"}, {"GLLMQ_MMF": "0"},
                                  {"GLLMQ_GEMV_F32": "1", "GLLMQ_MM8": "0", "GLLMQ_MMF": "0"},
-                                 {"GLLMQ_MM8_Q6K_MIN_M": "1"}, {"GLLMQ_MM8_Q6K_MIN_M": "0"}])
+                                 {"GLLMQ_MM8_Q6K_MIN_M": "1", "GLLMQ_MM8_Q5K_MIN_M": "1"},
+                                 {"GLLMQ_MM8_Q6K_MIN_M": "0", "GLLMQ_MM8_Q5K_MIN_M": "0"}])
 def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
     """The kernels the default dispatch does not pick: integer-dot GEMV for Q4_K, 8-row passes
-    for more than 8 rows, the f32 multiply-add flavour, Q6_K on the matrix cores for one and two
-    rows and on the GEMV kernels for more; selected per context at init."""
+    for more than 8 rows, the f32 multiply-add flavour, Q5_K and Q6_K on the matrix cores from one
+    row up and on the GEMV kernels throughout; selected per context at init."""
     from gllm_amd.backend import HipBackend
     for k_, v_ in env.items():
         monkeypatch.setenv(k_, v_)
