@@ -87,7 +87,7 @@ int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks_dev, size_t n_bytes, flo
  * Q4_K runs on the int8 matrix cores: activations become three signed base-256 digits of a
  * per-block fixed-point value, digit products accumulate exactly in i32, scales and the
  * final sum are f32; one pass over the weights serves up to 8 activation rows.  More than
- * 8 rows of Q4_K run a GEMM on the f16 matrix cores, 64 rows per pass: weights as the exact
+ * 8 rows of Q4_K or Q5_K run a GEMM on the f16 matrix cores, 64 rows per pass: weights as the exact
  * integers sc*q in f16, activations as two f16 terms (22 significant bits) of a per-block
  * scaled value, f32 accumulation; its scratch (activation images, partial sums of the K
  * split) lives in the context, so such calls on one context must not overlap in time.
