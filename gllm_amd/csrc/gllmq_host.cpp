@@ -4,6 +4,7 @@
 // (src/compat/hip_backend.rs:211-238), except that the module is loaded and every
 // function resolved once per context instead of once per launch.
 #include "gllm_hip_quant.h"
+#include "gq_params.h"
 
 #include <hip/hip_runtime_api.h>
 
@@ -64,106 +65,27 @@ int format_index(uint32_t dtype)
     return -1;
 }
 
-// Mirror of gq::GemvParams in gemv.hip.inc.
-struct GemvParams {
-    const uint8_t *w;
-    const float *x;
-    float *y;
-    uint32_t n, k, groups, row_bytes, ks, rps, rows_per_wg, ldx, ldy, x_vec, accumulate, prep_words, act_bf16;
-};
+using gq::GemvParams;
+using gq::Mm8Params;
+using gq::MmfParams;
+using gq::MmfPrepParams;
+using gq::MmfReduceParams;
+using gq::MoeActParams;
+using gq::MoeCombineParams;
+using gq::MoeGemvParams;
+using gq::MoeJob;
+using gq::MoeJob8;
+using gq::MoeMm8Params;
+using gq::MoePlanParams;
 
-// Mirror of gq::Mm8Params in mm8.hip.inc.
-struct Mm8Params {
-    const uint8_t *w;
-    const float *x;
-    float *y;
-    uint32_t n, k, groups, row_bytes, m, ldx, ldy, tiles, grid, act_bf16;
-    const uint32_t *xrows;
-};
-
-// Mirror of gq::MmfParams in mmf.hip.inc.
-struct MmfParams {
-    const uint8_t *w;
-    const float *x;
-    float *y;
-    uint8_t *ximg;
-    float *partial;
-    uint32_t n, k, groups, row_bytes, m, ldx, ldy, row_tiles, ksplit, blocks_per_split, act_bf16;
-};
-struct MmfReduceParams {
-    const float *partial;
-    float *y;
-    uint32_t m, n, ldy, ksplit;
-};
-struct MmfPrepParams {
-    const float *x;
-    uint8_t *ximg;
-    uint32_t m, k, ldx, act_bf16;
-};
-
-// gq::MmfLds<MT>::image: bytes of one block's activation image (hi, sums, inverse scales, lo),
-// padded to whole rounds of 256 x 16 bytes.
-uint32_t mmf_image_bytes(uint32_t mt)
-{
-    const uint32_t rows = 32u * mt;
-    const uint32_t raw = rows * 528u * 2u + rows * 32u + rows * 4u;
-    return (raw + 8191u) / 8192u * 8192u; // whole rounds of 512 threads x 16 bytes
-}
-
-// gq::MmfLds<MT, FMT>::total: image and one weight stage per wave (5 KiB for Q4_K, 6 KiB for
-// Q5_K), twice where that fits.
+// Bytes of one block's activation image and of the GEMM's LDS, by 32-row activation tiles (1 or
+// 2) and format (Q5_K or Q4_K).
+uint32_t mmf_image_bytes(uint32_t mt) { return mt == 1 ? gq::MmfLds<1>::image : gq::MmfLds<2>::image; }
 uint32_t mmf_lds_bytes(uint32_t mt, bool q5k)
 {
-    const uint32_t once = mmf_image_bytes(mt) + 8u * (q5k ? 6144u : 5120u);
-    return 2u * once <= 160u * 1024u ? 2u * once : once; // two sets that take turns, where they fit
+    if (mt == 1) return q5k ? gq::MmfLds<1, 1>::total : gq::MmfLds<1, 0>::total;
+    return q5k ? gq::MmfLds<2, 1>::total : gq::MmfLds<2, 0>::total;
 }
-
-// Mirrors of the structs in moe.hip.inc.
-struct MoeJob {
-    uint32_t expert, p0, m, t0, t1;
-};
-struct MoeJob8 {
-    uint32_t expert, p0, m, pad, tok[8];
-};
-struct MoePlanParams {
-    const uint32_t *route_expert;
-    const uint32_t *route_len;
-    uint32_t *pair_src;
-    uint32_t *pair_pos;
-    MoeJob *jobs;
-    MoeJob8 *jobs8;
-    uint32_t *counters;
-    uint32_t tokens, top_k, experts, pairs, fast;
-};
-struct MoeGemvParams {
-    GemvParams g;
-    const MoeJob *jobs;
-    const uint32_t *counters;
-    uint64_t expert_stride;
-    uint32_t wgs_per_job, x_by_token, x_stride, y_stride;
-};
-struct MoeMm8Params {
-    Mm8Params g;
-    const MoeJob8 *jobs;
-    const uint32_t *counters;
-    uint64_t expert_stride;
-    uint32_t slices, y_stride;
-    const uint32_t *rows;
-};
-struct MoeActParams {
-    const float *gu;
-    float *h;
-    const uint32_t *counters;
-    uint32_t ffn, relu_gate;
-};
-struct MoeCombineParams {
-    const float *o;
-    const float *route_weight;
-    const uint32_t *route_len;
-    const uint32_t *pair_pos;
-    float *out;
-    uint32_t tokens, top_k, hidden;
-};
 
 // Formats of the int8 matrix-core kernels, in the order of the kernel tables below.
 enum Mm8Kind { MM8_Q4K = 0, MM8_Q6K = 1, MM8_Q5K = 2, MM8_KINDS = 3 };
@@ -172,17 +94,13 @@ int mm8_kind(uint32_t dtype)
     return dtype == T_Q4_K ? MM8_Q4K : dtype == T_Q6_K ? MM8_Q6K : dtype == T_Q5_K ? MM8_Q5K : -1;
 }
 
-// Same carve-up as gq::mm8_lds_layout: bytes of LDS the int8 matrix-core kernels need.
-// Q6_K keeps 16 sub-block sums per block instead of 8; the weight stage of a wave is 5, 7.5 and
-// 6 KiB for Q4_K, Q6_K and Q5_K.
+// Bytes of LDS the int8 matrix-core kernels need: Q6_K keeps 16 sub-block sums per block
+// instead of 8, and the weight stage of a wave differs by format.
 uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs, int kind = MM8_Q4K)
 {
-    const uint32_t plane_stride = groups * 256u + 16u;
-    const uint32_t sums = 3u * m * plane_stride;
-    const uint32_t scales = sums + m * groups * (kind == MM8_Q6K ? 16u : 8u) * 4u;
-    const uint32_t red = (scales + m * groups * 4u + 15u) & ~15u;
-    const uint32_t stage = kind == MM8_Q6K ? 7680u : kind == MM8_Q5K ? 6144u : 5120u;
-    return red + 2u * 8u * pairs * 64u * 4u + 8u * stage;
+    const uint32_t stage = kind == MM8_Q6K ? gq::MM8Q6_STAGE_BYTES
+                         : kind == MM8_Q5K ? gq::Mm8Format<1>::STAGE : gq::Mm8Format<0>::STAGE;
+    return gq::mm8_lds_layout(groups, m, pairs, kind == MM8_Q6K ? 16u : 8u, stage).total;
 }
 
 } // namespace

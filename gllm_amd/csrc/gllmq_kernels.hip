@@ -5,6 +5,7 @@
 #include <stdint.h>
 
 #include "gq_device.h"
+#include "gq_params.h"
 
 #include "dequant.hip.inc"
 #include "gemv.hip.inc"

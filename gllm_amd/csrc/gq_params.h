@@ -1,0 +1,231 @@
+// Kernel parameter blocks and LDS layouts of the library, shared by the gfx950 kernels
+// (gllmq_kernels.hip) and the host launcher (gllmq_host.cpp): one definition, so the bytes the
+// host hands to hipModuleLaunchKernel are the struct the kernel reads.
+#ifndef GQ_PARAMS_H
+#define GQ_PARAMS_H
+
+#include <stdint.h>
+
+#if defined(__HIP__)
+#define GQ_HD __host__ __device__
+#else
+#define GQ_HD
+#endif
+
+namespace gq {
+
+struct GemvParams {
+    const uint8_t *w;
+    const float *x;
+    float *y;
+    uint32_t n;          // weight rows = outputs
+    uint32_t k;          // elements per row (activations beyond k read as zero)
+    uint32_t groups;     // 256-element groups per row = ceil(k / 256)
+    uint32_t row_bytes;  // bytes between rows
+    uint32_t ks;         // waves that share one row (K split)
+    uint32_t rps;        // rows side by side in one wave (1 when a row fills the wave)
+    uint32_t rows_per_wg;
+    uint32_t ldx;        // elements between activation rows
+    uint32_t ldy;        // elements between output rows
+    uint32_t x_vec;      // activation rows are 16-byte aligned: vector loads allowed
+    uint32_t accumulate; // add to y instead of overwriting it (K handled in several launches)
+    uint32_t prep_words; // integer-dot kernels: 32-bit words of LDS holding the prepared activations
+    uint32_t act_bf16;   // integer-dot kernels: round activations to bf16 before use
+};
+
+struct Mm8Params {
+    const uint8_t *w;
+    const float *x;
+    float *y;
+    uint32_t n;         // weight rows
+    uint32_t k;         // elements per row
+    uint32_t groups;    // 256-element blocks per row
+    uint32_t row_bytes; // bytes between rows
+    uint32_t m;         // activation rows (<= 2 * PAIRS of the kernel)
+    uint32_t ldx, ldy;
+    uint32_t tiles;     // ceil(n / 32)
+    uint32_t grid;      // workgroups launched (kept beside the other fields so one kernarg line holds all)
+    uint32_t act_bf16;  // round activations to bf16 before use
+    const uint32_t *xrows; // row of x (in units of ldx) behind each of the m activation rows: 0..m-1, or gathered rows
+};
+
+constexpr int MM8_WAVES = 8;
+constexpr int MM8_THREADS = 64 * MM8_WAVES;
+constexpr int MM8_LOADS = 5;            // 16-byte loads per lane for one 32-row block tile (4.5 used)
+constexpr int MM8_STAGE_BYTES = 5120;   // 32 rows x 144 bytes, rounded up to whole wave loads
+
+// What differs between the two formats of mm8.hip.inc.  Q5_K is Q4_K with a fifth bit per quant
+// (32 bytes of qh between the header and the nibbles): same sub-blocks, scales and mins.
+template <int FMT> struct Mm8Format;
+template <> struct Mm8Format<0> { // Q4_K
+    static constexpr uint32_t BLOCK = 144, CHUNKS = 9, QS = 16, STAGE = MM8_STAGE_BYTES;
+    static constexpr int LOADS = MM8_LOADS;
+};
+template <> struct Mm8Format<1> { // Q5_K
+    static constexpr uint32_t BLOCK = 176, CHUNKS = 11, QS = 48, STAGE = 6144; // 32 rows x 176 bytes, rounded up
+    static constexpr int LOADS = 6;                                           // 5.5 used
+};
+
+// LDS carve-up (bytes) of the int8 matrix-core kernels.
+struct Mm8Lds {
+    uint32_t plane_stride; // bytes between digit planes
+    uint32_t planes;       // offset of [3 * m][plane_stride]
+    uint32_t sums;         // offset of float [m][groups][8]: sum of X per sub-block
+    uint32_t scales;       // offset of float [m][groups]: 2^e per block (NaN if poisoned)
+    uint32_t red;          // offset of float [2][MM8_WAVES][PAIRS][64]
+    uint32_t stage;        // offset of [MM8_WAVES][MM8_STAGE_BYTES]: one weight block tile per wave
+    uint32_t total;
+};
+
+// `subs`: sub-block sums kept per 256-element block (8 of 32 elements for Q4_K, 16 of 16 for
+// Q6_K); `stage_bytes`: one wave's weight stage.
+GQ_HD inline Mm8Lds mm8_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, uint32_t subs = 8u,
+                                   uint32_t stage_bytes = MM8_STAGE_BYTES)
+{
+    Mm8Lds L;
+    L.plane_stride = groups * 256u + 16u; // +16 staggers the planes over the LDS banks
+    L.planes = 0;
+    L.sums = L.planes + 3u * m * L.plane_stride;
+    L.scales = L.sums + m * groups * subs * 4u;
+    L.red = (L.scales + m * groups * 4u + 15u) & ~15u;
+    L.stage = L.red + 2u * MM8_WAVES * pairs * 64u * 4u;
+    L.total = L.stage + MM8_WAVES * stage_bytes;
+    return L;
+}
+
+// Q6_K flavour (mm8_q6k.hip.inc)
+constexpr int MM8Q6_LOADS = 7;             // 16-byte loads per lane for one 32-row block tile (32 x 14 pieces)
+constexpr int MM8Q6_ROW_STRIDE = 240;      // bytes between rows in the stage: 224 used, padded against bank conflicts
+constexpr int MM8Q6_STAGE_BYTES = 32 * MM8Q6_ROW_STRIDE;
+
+struct MmfParams {
+    const uint8_t *w;
+    const float *x;
+    float *y;
+    uint8_t *ximg;       // [groups] images of the prepared activations, MmfLds<MT>::image bytes apart
+    float *partial;      // [ksplit][m][n] when ksplit > 1
+    uint32_t n, k, groups, row_bytes, m, ldx, ldy;
+    uint32_t row_tiles;        // ceil(n / 256)
+    uint32_t ksplit;           // workgroups per row tile
+    uint32_t blocks_per_split; // 256-element blocks of K per workgroup
+    uint32_t act_bf16;
+};
+
+constexpr int MMF_WAVES = 8;
+constexpr int MMF_ST = 1;                                  // 32-row sub-tiles per wave
+constexpr int MMF_THREADS = 64 * MMF_WAVES;
+constexpr int MMF_TILE_ROWS = 32 * MMF_ST * MMF_WAVES;     // weight rows per workgroup
+constexpr int MMF_PREP_THREADS = 1024;                     // threads that prepare one block of K
+constexpr int MMF_XROW_BYTES = 256 * 2 + 16;   // one activation row of a block in LDS (f16), padded
+constexpr int MMF_STAGE_BYTES = 5120;          // one 32-row sub-tile of one block, as fetched
+
+// FMT: 0 = Q4_K (144-byte blocks, 5 KiB per wave stage), 1 = Q5_K (176 bytes, 6 KiB).
+template <int FMT> struct MmfFormat;
+template <> struct MmfFormat<0> { static constexpr uint32_t BLOCK = 144, CHUNKS = 9, QS = 16, STAGE = 5120; static constexpr int LOADS = 5; };
+template <> struct MmfFormat<1> { static constexpr uint32_t BLOCK = 176, CHUNKS = 11, QS = 48, STAGE = 6144; static constexpr int LOADS = 6; };
+
+// LDS carve-up for MT 32-row activation tiles.  The first `image` bytes are the block image
+// that gq_mmf_prep_* writes and the GEMM copies verbatim: hi plane, sub-block sums, inverse
+// scales, lo plane, padded to whole rounds of one 16-byte chunk per thread.
+template <int MT, int FMT = 0>
+struct MmfLds {
+    static constexpr uint32_t rows = 32u * MT;
+    static constexpr uint32_t hi = 0;
+    static constexpr uint32_t sums = hi + rows * MMF_XROW_BYTES; // [rows][16] f16: 8 hi, 8 lo
+    static constexpr uint32_t inv = sums + rows * 32u;           // [rows] f32
+    static constexpr uint32_t lo = inv + rows * 4u;
+    static constexpr uint32_t round = MMF_THREADS * 16u;
+    static constexpr uint32_t loads_hi = (lo + round - 1u) / round;                           // copy rounds without the lo plane
+    static constexpr uint32_t loads_all = (lo + rows * MMF_XROW_BYTES + round - 1u) / round;  // with it
+    static constexpr uint32_t image = loads_all * round;
+    static constexpr uint32_t stages = MMF_WAVES * MMF_ST * MmfFormat<FMT>::STAGE; // one weight stage per wave
+    // One image and one set of stages, or (when two of each fit the 160 KiB of a CU) two that
+    // take turns: image p at p * image, stage set p behind the images.
+    static constexpr bool twice = 2u * (image + stages) <= 160u * 1024u;
+    static constexpr uint32_t stage = (twice ? 2u : 1u) * image; // [twice ? 2 : 1][waves][MMF_ST][MMF_STAGE_BYTES]
+    static constexpr uint32_t total = stage + (twice ? 2u : 1u) * stages;
+};
+
+struct MmfPrepParams {
+    const float *x;
+    uint8_t *ximg;
+    uint32_t m, k, ldx, act_bf16;
+};
+
+struct MmfReduceParams {
+    const float *partial; // [ksplit][m][n]
+    float *y;             // [m][ldy]
+    uint32_t m, n, ldy, ksplit;
+};
+
+struct MoeJob {
+    uint32_t expert;
+    uint32_t p0;     // sorted position of the job's first pair
+    uint32_t m;      // pairs in the job: 1 or 2
+    uint32_t t0, t1; // their tokens (t1 = t0 when m = 1)
+};
+
+// All tokens of one expert, up to eight at a time: a job of the int8 matrix-core kernel.
+struct MoeJob8 {
+    uint32_t expert;
+    uint32_t p0;     // sorted position of the job's first pair
+    uint32_t m;      // pairs in the job: 1..8
+    uint32_t pad;
+    uint32_t tok[8]; // their tokens (entries past m repeat the last one)
+};
+
+struct MoePlanParams {
+    const uint32_t *route_expert; // [tokens][top_k]
+    const uint32_t *route_len;    // [tokens]
+    uint32_t *pair_src;
+    uint32_t *pair_pos;
+    MoeJob *jobs;
+    MoeJob8 *jobs8;   // written when P.fast
+    uint32_t *counters; // [0] jobs, [1] routed pairs, [2] eight-token jobs
+    uint32_t tokens, top_k, experts, pairs;
+    uint32_t fast; // pairs are few enough for the per-pair placement (LDS has two more arrays of `pairs` words)
+};
+
+constexpr uint32_t MOE_NONE = 0xFFFFFFFFu;
+
+struct MoeGemvParams {
+    GemvParams g;            // shape, split and LDS fields; w/x/y are the bases
+    const MoeJob *jobs;
+    const uint32_t *counters;
+    uint64_t expert_stride;  // bytes between experts in g.w
+    uint32_t wgs_per_job;
+    uint32_t x_by_token;     // 1: activation row = token index, 0: sorted position
+    uint32_t x_stride;       // elements between activation rows
+    uint32_t y_stride;       // elements between output rows (by sorted position)
+};
+
+struct MoeMm8Params {
+    Mm8Params g;             // shape of one expert's matrix; w, x, y are the bases
+    const MoeJob8 *jobs;
+    const uint32_t *counters;
+    uint64_t expert_stride;  // bytes between experts in g.w
+    uint32_t slices;         // workgroups that share one job's tiles
+    uint32_t y_stride;       // elements between output rows (by sorted position)
+    const uint32_t *rows;    // null: the activation rows are the job's tokens; else this table (0, 1, ...)
+                             // counts from the job's first sorted position
+};
+
+struct MoeActParams {
+    const float *gu; // [pairs][2 * ffn]
+    float *h;        // [pairs][ffn]
+    const uint32_t *counters;
+    uint32_t ffn, relu_gate;
+};
+
+struct MoeCombineParams {
+    const float *o;               // [pairs][hidden] by sorted position
+    const float *route_weight;    // [tokens][top_k]
+    const uint32_t *route_len;    // [tokens]
+    const uint32_t *pair_pos;     // [tokens][top_k]
+    float *out;                   // [tokens][hidden]
+    uint32_t tokens, top_k, hidden;
+};
+
+} // namespace gq
+
+#endif
