@@ -79,12 +79,12 @@ using gq::MoeMm8Params;
 using gq::MoePlanParams;
 
 // Bytes of one block's activation image and of the GEMM's LDS, by 32-row activation tiles (1 or
-// 2) and format (Q5_K or Q4_K).
+// 2) and format (0 = Q4_K, 1 = Q5_K, 2 = Q6_K).
 uint32_t mmf_image_bytes(uint32_t mt) { return mt == 1 ? gq::MmfLds<1>::image : gq::MmfLds<2>::image; }
-uint32_t mmf_lds_bytes(uint32_t mt, bool q5k)
+uint32_t mmf_lds_bytes(uint32_t mt, int fmt)
 {
-    if (mt == 1) return q5k ? gq::MmfLds<1, 1>::total : gq::MmfLds<1, 0>::total;
-    return q5k ? gq::MmfLds<2, 1>::total : gq::MmfLds<2, 0>::total;
+    if (mt == 1) return fmt == 2 ? gq::MmfLds<1, 2>::total : fmt == 1 ? gq::MmfLds<1, 1>::total : gq::MmfLds<1, 0>::total;
+    return fmt == 2 ? gq::MmfLds<2, 2>::total : fmt == 1 ? gq::MmfLds<2, 1>::total : gq::MmfLds<2, 0>::total;
 }
 
 // Formats of the int8 matrix-core kernels, in the order of the kernel tables below.
@@ -130,7 +130,7 @@ struct gllmq_ctx {
     // GLLMQ_MM8_GRID, GLLMQ_MMF_KSPLIT, GLLMQ_MMF_ROWS, GLLMQ_MOE_JOB_WAVES, GLLMQ_MOE_SLICES
     uint32_t tune_mm8_grid = 0, tune_mmf_ksplit = 0, tune_mmf_rows = 0, tune_moe_job_waves = 0, tune_moe_slices = 0;
     hipFunction_t stream_read = nullptr;
-    hipFunction_t mmf_q4k[2][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K][32-row activation tiles - 1][bf16 mode]
+    hipFunction_t mmf_q4k[3][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K][32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
     hipFunction_t mmf_reduce = nullptr;         // and the in-order sum of its K-split partial results
     bool use_mmf = true;                        // GLLMQ_MMF=0 keeps m > 8 on the 8-row passes
@@ -349,8 +349,8 @@ constexpr uint32_t kMmfMaxRowTiles = 16384;
 int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
             size_t k, bool act_bf16, void *stream)
 {
-    if (!ctx->use_mmf || (f.dtype != T_Q4_K && f.dtype != T_Q5_K) || m <= 8) return -1;
-    const bool q5k = f.dtype == T_Q5_K;
+    if (!ctx->use_mmf || (f.dtype != T_Q4_K && f.dtype != T_Q5_K && f.dtype != T_Q6_K) || m <= 8) return -1;
+    const int fmt = f.dtype == T_Q6_K ? 2 : f.dtype == T_Q5_K ? 1 : 0;
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
     const uint32_t row_tiles = static_cast<uint32_t>((n + 255) / 256);
@@ -400,7 +400,7 @@ int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         MmfPrepParams Q{ P.x, P.ximg, mm, P.k, P.ldx, P.act_bf16 };
         int rc = launch2d(ctx, ctx->mmf_prep[mt - 1], groups, 16, 64, 0, stream, &Q, sizeof Q);
         if (rc != GLLMQ_OK) return rc;
-        rc = launch(ctx, ctx->mmf_q4k[q5k][mt - 1][act_bf16 ? 1 : 0], row_tiles * ksplit, 512, mmf_lds_bytes(mt, q5k), stream,
+        rc = launch(ctx, ctx->mmf_q4k[fmt][mt - 1][act_bf16 ? 1 : 0], row_tiles * ksplit, 512, mmf_lds_bytes(mt, fmt), stream,
                     &P, sizeof P);
         if (rc == GLLMQ_OK && ksplit > 1) {
             MmfReduceParams R{ P.partial, P.y, mm, P.n, P.ldy, ksplit };
@@ -516,10 +516,10 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[0], "gq_mmf_prep_t1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[1], "gq_mmf_prep_t2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_reduce, "gq_mmf_reduce");
-    for (int q = 0; q < 2 && rc == GLLMQ_OK; ++q)
+    for (int q = 0; q < 3 && rc == GLLMQ_OK; ++q)
         for (int t = 0; t < 2 && rc == GLLMQ_OK; ++t)
             for (int b = 0; b < 2 && rc == GLLMQ_OK; ++b) {
-                snprintf(name, sizeof name, "gq_mmf_%s_t%d%s", q ? "q5k" : "q4k", t + 1, b ? "_bf16" : "");
+                snprintf(name, sizeof name, "gq_mmf_%s_t%d%s", q == 2 ? "q6k" : q == 1 ? "q5k" : "q4k", t + 1, b ? "_bf16" : "");
                 rc = get_function(ctx, &ctx->mmf_q4k[q][t][b], name);
             }
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_plan, "gq_moe_plan");

@@ -13,5 +13,6 @@
 #include "mm8.hip.inc"
 #include "mm8_q6k.hip.inc"
 #include "mmf.hip.inc"
+#include "mmf_q6k.hip.inc"
 #include "moe.hip.inc"
 #include "probe.hip.inc"

@@ -87,9 +87,10 @@ int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks_dev, size_t n_bytes, flo
  * Q4_K runs on the int8 matrix cores: activations become three signed base-256 digits of a
  * per-block fixed-point value, digit products accumulate exactly in i32, scales and the
  * final sum are f32; one pass over the weights serves up to 8 activation rows.  More than
- * 8 rows of Q4_K or Q5_K run a GEMM on the f16 matrix cores, 64 rows per pass: weights as the exact
- * integers sc*q in f16, activations as two f16 terms (22 significant bits) of a per-block
- * scaled value, f32 accumulation; its scratch (activation images, partial sums of the K
+ * 8 rows of Q4_K, Q5_K or Q6_K run a GEMM on the f16 matrix cores, 64 rows per pass: weights
+ * as the exact integers sc*q in f16 (Q6_K: q-32, its scale applied per 16 elements in f32),
+ * activations as two f16 terms (22 significant bits) of a per-block scaled value, f32
+ * accumulation; its scratch (activation images, partial sums of the K
  * split) lives in the context, so such calls on one context must not overlap in time.
  * Q5_K with 2 or more rows and Q6_K with 3 or more run the same int8 matrix-core scheme,
  * 8 rows per pass.  Q8_0, Q5_K with one row and Q6_K with one or two rows run integer-dot
