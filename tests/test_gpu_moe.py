@@ -45,8 +45,14 @@ def expert_weights(dt_gu, dt_dn, experts, hidden, ffn, seed):
 
 def run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, re, rw, rl, relu_gate=False):
     tokens = x.shape[0]
-    gud, dnd = hip.upload_weights(gu), hip.upload_weights(dn)
-    xd = torch.from_numpy(np.ascontiguousarray(x, np.float32)).cuda()
+    # poison behind every input: a read past the end turns the result into NaN
+    def guarded(host, fill):
+        flat = torch.from_numpy(np.ascontiguousarray(host).reshape(-1))
+        buf = torch.full((flat.numel() + 4096,), fill, dtype=flat.dtype, device="cuda")
+        buf[:flat.numel()] = flat.cuda()
+        return buf[:flat.numel()]
+    gud, dnd = guarded(np.asarray(gu).view(np.uint8), 0xFF), guarded(np.asarray(dn).view(np.uint8), 0xFF)
+    xd = guarded(np.ascontiguousarray(x, np.float32), float("nan")).view(tokens, -1)
     out = torch.full((tokens, hidden), float("nan"), dtype=torch.float32, device="cuda")
     red = torch.from_numpy(np.ascontiguousarray(re, np.uint32).view(np.int32)).cuda()
     rwd = torch.from_numpy(np.ascontiguousarray(rw, np.float32)).cuda()

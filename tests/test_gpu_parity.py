@@ -36,9 +36,21 @@ def check_close(got, want, what=""):
     return rel
 
 
+GUARD = 4096  # elements of poison behind every device input: a read past the end shows up as NaN
+
+
+def guarded(torch, host, fill):
+    """`host` on the device at the start of a buffer whose tail is `fill` (NaN for floats, 0xFF
+    bytes for blocks: an f16 scale of 0xFFFF is a NaN)."""
+    flat = torch.from_numpy(np.ascontiguousarray(host).reshape(-1))
+    buf = torch.full((flat.numel() + GUARD,), fill, dtype=flat.dtype, device="cuda")
+    buf[:flat.numel()] = flat.cuda()
+    return buf[:flat.numel()]
+
+
 def gpu_matmul(hip, torch, w, x, dtype, m, n, k, act_mode=0):
-    wd = hip.upload_weights(w)
-    xd = torch.from_numpy(np.ascontiguousarray(x, np.float32)).cuda()
+    wd = guarded(torch, np.asarray(w).view(np.uint8), 0xFF)
+    xd = guarded(torch, np.ascontiguousarray(x, np.float32), float("nan")).view(m, k)
     yd = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
     hip.quantized_matmul(wd, xd, yd, dtype, m, n, k, act_mode=act_mode)
     torch.cuda.synchronize()
@@ -267,6 +279,26 @@ def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
             want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
             got = gpu_matmul(hip2, torch, w, x, dtype, m, n, k)
             check_close(got, want, f"env={env} dtype={dtype} m={m}")
+
+
+def test_random_shapes_sweep(hip, torch, oracle):
+    """Sixty seeded shapes across the formats, row counts on both sides of every kernel boundary
+    (1, 2, 3, 8, 9, 32, 33, 64, 65 and random ones), ragged n, k with and without a partial block."""
+    rng = np.random.default_rng(2024)
+    edge_m = [1, 2, 3, 8, 9, 32, 33, 64, 65]
+    for case in range(60):
+        dtype = ALL[case % len(ALL)]
+        m = edge_m[case % len(edge_m)] if case < 36 else int(rng.integers(1, 71))
+        n = int(rng.integers(1, 300))
+        step = 32 if dtype == Q8_0 else 256
+        k = int(rng.integers(1, 12)) * step
+        if case % 5 == 4:
+            k -= int(rng.integers(1, step // 4)) * 4  # a partial last block (k stays a multiple of 4)
+        print(f"sweep case {case}: dtype={dtype} m={m} n={n} k={k}", flush=True)
+        w, x = random_weight(dtype, n, k, seed=1000 + case), random_activations(m, k, seed=2000 + case)
+        want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+        got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+        check_close(got, want, f"case {case} dtype={dtype} m={m} n={n} k={k}")
 
 
 def test_empty_shapes_are_no_ops(hip, torch):
