@@ -190,6 +190,27 @@ def test_moe_grouped_kernel_alternatives(torch, oracle, monkeypatch):
         check_close(got, want, f"moe {env}")
 
 
+def test_moe_random_shapes_sweep(hip, torch, oracle):
+    """Sixteen seeded MoE shapes: formats in every role, expert counts from 2 to 40, top-k from 1
+    to 6, ragged hidden/ffn sizes on both sides of the matrix-core kernels' limits."""
+    rng = np.random.default_rng(77)
+    fmts = [Q4_K, Q5_K, Q6_K, Q8_0]
+    for case in range(16):
+        dt_gu, dt_dn = fmts[case % 4], fmts[(case // 4 + case) % 4]
+        experts = int(rng.integers(2, 41))
+        top_k = int(rng.integers(1, min(6, experts) + 1))
+        tokens = int(rng.integers(1, 30))
+        hidden = int(rng.integers(1, 9)) * 256
+        ffn = int(rng.integers(1, 10)) * 256
+        print(f"moe sweep case {case}: gu={dt_gu} dn={dt_dn} E={experts} k={top_k} T={tokens} H={hidden} F={ffn}", flush=True)
+        gu, dn = expert_weights(dt_gu, dt_dn, experts, hidden, ffn, seed=300 + case)
+        x = random_activations(tokens, hidden, seed=400 + case)
+        r = oracle.route(random_gate_logits(tokens, experts, seed=500 + case), top_k, capacity_factor=float(experts))
+        want = oracle.moe_ffn(gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
+        got = run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
+        check_close(got, want, f"moe sweep case {case}")
+
+
 def test_moe_many_pairs(hip, torch, oracle):
     """More (token, expert) pairs than the plan kernel's per-pair placement takes (4096): the
     per-expert walk is used; experts get hundreds of tokens each."""

@@ -51,9 +51,13 @@ def guarded(torch, host, fill):
 def gpu_matmul(hip, torch, w, x, dtype, m, n, k, act_mode=0):
     wd = guarded(torch, np.asarray(w).view(np.uint8), 0xFF)
     xd = guarded(torch, np.ascontiguousarray(x, np.float32), float("nan")).view(m, k)
-    yd = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+    # outputs start as NaN (an element nobody writes stays visible); a marker behind them must survive
+    ybuf = torch.full((m * n + GUARD,), float("nan"), dtype=torch.float32, device="cuda")
+    ybuf[m * n:] = 7.0
+    yd = ybuf[:m * n].view(m, n)
     hip.quantized_matmul(wd, xd, yd, dtype, m, n, k, act_mode=act_mode)
     torch.cuda.synchronize()
+    assert bool(torch.all(ybuf[m * n:] == 7.0)), "write past the end of the output"
     return yd.cpu().numpy()
 
 
