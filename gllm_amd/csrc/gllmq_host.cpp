@@ -88,19 +88,20 @@ uint32_t mmf_lds_bytes(uint32_t mt, int fmt)
 }
 
 // Formats of the int8 matrix-core kernels, in the order of the kernel tables below.
-enum Mm8Kind { MM8_Q4K = 0, MM8_Q6K = 1, MM8_Q5K = 2, MM8_KINDS = 3 };
+// (the grouped MoE kernels exist for the first MM8_MOE_KINDS of them)
+enum Mm8Kind { MM8_Q4K = 0, MM8_Q6K = 1, MM8_Q5K = 2, MM8_Q8_0 = 3, MM8_KINDS = 4, MM8_MOE_KINDS = 3 };
 int mm8_kind(uint32_t dtype)
 {
-    return dtype == T_Q4_K ? MM8_Q4K : dtype == T_Q6_K ? MM8_Q6K : dtype == T_Q5_K ? MM8_Q5K : -1;
+    return dtype == T_Q4_K ? MM8_Q4K : dtype == T_Q6_K ? MM8_Q6K : dtype == T_Q5_K ? MM8_Q5K : dtype == T_Q8_0 ? MM8_Q8_0 : -1;
 }
 
 // Bytes of LDS the int8 matrix-core kernels need: Q6_K keeps 16 sub-block sums per block
-// instead of 8, and the weight stage of a wave differs by format.
+// instead of 8, Q8_0 none, and the weight stage of a wave differs by format.
 uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs, int kind = MM8_Q4K)
 {
-    const uint32_t stage = kind == MM8_Q6K ? gq::MM8Q6_STAGE_BYTES
+    const uint32_t stage = kind == MM8_Q6K ? gq::MM8Q6_STAGE_BYTES : kind == MM8_Q8_0 ? gq::MM8Q8_STAGE_BYTES
                          : kind == MM8_Q5K ? gq::Mm8Format<1>::STAGE : gq::Mm8Format<0>::STAGE;
-    return gq::mm8_lds_layout(groups, m, pairs, kind == MM8_Q6K ? 16u : 8u, stage).total;
+    return gq::mm8_lds_layout(groups, m, pairs, kind == MM8_Q6K ? 16u : kind == MM8_Q8_0 ? 0u : 8u, stage).total;
 }
 
 } // namespace
@@ -123,6 +124,7 @@ struct gllmq_ctx {
     // kernels are as fast or faster.  GLLMQ_MM8_Q6K_MIN_M overrides (1 = always, 0 = never).
     uint32_t mm8_q6k_min_m = 3;
     uint32_t mm8_q5k_min_m = 2;                 // the same for Q5_K (GLLMQ_MM8_Q5K_MIN_M): one row is as fast on the GEMV
+    uint32_t mm8_q8_0_min_m = 3;                // the same for Q8_0 (GLLMQ_MM8_Q8_0_MIN_M)
     bool moe_mm8 = true;                        // GLLMQ_MOE_MM8=0 keeps the MoE expert rows on the GEMV kernels
     bool moe_mm8_q6k = true;                    // GLLMQ_MOE_MM8_Q6K=0 keeps Q6_K expert rows there
     bool moe_mm8_rows = true;                   // GLLMQ_MOE_MM8_ROWS=0: no wave-per-tile kernel for short Q6_K rows
@@ -302,6 +304,8 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     if (!ctx->use_mm8 || kind < 0) return -1;
     if (kind == MM8_Q6K && (ctx->mm8_q6k_min_m == 0 || m < ctx->mm8_q6k_min_m)) return -1;
     if (kind == MM8_Q5K && (ctx->mm8_q5k_min_m == 0 || m < ctx->mm8_q5k_min_m)) return -1;
+    if (kind == MM8_Q8_0 && (ctx->mm8_q8_0_min_m == 0 || m < ctx->mm8_q8_0_min_m)) return -1;
+    if (kind == MM8_Q8_0 && k < 256) return -1; // its fetch window is one whole group of 8 blocks
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
     // Rows per pass: as many as the prepared activations leave room for in the 160 KiB of LDS.
@@ -547,7 +551,7 @@ int gllmq_init(gllmq_ctx **out, int device)
         static const struct { int pi, ei; const char *tag; } kMm8[] = {
             { 0, 0, "p1_e1" }, { 0, 1, "p1_e2" }, { 0, 2, "p1_e4" }, { 1, 1, "p2_e2" }, { 1, 2, "p2_e4" }, { 2, 2, "p4_e4" },
         };
-        static const char *const kMm8Format[MM8_KINDS] = { "q4k", "q6k", "q5k" };
+        static const char *const kMm8Format[MM8_KINDS] = { "q4k", "q6k", "q5k", "q8_0" };
         for (int q = 0; q < MM8_KINDS; ++q)
             for (const auto &k : kMm8) {
                 snprintf(name, sizeof name, "gq_mm8_%s_%s", kMm8Format[q], k.tag);
@@ -577,6 +581,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (const char *v = getenv("GLLMQ_MM8_AREG")) ctx->mm8_areg_on = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MM8_Q6K_MIN_M")) ctx->mm8_q6k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
     if (const char *v = getenv("GLLMQ_MM8_Q5K_MIN_M")) ctx->mm8_q5k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
+    if (const char *v = getenv("GLLMQ_MM8_Q8_0_MIN_M")) ctx->mm8_q8_0_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
     if (const char *v = getenv("GLLMQ_MOE_MM8")) ctx->moe_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MOE_MM8_Q6K")) ctx->moe_mm8_q6k = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MOE_MM8_ROWS")) ctx->moe_mm8_rows = (v[0] != '0');
@@ -809,7 +814,7 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
     auto fits_mm8 = [&](const Format &f, size_t k) {
         const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
         const int kind = mm8_kind(f.dtype);
-        if (!(fast && ctx->use_mm8 && ctx->moe_mm8) || kind < 0 || groups > 16 || k % 8 != 0) return false;
+        if (!(fast && ctx->use_mm8 && ctx->moe_mm8) || kind < 0 || kind >= MM8_MOE_KINDS || groups > 16 || k % 8 != 0) return false;
         if (kind == MM8_Q6K && !ctx->moe_mm8_q6k) return false;
         return mm8_lds_bytes(groups, 8, 4, kind) <= 160u * 1024u;
     };

@@ -12,6 +12,7 @@
 #include "gemv_i8.hip.inc"
 #include "mm8.hip.inc"
 #include "mm8_q6k.hip.inc"
+#include "mm8_q8_0.hip.inc"
 #include "mmf.hip.inc"
 #include "mmf_q6k.hip.inc"
 #include "moe.hip.inc"

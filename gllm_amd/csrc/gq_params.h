@@ -78,7 +78,7 @@ struct Mm8Lds {
 };
 
 // `subs`: sub-block sums kept per 256-element block (8 of 32 elements for Q4_K, 16 of 16 for
-// Q6_K); `stage_bytes`: one wave's weight stage.
+// Q6_K, none for Q8_0); `stage_bytes`: one wave's weight stage.
 GQ_HD inline Mm8Lds mm8_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, uint32_t subs = 8u,
                                    uint32_t stage_bytes = MM8_STAGE_BYTES)
 {
@@ -97,6 +97,11 @@ GQ_HD inline Mm8Lds mm8_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, 
 constexpr int MM8Q6_LOADS = 7;             // 16-byte loads per lane for one 32-row block tile (32 x 14 pieces)
 constexpr int MM8Q6_ROW_STRIDE = 240;      // bytes between rows in the stage: 224 used, padded against bank conflicts
 constexpr int MM8Q6_STAGE_BYTES = 32 * MM8Q6_ROW_STRIDE;
+
+// Q8_0 flavour (mm8_q8_0.hip.inc): 8 blocks of 34 bytes per 256 elements
+constexpr int MM8Q8_LOADS = 9;             // 16-byte loads per lane for one 32-row group tile (32 x 17 pieces, 8.5 used)
+constexpr int MM8Q8_ROW_STRIDE = 272;      // bytes between rows in the stage: the 8 blocks as they lie in memory
+constexpr int MM8Q8_STAGE_BYTES = 32 * MM8Q8_ROW_STRIDE;
 
 struct MmfParams {
     const uint8_t *w;

@@ -265,12 +265,12 @@ def test_bf16_activation_mode(hip, torch, oracle, dtype, m):
 
 @pytest.mark.parametrize("env", [{"GLLMQ_MM8": "0", "GLLMQ_MMF": "0"}, {"GLLMQ_MMF": "0"},
                                  {"GLLMQ_GEMV_F32": "1", "GLLMQ_MM8": "0", "GLLMQ_MMF": "0"},
-                                 {"GLLMQ_MM8_Q6K_MIN_M": "1", "GLLMQ_MM8_Q5K_MIN_M": "1"},
-                                 {"GLLMQ_MM8_Q6K_MIN_M": "0", "GLLMQ_MM8_Q5K_MIN_M": "0"}])
+                                 {"GLLMQ_MM8_Q6K_MIN_M": "1", "GLLMQ_MM8_Q5K_MIN_M": "1", "GLLMQ_MM8_Q8_0_MIN_M": "1"},
+                                 {"GLLMQ_MM8_Q6K_MIN_M": "0", "GLLMQ_MM8_Q5K_MIN_M": "0", "GLLMQ_MM8_Q8_0_MIN_M": "0"}])
 def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
     """The kernels the default dispatch does not pick: integer-dot GEMV for Q4_K, 8-row passes
     for more than 8 rows, the f32 multiply-add flavour, Q5_K and Q6_K on the matrix cores from one
-    row up and on the GEMV kernels throughout; selected per context at init."""
+    row up and on the GEMV kernels throughout (Q8_0 too); selected per context at init."""
     from gllm_amd.backend import HipBackend
     for k_, v_ in env.items():
         monkeypatch.setenv(k_, v_)
@@ -303,6 +303,20 @@ def test_random_shapes_sweep(hip, torch, oracle):
         want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
         got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
         check_close(got, want, f"case {case} dtype={dtype} m={m} n={n} k={k}")
+
+
+def test_q8_0_matrix_core_shapes(hip, torch, oracle):
+    """Q8_0 with three rows and more runs on the int8 matrix cores in groups of 8 blocks: rows of
+    whole groups, rows whose last group has 1..7 blocks (its window ends with the row), one group
+    only, long rows (several passes per tile, fewer rows per pass), ragged n."""
+    cases = [(3, 70, 256), (4, 33, 288), (8, 129, 480), (5, 64, 512), (7, 31, 544), (3, 257, 4096),
+             (8, 100, 4128), (6, 40, 14336), (9, 65, 1056), (20, 50, 2272), (3, 1, 256 + 224)]
+    for m, n, k in cases:
+        print(f"q8_0 matrix cores m={m} n={n} k={k}", flush=True)
+        w, x = random_weight(Q8_0, n, k, seed=m * 1000 + n), random_activations(m, k, seed=k)
+        want = oracle.quantized_matmul(w, x, Q8_0, m, n, k, acc=oracle.ACC_F64, threads=4)
+        got = gpu_matmul(hip, torch, w, x, Q8_0, m, n, k)
+        check_close(got, want, f"q8_0 m={m} n={n} k={k}")
 
 
 def test_empty_shapes_are_no_ops(hip, torch):
