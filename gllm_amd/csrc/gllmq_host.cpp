@@ -83,8 +83,11 @@ using gq::MoePlanParams;
 uint32_t mmf_image_bytes(uint32_t mt) { return mt == 1 ? gq::MmfLds<1>::image : gq::MmfLds<2>::image; }
 uint32_t mmf_lds_bytes(uint32_t mt, int fmt)
 {
-    if (mt == 1) return fmt == 2 ? gq::MmfLds<1, 2>::total : fmt == 1 ? gq::MmfLds<1, 1>::total : gq::MmfLds<1, 0>::total;
-    return fmt == 2 ? gq::MmfLds<2, 2>::total : fmt == 1 ? gq::MmfLds<2, 1>::total : gq::MmfLds<2, 0>::total;
+    static const uint32_t kTotal[2][4] = {
+        { gq::MmfLds<1, 0>::total, gq::MmfLds<1, 1>::total, gq::MmfLds<1, 2>::total, gq::MmfLds<1, 3>::total },
+        { gq::MmfLds<2, 0>::total, gq::MmfLds<2, 1>::total, gq::MmfLds<2, 2>::total, gq::MmfLds<2, 3>::total },
+    };
+    return kTotal[mt - 1][fmt];
 }
 
 // Formats of the int8 matrix-core kernels, in the order of the kernel tables below.
@@ -132,10 +135,14 @@ struct gllmq_ctx {
     // GLLMQ_MM8_GRID, GLLMQ_MMF_KSPLIT, GLLMQ_MMF_ROWS, GLLMQ_MOE_JOB_WAVES, GLLMQ_MOE_SLICES
     uint32_t tune_mm8_grid = 0, tune_mmf_ksplit = 0, tune_mmf_rows = 0, tune_moe_job_waves = 0, tune_moe_slices = 0;
     hipFunction_t stream_read = nullptr;
-    hipFunction_t mmf_q4k[3][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K][32-row activation tiles - 1][bf16 mode]
+    hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
     hipFunction_t mmf_reduce = nullptr;         // and the in-order sum of its K-split partial results
     bool use_mmf = true;                        // GLLMQ_MMF=0 keeps m > 8 on the 8-row passes
+    // Fewest rows the GEMM takes when the 8-row kernel would need more than one pass over the
+    // weights (long rows: the prepared activations of all rows do not fit the LDS of a CU).
+    // GLLMQ_MMF_SMALL_MIN_M overrides (0 = never).
+    uint32_t mmf_small_min_m = 3;
     // Scratch of the GEMM: activation images and partial sums of K-split workgroups.  Shared
     // by all calls on this context, like `workspace`.
     void *mmf_partial = nullptr;
@@ -298,7 +305,7 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
 // not fit the kernel (LDS for the prepared activations, alignment), so that the caller
 // takes the GEMV kernels.
 int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
-            size_t k, bool act_bf16, void *stream)
+            size_t k, bool act_bf16, void *stream, bool one_pass_only = false)
 {
     const int kind = mm8_kind(f.dtype);
     if (!ctx->use_mm8 || kind < 0) return -1;
@@ -314,6 +321,7 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass), kind) > 160u * 1024u)
         --rows_per_pass;
     if (rows_per_pass == 0) return -1;
+    if (one_pass_only && rows_per_pass < m) return -1;
     for (size_t m0 = 0; m0 < m; m0 += rows_per_pass) {
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(rows_per_pass, m - m0));
         const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
@@ -351,10 +359,11 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
 constexpr uint32_t kMmfMaxRowTiles = 16384;
 
 int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
-            size_t k, bool act_bf16, void *stream)
+            size_t k, bool act_bf16, void *stream, size_t min_m = 9)
 {
-    if (!ctx->use_mmf || (f.dtype != T_Q4_K && f.dtype != T_Q5_K && f.dtype != T_Q6_K) || m <= 8) return -1;
-    const int fmt = f.dtype == T_Q6_K ? 2 : f.dtype == T_Q5_K ? 1 : 0;
+    if (!ctx->use_mmf || m < min_m) return -1;
+    const int fmt = f.dtype == T_Q8_0 ? 3 : f.dtype == T_Q6_K ? 2 : f.dtype == T_Q5_K ? 1 : 0;
+    if (fmt == 3 && k < 256) return -1; // the Q8_0 fetch window is one whole group of 8 blocks
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
     const uint32_t row_tiles = static_cast<uint32_t>((n + 255) / 256);
@@ -520,10 +529,10 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[0], "gq_mmf_prep_t1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[1], "gq_mmf_prep_t2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_reduce, "gq_mmf_reduce");
-    for (int q = 0; q < 3 && rc == GLLMQ_OK; ++q)
+    for (int q = 0; q < 4 && rc == GLLMQ_OK; ++q)
         for (int t = 0; t < 2 && rc == GLLMQ_OK; ++t)
             for (int b = 0; b < 2 && rc == GLLMQ_OK; ++b) {
-                snprintf(name, sizeof name, "gq_mmf_%s_t%d%s", q == 2 ? "q6k" : q == 1 ? "q5k" : "q4k", t + 1, b ? "_bf16" : "");
+                snprintf(name, sizeof name, "gq_mmf_%s_t%d%s", q == 3 ? "q8_0" : q == 2 ? "q6k" : q == 1 ? "q5k" : "q4k", t + 1, b ? "_bf16" : "");
                 rc = get_function(ctx, &ctx->mmf_q4k[q][t][b], name);
             }
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_plan, "gq_moe_plan");
@@ -572,6 +581,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (const char *v = getenv("GLLMQ_GEMV_F32")) ctx->gemv_f32 = (v[0] == '1');
     if (const char *v = getenv("GLLMQ_MM8")) ctx->use_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MMF")) ctx->use_mmf = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_MMF_SMALL_MIN_M")) ctx->mmf_small_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
     auto tune = [](const char *name) { const char *v = getenv(name); return v ? static_cast<uint32_t>(std::max(0, atoi(v))) : 0u; };
     ctx->tune_mm8_grid = tune("GLLMQ_MM8_GRID");
     ctx->tune_mmf_ksplit = tune("GLLMQ_MMF_KSPLIT");
@@ -646,6 +656,13 @@ int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, con
         return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "quantized_matmul: bf16 activations are not built for GLLMQ_GEMV_F32=1");
     rc = run_mmf(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
     if (rc >= 0) return rc;
+    // up to 8 rows: the int8 kernel when one pass over the weights does it, else the GEMM
+    rc = run_mm8(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream, true);
+    if (rc >= 0) return rc;
+    if (ctx->mmf_small_min_m > 0) {
+        rc = run_mmf(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream, ctx->mmf_small_min_m);
+        if (rc >= 0) return rc;
+    }
     rc = run_mm8(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
     if (rc >= 0) return rc;
     return run_gemv(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);

@@ -15,5 +15,6 @@
 #include "mm8_q8_0.hip.inc"
 #include "mmf.hip.inc"
 #include "mmf_q6k.hip.inc"
+#include "mmf_q8_0.hip.inc"
 #include "moe.hip.inc"
 #include "probe.hip.inc"

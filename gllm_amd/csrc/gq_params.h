@@ -124,11 +124,12 @@ constexpr int MMF_PREP_THREADS = 1024;                     // threads that prepa
 constexpr int MMF_XROW_BYTES = 256 * 2 + 16;   // one activation row of a block in LDS (f16), padded
 constexpr int MMF_STAGE_BYTES = 5120;          // one 32-row sub-tile of one block, as fetched
 
-// FMT: 0 = Q4_K (144-byte blocks, 5 KiB per wave stage), 1 = Q5_K (176 bytes, 6 KiB), 2 = Q6_K.
+// FMT: 0 = Q4_K (144-byte blocks, 5 KiB per wave stage), 1 = Q5_K (176 bytes, 6 KiB), 2 = Q6_K, 3 = Q8_0.
 template <int FMT> struct MmfFormat;
 template <> struct MmfFormat<0> { static constexpr uint32_t BLOCK = 144, CHUNKS = 9, QS = 16, STAGE = 5120; static constexpr int LOADS = 5; };
 template <> struct MmfFormat<1> { static constexpr uint32_t BLOCK = 176, CHUNKS = 11, QS = 48, STAGE = 6144; static constexpr int LOADS = 6; };
 template <> struct MmfFormat<2> { static constexpr uint32_t STAGE = MM8Q6_STAGE_BYTES; }; // Q6_K (mmf_q6k.hip.inc): 7.5 KiB
+template <> struct MmfFormat<3> { static constexpr uint32_t STAGE = MM8Q8_STAGE_BYTES; }; // Q8_0 (mmf_q8_0.hip.inc): 8.5 KiB
 
 // LDS carve-up for MT 32-row activation tiles.  The first `image` bytes are the block image
 // that gq_mmf_prep_* writes and the GEMM copies verbatim: hi plane, sub-block sums, inverse

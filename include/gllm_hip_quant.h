@@ -86,15 +86,18 @@ int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks_dev, size_t n_bytes, flo
  * Alignment: w_dev 16 bytes for Q4_K/Q5_K, 2 bytes for Q6_K/Q8_0; x_dev 16, y_dev 4.
  * Q4_K runs on the int8 matrix cores: activations become three signed base-256 digits of a
  * per-block fixed-point value, digit products accumulate exactly in i32, scales and the
- * final sum are f32; one pass over the weights serves up to 8 activation rows.  More than
- * 8 rows of Q4_K, Q5_K or Q6_K run a GEMM on the f16 matrix cores, 64 rows per pass: weights
- * as the exact integers sc*q in f16 (Q6_K: q-32, its scale applied per 16 elements in f32),
- * activations as two f16 terms (22 significant bits) of a per-block scaled value, f32
- * accumulation; its scratch (activation images, partial sums of the K
- * split) lives in the context, so such calls on one context must not overlap in time.
- * Q5_K with 2 or more rows and Q6_K with 3 or more run the same int8 matrix-core scheme,
- * 8 rows per pass.  Q8_0, Q5_K with one row and Q6_K with one or two rows run integer-dot
- * GEMV kernels, two activation rows per pass. */
+ * final sum are f32; one pass over the weights serves up to 8 activation rows.  Q5_K with 2
+ * or more rows, Q6_K and Q8_0 with 3 or more run the same scheme (Q8_0: one matrix-core step
+ * per 32-element block, its f16 scale applied in f32).  More than 8 rows run a GEMM on the
+ * f16 matrix cores, 64 rows per pass: weights as the exact integers sc*q in f16 (Q6_K: q-32,
+ * Q8_0: q, their scales applied per 16 or 32 elements in f32), activations as two f16 terms
+ * (22 significant bits) of a per-block scaled value, f32 accumulation; its scratch
+ * (activation images, partial sums of the K split) lives in the context, so such calls on
+ * one context must not overlap in time.  The GEMM also takes 3..8 rows when the rows are so
+ * long that the prepared activations do not fit the LDS of one 8-row pass (K above about
+ * 4096..12288, by format and rows).  Q5_K with one row, Q6_K and Q8_0 with one or two, and
+ * Q8_0 rows shorter than 256 elements run integer-dot GEMV kernels, two activation rows per
+ * pass. */
 int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev,
                            float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,
                            void *stream);

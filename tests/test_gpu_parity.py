@@ -134,10 +134,11 @@ def test_small_m_matches_oracle(hip, torch, oracle, dtype, m):
     check_close(got, want, f"dtype={dtype} m={m}")
 
 
-@pytest.mark.parametrize("dtype", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("dtype", ALL)
 @pytest.mark.parametrize("m", [3, 8])
 def test_small_m_down_projection_shape(hip, torch, oracle, dtype, m):
-    # K = 14336: seven passes per tile on the matrix-core kernels, activation operands read from LDS
+    # K = 14336: the prepared activations of all rows do not fit the LDS of one pass of the
+    # 8-row kernels, so these few rows take the GEMM kernels
     n, k = 70, 14336
     print(f"small-m long rows dtype={dtype} m={m}", flush=True)
     w, x = random_weight(dtype, n, k, seed=40 + m), random_activations(m, k, seed=41)
@@ -266,11 +267,12 @@ def test_bf16_activation_mode(hip, torch, oracle, dtype, m):
 @pytest.mark.parametrize("env", [{"GLLMQ_MM8": "0", "GLLMQ_MMF": "0"}, {"GLLMQ_MMF": "0"},
                                  {"GLLMQ_GEMV_F32": "1", "GLLMQ_MM8": "0", "GLLMQ_MMF": "0"},
                                  {"GLLMQ_MM8_Q6K_MIN_M": "1", "GLLMQ_MM8_Q5K_MIN_M": "1", "GLLMQ_MM8_Q8_0_MIN_M": "1"},
-                                 {"GLLMQ_MM8_Q6K_MIN_M": "0", "GLLMQ_MM8_Q5K_MIN_M": "0", "GLLMQ_MM8_Q8_0_MIN_M": "0"}])
+                                 {"GLLMQ_MM8_Q6K_MIN_M": "0", "GLLMQ_MM8_Q5K_MIN_M": "0", "GLLMQ_MM8_Q8_0_MIN_M": "0"},
+                                 {"GLLMQ_MMF_SMALL_MIN_M": "0"}])
 def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
     """The kernels the default dispatch does not pick: integer-dot GEMV for Q4_K, 8-row passes
     for more than 8 rows, the f32 multiply-add flavour, Q5_K and Q6_K on the matrix cores from one
-    row up and on the GEMV kernels throughout (Q8_0 too); selected per context at init."""
+    row up and on the GEMV kernels throughout (Q8_0 too), no GEMM for few rows; selected per context at init."""
     from gllm_amd.backend import HipBackend
     for k_, v_ in env.items():
         monkeypatch.setenv(k_, v_)
@@ -283,6 +285,15 @@ def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
             want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
             got = gpu_matmul(hip2, torch, w, x, dtype, m, n, k)
             check_close(got, want, f"env={env} dtype={dtype} m={m}")
+    if "GLLMQ_MMF_SMALL_MIN_M" in env:
+        # long rows on the 8-row kernels: several passes over the weights, seven blocks per wave and tile
+        for dtype in ALL:
+            for m in (3, 8):
+                n, k = 70, 14336
+                w, x = random_weight(dtype, n, k, seed=40 + m), random_activations(m, k, seed=41)
+                want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+                got = gpu_matmul(hip2, torch, w, x, dtype, m, n, k)
+                check_close(got, want, f"env={env} dtype={dtype} m={m} k={k}")
 
 
 def test_random_shapes_sweep(hip, torch, oracle):
@@ -306,11 +317,12 @@ def test_random_shapes_sweep(hip, torch, oracle):
 
 
 def test_q8_0_matrix_core_shapes(hip, torch, oracle):
-    """Q8_0 with three rows and more runs on the int8 matrix cores in groups of 8 blocks: rows of
-    whole groups, rows whose last group has 1..7 blocks (its window ends with the row), one group
+    """Q8_0 with three rows and more runs on the matrix cores in groups of 8 blocks (int8 up to 8
+    rows, the f16 GEMM beyond): rows of whole groups, rows whose last group has 1..7 blocks (its window ends with the row), one group
     only, long rows (several passes per tile, fewer rows per pass), ragged n."""
     cases = [(3, 70, 256), (4, 33, 288), (8, 129, 480), (5, 64, 512), (7, 31, 544), (3, 257, 4096),
-             (8, 100, 4128), (6, 40, 14336), (9, 65, 1056), (20, 50, 2272), (3, 1, 256 + 224)]
+             (8, 100, 4128), (6, 40, 14336), (9, 65, 1056), (20, 50, 2272), (3, 1, 256 + 224),
+             (40, 300, 4096), (64, 257, 480), (33, 64, 256), (17, 513, 14336 + 96), (12, 20, 272)]
     for m, n, k in cases:
         print(f"q8_0 matrix cores m={m} n={n} k={k}", flush=True)
         w, x = random_weight(Q8_0, n, k, seed=m * 1000 + n), random_activations(m, k, seed=k)
