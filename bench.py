@@ -220,6 +220,39 @@ def run_other(args):
             sec *= 8.0
             sample = f"{creps} decodes of an eighth of the matrix ({n // 8} x {k}) on one thread in {cdt:.1f} s, scaled by 8"
             threads = 1
+    elif name.startswith("gather_"):
+        # Op::QuantGather: 2048 token ids (a prefill) into a 32000 x 4096 embedding table;
+        # algorithmic bytes = the looked-up rows' block bytes + the ids in, 4 bytes per element out
+        dtype = {"gather_q4k": 12, "gather_q6k": 14, "gather_q8_0": 8}.get(name)
+        if dtype is None:
+            log(f"bench.py: unknown workload {name}")
+            sys.exit(2)
+        vocab, hidden, count = 32000, 4096, 2048
+        table = device_weight_any(torch, g, dtype, vocab, hidden)
+        copies = 12  # 12 x 33.5 MB of outputs rotate past the Infinity Cache
+        ids = [torch.randint(0, vocab, (count,), generator=g, device="cuda", dtype=torch.int32) for _ in range(copies)]
+        outs = [torch.empty(count * hidden, device="cuda") for _ in range(copies)]
+        it = [0]
+
+        def run():
+            i = it[0] % copies
+            it[0] += 1
+            hip.quant_gather(table, dtype, vocab, hidden, ids[i], outs[i])
+        run()
+        us = timed(run, max(8, steps // 4))
+        byts = count * row_bytes(dtype, hidden) + count * 4 + count * hidden * 4
+        flops = 0
+        desc = (f"Op::QuantGather {TAGS[dtype]}: {count} ids into a {vocab} x {hidden} table (row blocks in, f32 rows out), "
+                f"rotating over {copies} id sets and outputs")
+        host_t = random_weight(dtype, 1024, hidden, seed=0)
+        host_ids = np.random.default_rng(0).integers(0, 1024, count // 8).astype(np.uint32)
+        if args.no_cpu:
+            sec, sample = None, None
+        else:
+            sec, creps, cdt = cpu_time(lambda: cref.quant_gather(host_t, dtype, 1024, hidden, host_ids))
+            sec *= 8.0
+            sample = f"{creps} lookups of {count // 8} ids in a 1024-row table on one thread in {cdt:.1f} s, scaled by 8"
+            threads = 1
     else:
         log(f"bench.py: unknown workload {name}")
         sys.exit(2)
@@ -230,7 +263,7 @@ def run_other(args):
         "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6), "us_per_call": round(us, 3),
         "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 2), "tflops": round(flops / us / 1e6, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16" if name.startswith("gemm") else ("f32" if name.startswith("dequant") else "i8"), "data": "synthetic",
+        "dtype": "f16" if name.startswith("gemm") else ("f32" if name.startswith(("dequant", "gather")) else "i8"), "data": "synthetic",
         "config": {"workload": desc, "bytes_per_call": byts},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
@@ -276,7 +309,7 @@ def main():
                     help="skip the cache-resident and streaming-read context runs (profiling: only the timed kernel launches)")
     ap.add_argument("--workload", default="gemv_q4k",
                     help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, moe, "
-                         "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0")
+                         "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch plain device-to-device copies of one 33 MB weight buffer (counter calibration)")
     args = ap.parse_args()

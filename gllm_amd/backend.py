@@ -90,10 +90,14 @@ def load_library() -> C.CDLL:
     L.gllmq_quantized_matmul_batch.argtypes = [vp, C.POINTER(MatmulDesc), sz, vp]
     L.gllmq_moe_matvec.restype = C.c_int
     L.gllmq_moe_matvec.argtypes = [vp, vp, u32, vp, u32, vp, vp, sz, sz, sz, sz, sz, vp, vp, vp, C.c_int, vp]
+    L.gllmq_quant_gather.restype = C.c_int
+    L.gllmq_quant_gather.argtypes = [vp, vp, sz, u32, sz, sz, vp, sz, C.c_float, vp, vp]
     L.gllmq_stream_read.restype = C.c_int
     L.gllmq_stream_read.argtypes = [vp, vp, sz, vp, vp]
     L.gllmq_dequantize_host.restype = C.c_int
     L.gllmq_dequantize_host.argtypes = [vp, vp, sz, vp, sz, u32]
+    L.gllmq_quant_gather_host.restype = C.c_int
+    L.gllmq_quant_gather_host.argtypes = [vp, vp, sz, u32, sz, sz, vp, sz, C.c_float, vp]
     L.gllmq_quantized_matmul_host.restype = C.c_int
     L.gllmq_quantized_matmul_host.argtypes = [vp, vp, sz, vp, vp, u32, sz, sz, sz]
     _lib = L
@@ -104,7 +108,7 @@ EXPORTED_SYMBOLS = [
     "gllmq_init", "gllmq_destroy", "gllmq_last_error", "gllmq_status_string", "gllmq_version",
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
-    "gllmq_moe_matvec", "gllmq_stream_read", "gllmq_dequantize_host", "gllmq_quantized_matmul_host",
+    "gllmq_moe_matvec", "gllmq_quant_gather", "gllmq_stream_read", "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
 ]
 
 
@@ -228,6 +232,27 @@ class HipBackend:
         rc = self._lib.gllmq_quantized_matmul_batch(self._ctx, arr, len(items), self._stream())
         if rc != OK:
             self._raise(rc, "quantized_matmul_batch")
+
+    def quant_gather(self, table, quant_type, vocab_size: int, hidden_dim: int, token_ids, output,
+                     scale: float | None = None) -> None:
+        """Op::QuantGather: ``output[i] = scale * dequantize(table row token_ids[i])``.
+
+        ``table``: device bytes of ``vocab_size`` rows of ``hidden_dim`` quantized elements;
+        ``token_ids``: device int32/uint32 tensor; ``output``: device f32 ``[len(ids), hidden_dim]``;
+        ``scale``: the embedding scale, None for none (the reference's ``Option<f32>``)."""
+        dt = _dtype_id(quant_type)
+        if not (_is_torch(table) and table.is_cuda and token_ids.is_cuda and output.is_cuda):
+            raise OtherError("quant_gather: tensors must live on the GPU")
+        if token_ids.element_size() != 4 or token_ids.is_floating_point() or output.dtype != self._torch.float32:
+            raise OtherError("quant_gather: token ids must be 32-bit integers, output f32")
+        count = token_ids.numel()
+        if output.numel() < count * hidden_dim:
+            raise OtherError("quant_gather: output shorter than len(ids) * hidden_dim")
+        rc = self._lib.gllmq_quant_gather(self._ctx, table.data_ptr(), table.numel() * table.element_size(), dt,
+                                          vocab_size, hidden_dim, token_ids.data_ptr(), count,
+                                          1.0 if scale is None else float(scale), output.data_ptr(), self._stream())
+        if rc != OK:
+            self._raise(rc, "quant_gather")
 
     def stream_read(self, buf, sink) -> None:
         """Calibration: one streaming read of ``buf`` (device tensor, 16-byte multiple)."""

@@ -65,6 +65,7 @@ int format_index(uint32_t dtype)
     return -1;
 }
 
+using gq::GatherParams;
 using gq::GemvParams;
 using gq::Mm8Params;
 using gq::MmfParams;
@@ -113,6 +114,7 @@ struct gllmq_ctx {
     int device = 0;
     hipModule_t module = nullptr;
     hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
+    hipFunction_t gather[kNumFormats][2] = {};  // quantized embedding lookup [format][0 = scalar stores, 1 = float4 stores]
     hipFunction_t dequant_wave = nullptr;       // Q4_K with 16-byte aligned blocks and outputs: one block per wave
     hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1], f32 multiply-add flavour
     hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
@@ -517,6 +519,12 @@ int gllmq_init(gllmq_ctx **out, int device)
         if (rc != GLLMQ_OK) break;
         snprintf(name, sizeof name, "gq_dequant_%s_v4", kFormats[i].tag);
         rc = get_function(ctx, &ctx->dequant[i][1], name);
+        if (rc != GLLMQ_OK) break;
+        snprintf(name, sizeof name, "gq_gather_%s_v1", kFormats[i].tag);
+        rc = get_function(ctx, &ctx->gather[i][0], name);
+        if (rc != GLLMQ_OK) break;
+        snprintf(name, sizeof name, "gq_gather_%s_v4", kFormats[i].tag);
+        rc = get_function(ctx, &ctx->gather[i][1], name);
         for (int m = 1; m <= 2 && rc == GLLMQ_OK; ++m) {
             snprintf(name, sizeof name, "gq_gemv_%s_m%d", kFormats[i].tag, m);
             rc = get_function(ctx, &ctx->gemv[i][m - 1], name);
@@ -640,6 +648,41 @@ int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *
     // (the same form for Q5_K measured slower than the per-quad kernel: 93 against 88 us)
     if (vec && aligned(blocks, 16) && dtype == T_Q4_K) fn = ctx->dequant_wave;
     return launch(ctx, fn, grid, 256, 0, stream, &args, sizeof args);
+}
+
+int gllmq_quant_gather(gllmq_ctx *ctx, const void *table, size_t table_bytes, uint32_t dtype, size_t vocab,
+                       size_t hidden, const uint32_t *ids, size_t count, float scale, float *out, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    const Format *f = find_format(dtype);
+    if (!f)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
+                    "quant_gather: ggml dtype %u is not covered (supported: Q8_0=8, Q4_K=12, Q5_K=13, Q6_K=14)", dtype);
+    if (count == 0 || hidden == 0) return GLLMQ_OK;
+    if (!table || !ids || !out) return fail(ctx, GLLMQ_ERR_INVALID, "quant_gather: NULL device pointer");
+    if (hidden % 4 != 0) return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quant_gather: hidden = %zu is not a multiple of 4", hidden);
+    if (vocab > 0xFFFFFFFFu || hidden > 0x7FFFFFFFu || count > 0x7FFFFFFFu)
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quant_gather: dimension exceeds its 32-bit range");
+    const size_t rb = gllmq_row_bytes(dtype, hidden);
+    if (table_bytes < vocab * rb)
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quant_gather: table has %zu bytes, %zu rows of %zu elements need %zu",
+                    table_bytes, vocab, hidden, vocab * rb);
+    if (!aligned(ids, 4) || !aligned(out, 4))
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "quant_gather: ids and output must be 4-byte aligned");
+    GatherParams P{};
+    P.table = static_cast<const uint8_t *>(table);
+    P.ids = ids;
+    P.out = out;
+    P.vocab = static_cast<uint32_t>(vocab);
+    P.hidden = static_cast<uint32_t>(hidden);
+    P.row_bytes = static_cast<uint32_t>(rb);
+    P.quads_per_row = static_cast<uint32_t>(hidden / 4);
+    P.count = static_cast<uint32_t>(count);
+    P.scale = scale;
+    const int vec = aligned(out, 16) ? 1 : 0; // hidden is a multiple of 4, so every row then is
+    // (a one-block-per-wave form as in gq_dequant_q4k_wave measured the same: 15.9 against 16.0 us)
+    return launch2d(ctx, ctx->gather[format_index(dtype)][vec], (P.quads_per_row + 255u) / 256u,
+                    static_cast<uint32_t>(std::min<size_t>(count, 65535)), 256, 0, stream, &P, sizeof P);
 }
 
 int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y,
@@ -892,6 +935,38 @@ int gllmq_dequantize_host(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, fl
         rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy D2H: %s", hipGetErrorString(e));
     (void)hipFree(d_in);
     (void)hipFree(d_out);
+    return rc;
+}
+
+int gllmq_quant_gather_host(gllmq_ctx *ctx, const void *table, size_t table_bytes, uint32_t dtype, size_t vocab,
+                            size_t hidden, const uint32_t *ids, size_t count, float scale, float *out)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    const Format *f = find_format(dtype);
+    if (!f || count == 0 || hidden == 0 || !table || !ids || !out || hidden % 4 != 0 ||
+        table_bytes < vocab * gllmq_row_bytes(dtype, hidden)) // the device entry point reports these
+        return gllmq_quant_gather(ctx, table, table_bytes, dtype, vocab, hidden, ids, count, scale, out, nullptr);
+    for (size_t i = 0; i < count; ++i)
+        if (ids[i] >= vocab)
+            return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quant_gather: id %u at position %zu is outside the %zu-row table",
+                        ids[i], i, vocab);
+    const size_t tb = vocab * gllmq_row_bytes(dtype, hidden);
+    void *d_t = nullptr, *d_i = nullptr, *d_o = nullptr;
+    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipError_t e = hipMalloc(&d_t, tb);
+    if (e == hipSuccess) e = hipMalloc(&d_i, count * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc(&d_o, count * hidden * sizeof(float));
+    if (e == hipSuccess) e = hipMemcpy(d_t, table, tb, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(d_i, ids, count * sizeof(uint32_t), hipMemcpyHostToDevice);
+    int rc = e == hipSuccess ? GLLMQ_OK : fail(ctx, GLLMQ_ERR_HIP, "quant_gather: %s", hipGetErrorString(e));
+    if (rc == GLLMQ_OK)
+        rc = gllmq_quant_gather(ctx, d_t, tb, dtype, vocab, hidden, static_cast<const uint32_t *>(d_i), count, scale,
+                                static_cast<float *>(d_o), nullptr);
+    if (rc == GLLMQ_OK && (e = hipMemcpy(out, d_o, count * hidden * sizeof(float), hipMemcpyDeviceToHost)) != hipSuccess)
+        rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy D2H: %s", hipGetErrorString(e));
+    (void)hipFree(d_t);
+    (void)hipFree(d_i);
+    (void)hipFree(d_o);
     return rc;
 }
 

@@ -165,6 +165,16 @@ struct MmfReduceParams {
     uint32_t m, n, ldy, ksplit;
 };
 
+struct GatherParams {
+    const uint8_t *table;   // [vocab] rows of row_bytes
+    const uint32_t *ids;    // [count]
+    float *out;             // [count][hidden]
+    uint32_t vocab, hidden, row_bytes;
+    uint32_t quads_per_row; // hidden / 4
+    uint32_t count;
+    float scale;            // 1.0f when the lookup is not scaled
+};
+
 struct MoeJob {
     uint32_t expert;
     uint32_t p0;     // sorted position of the job's first pair

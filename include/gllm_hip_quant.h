@@ -81,6 +81,22 @@ size_t gllmq_row_bytes(uint32_t ggml_dtype, size_t k);
 int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks_dev, size_t n_bytes, float *out_dev,
                      size_t n_out, uint32_t ggml_dtype, void *stream);
 
+/* ---- Op::QuantGather: quantized embedding lookup -------------------------------------
+ * Replaces the graph op the reference emits when the embedding table is quantized
+ * (src/arch/auto_graph_fragments/build_graph.inc.rs:203-211; table bytes
+ * vocab * (hidden / block) * block_bytes, :2964-2976; scalar contract
+ * (indices u32, table, output, seq_len, hidden_dim, vocab_size),
+ * SPEC/MD-ARCHIVE/24-QUANT-PIPELINE-JIT.md:248-259).
+ * out[i][0..hidden) = scale * dequantize(row ids[i] of the table), f32; the decoders are
+ * those of gllmq_dequantize, so the values are bit-exact, and scale = 1.0f (no embedding
+ * scale; the reference uses sqrt(hidden) for models that ask for one, :3009-3013) changes no
+ * bit.  Table rows are gllmq_row_bytes(dtype, hidden) apart; hidden must be a multiple of 4.
+ * ids live on the device and are not validated by the host: an id >= vocab produces a row
+ * of NaN. */
+int gllmq_quant_gather(gllmq_ctx *ctx, const void *table_dev, size_t table_bytes, uint32_t ggml_dtype,
+                       size_t vocab, size_t hidden, const uint32_t *ids_dev, size_t count, float scale,
+                       float *out_dev, void *stream);
+
 /* ---- Backend::quantized_matmul ----------------------------------------------------
  * y[m x n] = x[m x k] . W[n x k]^T.  w_bytes must be at least n * gllmq_row_bytes(dtype,k).
  * Alignment: w_dev 16 bytes for Q4_K/Q5_K, 2 bytes for Q6_K/Q8_0; x_dev 16, y_dev 4.
@@ -154,6 +170,8 @@ int gllmq_stream_read(gllmq_ctx *ctx, const void *buf_dev, size_t n_bytes, void 
 /* ---- host-pointer convenience (upload, run, download, synchronise) ---------------- */
 int gllmq_dequantize_host(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *out,
                           size_t n_out, uint32_t ggml_dtype);
+int gllmq_quant_gather_host(gllmq_ctx *ctx, const void *table, size_t table_bytes, uint32_t ggml_dtype,
+                            size_t vocab, size_t hidden, const uint32_t *ids, size_t count, float scale, float *out);
 int gllmq_quantized_matmul_host(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x,
                                 float *y, uint32_t ggml_dtype, size_t m, size_t n, size_t k);
 

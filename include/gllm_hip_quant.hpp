@@ -107,6 +107,32 @@ public:
         return make(gllmq_quantized_matmul_batch(ctx_, descs, count, stream), "quantized_matmul_batch");
     }
 
+    // Op::QuantGather over host slices (table uploaded, rows downloaded); ids outside the table
+    // are an error of kind Other here, since the host can see them.
+    BackendError quant_gather(const uint8_t *table, size_t table_len, QuantType quant_type, size_t vocab_size,
+                              size_t hidden_dim, const uint32_t *token_ids, size_t count, const float *scale,
+                              float *output, size_t output_len) const
+    {
+        if (!ctx_) return init_error_;
+        if (output_len < count * hidden_dim)
+            return BackendError{ BackendError::Kind::Other, "quant_gather: output shorter than count * hidden_dim" };
+        return make(gllmq_quant_gather_host(ctx_, table, table_len, static_cast<uint32_t>(quant_type), vocab_size,
+                                            hidden_dim, token_ids, count, scale ? *scale : 1.0f, output),
+                    "quant_gather");
+    }
+
+    // Op::QuantGather { quant_type, vocab_size, hidden_dim, scale } over device buffers
+    // (src/arch/auto_graph_fragments/build_graph.inc.rs:203-211); scale = nullptr: none.
+    BackendError quant_gather_device(const void *table_dev, size_t table_bytes, QuantType quant_type, size_t vocab_size,
+                                     size_t hidden_dim, const uint32_t *token_ids_dev, size_t count, const float *scale,
+                                     float *out_dev, void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_quant_gather(ctx_, table_dev, table_bytes, static_cast<uint32_t>(quant_type), vocab_size,
+                                       hidden_dim, token_ids_dev, count, scale ? *scale : 1.0f, out_dev, stream),
+                    "quant_gather");
+    }
+
     // Expert FFN over a route table (ExpertRouteTable, src/moe/routing.rs:100-173).
     BackendError moe_matvec_device(const void *gate_up_dev, QuantType t_gate_up, const void *down_dev, QuantType t_down,
                                    const float *x_dev, float *out_dev, size_t tokens, size_t hidden, size_t ffn,

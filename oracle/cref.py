@@ -51,6 +51,8 @@ def lib() -> C.CDLL:
         L.gq_scale_min_k4.argtypes = [C.c_int, u8p, u8p, u8p]
         L.gq_dequantize.restype = C.c_int
         L.gq_dequantize.argtypes = [u8p, sz, f32p, sz, C.c_uint32]
+        L.gq_quant_gather.restype = C.c_int
+        L.gq_quant_gather.argtypes = [u8p, C.c_uint32, sz, sz, u32p, sz, C.c_float, C.c_int, f32p]
         L.gq_quantized_matmul.restype = C.c_int
         L.gq_quantized_matmul.argtypes = [u8p, f32p, f32p, C.c_uint32, sz, sz, sz, C.c_int, C.c_int]
         L.gq_quantized_matmul_bf16.restype = C.c_int
@@ -129,6 +131,22 @@ def dequantize(raw, dtype: int, n_out: int | None = None) -> np.ndarray:
     rc = lib().gq_dequantize(_u8(b), b.size, _f32(out), n_out, dtype)
     if rc != OK:
         raise NotImplementedError(f"dequantize: rc={rc}")
+    return out
+
+
+def quant_gather(table, dtype: int, vocab: int, hidden: int, ids, scale: float | None = None) -> np.ndarray:
+    """Op::QuantGather: rows ``ids`` of the quantized table, decoded, times ``scale`` if given."""
+    t = _bytes_arr(table)
+    idx = np.ascontiguousarray(ids, dtype=np.uint32)
+    if t.size < vocab * row_bytes(dtype, hidden):
+        raise ValueError("quant_gather: table shorter than vocab rows")
+    out = np.zeros((idx.size, hidden), np.float32)
+    rc = lib().gq_quant_gather(_u8(t), dtype, vocab, hidden, _u32(idx), idx.size,
+                               1.0 if scale is None else float(scale), 0 if scale is None else 1, _f32(out))
+    if rc == 1:
+        raise NotImplementedError(f"quant_gather: ggml dtype {dtype}")
+    if rc != OK:
+        raise ValueError(f"quant_gather: rc={rc} (an id outside the table?)")
     return out
 
 

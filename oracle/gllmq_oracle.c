@@ -214,6 +214,31 @@ int gq_dequantize(const uint8_t *blocks, size_t n_bytes, float *out, size_t n_ou
     return GQ_OK;
 }
 
+/* Op::QuantGather (src/arch/auto_graph_fragments/build_graph.inc.rs:203-211): row ids[i] of a
+ * quantized table, decoded, times the embedding scale when there is one (`scaled`).  The op is
+ * executed by generated code of gllm-kernels, which is not in the reference tree: that the scale
+ * multiplies the decoded f32 value (one rounding) is this restatement's reading of
+ * `Op::QuantGather { scale: Option<f32> }`; PARITY UNPINNED for scaled lookups.  An id outside
+ * the table is an error here. */
+int gq_quant_gather(const uint8_t *table, uint32_t t, size_t vocab, size_t hidden, const uint32_t *ids,
+                    size_t count, float scale, int scaled, float *out)
+{
+    block_fn f = codec_for(t);
+    if (!f) return GQ_ERR_UNIMPLEMENTED;
+    const size_t bb = gq_block_bytes(t), bs = gq_block_size(t), rb = gq_row_bytes(t, hidden);
+    float tmp[256];
+    for (size_t i = 0; i < count; ++i) {
+        if (ids[i] >= vocab) return GQ_ERR_BAD_SHAPE;
+        const uint8_t *row = table + (size_t)ids[i] * rb;
+        for (size_t e0 = 0, b = 0; e0 < hidden; e0 += bs, ++b) {
+            f(row + b * bb, tmp);
+            const size_t n = hidden - e0 < bs ? hidden - e0 : bs;
+            for (size_t e = 0; e < n; ++e) out[i * hidden + e0 + e] = scaled ? tmp[e] * scale : tmp[e];
+        }
+    }
+    return GQ_OK;
+}
+
 /* ------------------------------------------------------------------- matmul */
 typedef struct {
     const uint8_t *w;

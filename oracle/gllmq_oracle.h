@@ -29,6 +29,11 @@
  *                                         summation order, threading and any internal
  *                                         activation handling are PARITY UNPINNED (no
  *                                         test or fixture of the reference exercises it)
+ *   gq_quant_gather                     : unscaled lookups are pinned with gq_dequantize (a row
+ *                                         gather of its output); where the embedding scale is
+ *                                         applied is PARITY UNPINNED (the op runs in generated
+ *                                         code of gllm-kernels, no test of the reference holds
+ *                                         a value)
  *   gq_moe_ffn                          : PARITY UNPINNED beyond routing + combine rule
  *                                         (the reference's quantized expert template is
  *                                         unfinished, build_graph.inc.rs:2922-2942)
@@ -86,6 +91,12 @@ void gq_dequant_block_q8_0(const uint8_t *blk, float *out32);
  * of `out`; trailing partial chunks on either side are ignored. */
 int gq_dequantize(const uint8_t *blocks, size_t n_bytes, float *out, size_t n_out,
                   uint32_t ggml_dtype);
+
+/* Op::QuantGather (build_graph.inc.rs:203-211): out[i] = row ids[i] of the quantized table
+ * (vocab rows of `hidden` elements), decoded, times `scale` when `scaled`.  GQ_ERR_BAD_SHAPE
+ * for an id >= vocab. */
+int gq_quant_gather(const uint8_t *table, uint32_t ggml_dtype, size_t vocab, size_t hidden,
+                    const uint32_t *ids, size_t count, float scale, int scaled, float *out);
 
 /* Backend::quantized_matmul: y[m x n] = x[m x k] . W[n x k]^T, W as n rows of
  * gq_row_bytes(dtype,k) bytes.  threads <= 1 runs on the calling thread. */

@@ -59,6 +59,12 @@ extern "C" {
                             tokens: usize, hidden: usize, ffn: usize, experts: usize, top_k: usize,
                             route_expert_dev: *const u32, route_weight_dev: *const f32,
                             route_len_dev: *const u32, relu_gate: c_int, stream: *mut c_void) -> c_int;
+    pub fn gllmq_quant_gather(ctx: *mut gllmq_ctx, table_dev: *const c_void, table_bytes: usize, ggml_dtype: u32,
+                              vocab: usize, hidden: usize, ids_dev: *const u32, count: usize, scale: f32,
+                              out_dev: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn gllmq_quant_gather_host(ctx: *mut gllmq_ctx, table: *const c_void, table_bytes: usize, ggml_dtype: u32,
+                                   vocab: usize, hidden: usize, ids: *const u32, count: usize, scale: f32,
+                                   out: *mut f32) -> c_int;
     pub fn gllmq_dequantize_host(ctx: *mut gllmq_ctx, blocks: *const c_void, n_bytes: usize, out: *mut f32,
                                  n_out: usize, ggml_dtype: u32) -> c_int;
     pub fn gllmq_quantized_matmul_host(ctx: *mut gllmq_ctx, w: *const c_void, w_bytes: usize, x: *const f32,
@@ -137,6 +143,32 @@ impl HipQuant {
                                           ggml_dtype: u32, m: usize, n: usize, k: usize,
                                           stream: *mut c_void) -> Result<(), QuantError> {
         self.check(gllmq_quantized_matmul(self.ctx, w, w_bytes, x, y, ggml_dtype, m, n, k, stream), "quantized_matmul")
+    }
+
+    /// `Op::QuantGather { quant_type, vocab_size, hidden_dim, scale }` over device tensors
+    /// (src/arch/auto_graph_fragments/build_graph.inc.rs:203-211): `out[i] = scale * row ids[i]`.
+    ///
+    /// # Safety
+    /// The pointers must be valid device allocations: `table` of `table_bytes`, `ids` of `count`
+    /// u32, `out` of `count * hidden_dim` f32, on this context's device.
+    pub unsafe fn quant_gather_device(&self, table: *const c_void, table_bytes: usize, ggml_dtype: u32,
+                                      vocab_size: usize, hidden_dim: usize, ids: *const u32, count: usize,
+                                      scale: Option<f32>, out: *mut f32, stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_quant_gather(self.ctx, table, table_bytes, ggml_dtype, vocab_size, hidden_dim, ids, count,
+                                      scale.unwrap_or(1.0), out, stream), "quant_gather")
+    }
+
+    /// The same lookup with host slices (table uploaded, rows downloaded).
+    pub fn quant_gather(&self, table: &[u8], ggml_dtype: u32, vocab_size: usize, hidden_dim: usize, ids: &[u32],
+                        scale: Option<f32>, output: &mut [f32]) -> Result<(), QuantError> {
+        if output.len() < ids.len() * hidden_dim {
+            return Err(QuantError::Other("quant_gather: output shorter than ids.len() * hidden_dim".into()));
+        }
+        let rc = unsafe {
+            gllmq_quant_gather_host(self.ctx, table.as_ptr().cast(), table.len(), ggml_dtype, vocab_size, hidden_dim,
+                                    ids.as_ptr(), ids.len(), scale.unwrap_or(1.0), output.as_mut_ptr())
+        };
+        self.check(rc, "quant_gather")
     }
 }
 

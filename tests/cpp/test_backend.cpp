@@ -115,6 +115,22 @@ int main()
         // short output slice: an error of kind Other, nothing written
         e = backend.quantized_matmul(w.data(), w.size(), x.data(), x.size(), y.data(), m * n - 1, qt, m, n, k);
         CHECK(e.kind == BackendError::Kind::Other, "short output slice must be rejected");
+
+        // quant_gather: the n rows as an embedding table, bit-exact, with and without a scale
+        const uint32_t ids[5] = { 36, 0, 7, 7, 20 };
+        const float scale = 32.0f; // sqrt(k)
+        std::vector<float> rows(5 * k, -1.0f), rows_ref(5 * k, -2.0f);
+        e = backend.quant_gather(w.data(), w.size(), qt, n, k, ids, 5, nullptr, rows.data(), rows.size());
+        CHECK(e.ok(), "quant_gather: %s", e.message.c_str());
+        gq_quant_gather(w.data(), dtype, n, k, ids, 5, 1.0f, 0, rows_ref.data());
+        CHECK(std::memcmp(rows.data(), rows_ref.data(), rows.size() * 4) == 0, "quant_gather differs from the oracle");
+        e = backend.quant_gather(w.data(), w.size(), qt, n, k, ids, 5, &scale, rows.data(), rows.size());
+        CHECK(e.ok(), "scaled quant_gather: %s", e.message.c_str());
+        gq_quant_gather(w.data(), dtype, n, k, ids, 5, scale, 1, rows_ref.data());
+        CHECK(std::memcmp(rows.data(), rows_ref.data(), rows.size() * 4) == 0, "scaled quant_gather differs from the oracle");
+        const uint32_t bad[1] = { 37 };
+        e = backend.quant_gather(w.data(), w.size(), qt, n, k, bad, 1, nullptr, rows.data(), rows.size());
+        CHECK(e.kind == BackendError::Kind::Other, "an id outside the table must be rejected");
     }
     // formats outside the four are Unimplemented, never a fallback (cpu_backend.rs:1020-1046)
     {
