@@ -120,7 +120,7 @@ def run_other(args):
             if dt > budget_s or reps >= 200:
                 return dt / reps, reps, dt
 
-    if name in ("gemv_q4k_4096", "gemv_q6k", "gemm_m16", "gemm_m32", "gemm_m64", "layer_mix", "layer_mix_m32"):
+    if name in ("gemv_q4k_4096", "gemv_q6k", "gemm_m16", "gemm_m32", "gemm_m64", "layer_mix", "layer_mix_m32", "lm_head_q6k"):
         if name.startswith("layer_mix"):
             mm = 32 if name.endswith("_m32") else 1  # decode, or batched decode of 32 sequences
             ops = [(12, 6144, 4096, mm), (12, 4096, 4096, mm), (12, 2 * 14336, 4096, mm), (14, 4096, 14336, mm)]
@@ -128,7 +128,9 @@ def run_other(args):
         else:
             dtype, n, k, m = {"gemv_q4k_4096": (12, 4096, 4096, 1), "gemv_q6k": (14, 14336, 4096, 1),
                               "gemm_m16": (12, 14336, 4096, 16), "gemm_m32": (12, 14336, 4096, 32),
-                              "gemm_m64": (12, 14336, 4096, 64)}[name]
+                              "gemm_m64": (12, 14336, 4096, 64),
+                              # the output projection of a 128256-token vocabulary: Q6_K even in Q4 files
+                              "lm_head_q6k": (14, 128256, 4096, 1)}[name]
             ops = [(dtype, n, k, m)]
             copies = max(2, (300 << 20) // (n * row_bytes(dtype, k)) + 1)
         sets = []
@@ -308,7 +310,7 @@ def main():
     ap.add_argument("--no-context", action="store_true",
                     help="skip the cache-resident and streaming-read context runs (profiling: only the timed kernel launches)")
     ap.add_argument("--workload", default="gemv_q4k",
-                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, moe, "
+                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, lm_head_q6k, moe, "
                          "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch plain device-to-device copies of one 33 MB weight buffer (counter calibration)")

@@ -27,6 +27,9 @@ OK, ERR_UNIMPLEMENTED, ERR_BAD_SHAPE, ERR_BAD_ALIGNMENT, ERR_HIP, ERR_INVALID = 
 ACT_F32_SPLIT, ACT_BF16 = 0, 1
 
 
+ARGMAX_NONE = 0xFFFFFFFF  # gllmq_argmax: the row has no entry that is not NaN
+
+
 class BackendError(Exception):
     """``BackendError`` of the reference; subclasses are its variants."""
 
@@ -92,6 +95,8 @@ def load_library() -> C.CDLL:
     L.gllmq_moe_matvec.argtypes = [vp, vp, u32, vp, u32, vp, vp, sz, sz, sz, sz, sz, vp, vp, vp, C.c_int, vp]
     L.gllmq_quant_gather.restype = C.c_int
     L.gllmq_quant_gather.argtypes = [vp, vp, sz, u32, sz, sz, vp, sz, C.c_float, vp, vp]
+    L.gllmq_argmax.restype = C.c_int
+    L.gllmq_argmax.argtypes = [vp, vp, sz, sz, sz, vp, vp, vp]
     L.gllmq_stream_read.restype = C.c_int
     L.gllmq_stream_read.argtypes = [vp, vp, sz, vp, vp]
     L.gllmq_dequantize_host.restype = C.c_int
@@ -108,7 +113,7 @@ EXPORTED_SYMBOLS = [
     "gllmq_init", "gllmq_destroy", "gllmq_last_error", "gllmq_status_string", "gllmq_version",
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
-    "gllmq_moe_matvec", "gllmq_quant_gather", "gllmq_stream_read", "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
+    "gllmq_moe_matvec", "gllmq_argmax", "gllmq_quant_gather", "gllmq_stream_read", "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
 ]
 
 
@@ -253,6 +258,24 @@ class HipBackend:
                                           1.0 if scale is None else float(scale), output.data_ptr(), self._stream())
         if rc != OK:
             self._raise(rc, "quant_gather")
+
+    def argmax(self, logits, token, value=None) -> None:
+        """Op::Argmax with the semantics of the reference's ``argmax_token``: ``token[r]`` = index of
+        the largest non-NaN entry of row ``r`` of the device f32 matrix ``logits`` (a view with a row
+        stride is fine), the last of equal maxima, ``ARGMAX_NONE`` when there is none."""
+        if not (logits.is_cuda and token.is_cuda and logits.dtype == self._torch.float32 and token.element_size() == 4):
+            raise OtherError("argmax: logits must be device f32, token a device 32-bit integer tensor")
+        lg = logits if logits.dim() == 2 else logits.reshape(1, -1)
+        if lg.stride(1) != 1 and lg.shape[1] > 1:
+            raise OtherError("argmax: rows must be contiguous")
+        rows, n = lg.shape
+        ld = lg.stride(0) if rows > 1 else max(n, 1)
+        if token.numel() < rows or (value is not None and value.numel() < rows):
+            raise OtherError("argmax: token/value shorter than the number of rows")
+        rc = self._lib.gllmq_argmax(self._ctx, lg.data_ptr(), rows, n, ld, token.data_ptr(),
+                                    value.data_ptr() if value is not None else None, self._stream())
+        if rc != OK:
+            self._raise(rc, "argmax")
 
     def stream_read(self, buf, sink) -> None:
         """Calibration: one streaming read of ``buf`` (device tensor, 16-byte multiple)."""

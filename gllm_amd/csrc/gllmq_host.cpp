@@ -65,6 +65,7 @@ int format_index(uint32_t dtype)
     return -1;
 }
 
+using gq::ArgmaxParams;
 using gq::GatherParams;
 using gq::GemvParams;
 using gq::Mm8Params;
@@ -115,6 +116,8 @@ struct gllmq_ctx {
     hipModule_t module = nullptr;
     hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
     hipFunction_t gather[kNumFormats][2] = {};  // quantized embedding lookup [format][0 = scalar stores, 1 = float4 stores]
+    hipFunction_t argmax_part = nullptr, argmax_final = nullptr;
+    uint64_t *argmax_keys = nullptr;            // [ARGMAX_MAX_ROWS][ARGMAX_MAX_PARTS] scratch of gllmq_argmax
     hipFunction_t dequant_wave = nullptr;       // Q4_K with 16-byte aligned blocks and outputs: one block per wave
     hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1], f32 multiply-add flavour
     hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
@@ -558,6 +561,13 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[2][1], "gq_moe_mm8_q5k_a2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_q6k_rows, "gq_moe_mm8_q6k_rows");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->dequant_wave, "gq_dequant_q4k_wave");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->argmax_part, "gq_argmax_part");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->argmax_final, "gq_argmax_final");
+    if (rc == GLLMQ_OK) {
+        hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->argmax_keys),
+                                  sizeof(uint64_t) * gq::ARGMAX_MAX_ROWS * gq::ARGMAX_MAX_PARTS);
+        if (he != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "argmax scratch: %s", hipGetErrorString(he));
+    }
     if (rc == GLLMQ_OK) {
         static const uint32_t kRows[8] = { 0, 1, 2, 3, 4, 5, 6, 7 };
         hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->identity_rows), sizeof kRows);
@@ -616,6 +626,7 @@ void gllmq_destroy(gllmq_ctx *ctx)
     if (!ctx) return;
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->identity_rows) (void)hipFree(ctx->identity_rows);
+    if (ctx->argmax_keys) (void)hipFree(ctx->argmax_keys);
     if (ctx->mmf_partial) (void)hipFree(ctx->mmf_partial);
     if (ctx->module) (void)hipModuleUnload(ctx->module);
     delete ctx;
@@ -683,6 +694,34 @@ int gllmq_quant_gather(gllmq_ctx *ctx, const void *table, size_t table_bytes, ui
     // (a one-block-per-wave form as in gq_dequant_q4k_wave measured the same: 15.9 against 16.0 us)
     return launch2d(ctx, ctx->gather[format_index(dtype)][vec], (P.quads_per_row + 255u) / 256u,
                     static_cast<uint32_t>(std::min<size_t>(count, 65535)), 256, 0, stream, &P, sizeof P);
+}
+
+int gllmq_argmax(gllmq_ctx *ctx, const float *logits, size_t rows, size_t n, size_t ld, uint32_t *token, float *value,
+                 void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    if (rows == 0) return GLLMQ_OK;
+    if ((!logits && n > 0) || !token) return fail(ctx, GLLMQ_ERR_INVALID, "argmax: NULL device pointer");
+    if (n > 0xFFFFFFFEu || ld > 0xFFFFFFFFu || rows > 0x7FFFFFFFu || ld < n)
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "argmax: n = %zu, ld = %zu, rows = %zu out of range", n, ld, rows);
+    if (!aligned(logits, 4) || !aligned(token, 4) || (value && !aligned(value, 4)))
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "argmax: buffers must be 4-byte aligned");
+    ArgmaxParams P{};
+    P.keys = ctx->argmax_keys;
+    P.n = static_cast<uint32_t>(n);
+    P.ld = static_cast<uint32_t>(ld);
+    P.parts = static_cast<uint32_t>(std::min<size_t>(gq::ARGMAX_MAX_PARTS, std::max<size_t>(1, (n + 4095) / 4096)));
+    P.chunk = static_cast<uint32_t>((n + P.parts - 1) / P.parts);
+    for (size_t r0 = 0; r0 < rows; r0 += gq::ARGMAX_MAX_ROWS) {
+        const uint32_t rr = static_cast<uint32_t>(std::min<size_t>(gq::ARGMAX_MAX_ROWS, rows - r0));
+        P.logits = logits + r0 * ld;
+        P.token = token + r0;
+        P.value = value ? value + r0 : nullptr;
+        int rc = launch2d(ctx, ctx->argmax_part, P.parts, rr, 256, 0, stream, &P, sizeof P);
+        if (rc == GLLMQ_OK && P.parts > 1) rc = launch(ctx, ctx->argmax_final, rr, 256, 0, stream, &P, sizeof P);
+        if (rc != GLLMQ_OK) return rc;
+    }
+    return GLLMQ_OK;
 }
 
 int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y,

@@ -17,4 +17,5 @@
 #include "mmf_q6k.hip.inc"
 #include "mmf_q8_0.hip.inc"
 #include "moe.hip.inc"
+#include "argmax.hip.inc"
 #include "probe.hip.inc"

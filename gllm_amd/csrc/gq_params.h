@@ -175,6 +175,19 @@ struct GatherParams {
     float scale;            // 1.0f when the lookup is not scaled
 };
 
+struct ArgmaxParams {
+    const float *logits; // [rows][ld]
+    uint32_t *token;     // [rows]
+    float *value;        // [rows] or null: the winning logit
+    uint64_t *keys;      // [rows][parts] scratch between the two launches
+    uint32_t n, ld;      // entries per row, elements between rows
+    uint32_t parts;      // workgroups per row
+    uint32_t chunk;      // entries per part
+};
+
+constexpr uint32_t ARGMAX_NONE = 0xFFFFFFFFu; // the row has no entry that is not NaN
+constexpr uint32_t ARGMAX_MAX_PARTS = 128, ARGMAX_MAX_ROWS = 64; // scratch keys per launch pair
+
 struct MoeJob {
     uint32_t expert;
     uint32_t p0;     // sorted position of the job's first pair

@@ -97,6 +97,18 @@ int gllmq_quant_gather(gllmq_ctx *ctx, const void *table_dev, size_t table_bytes
                        size_t vocab, size_t hidden, const uint32_t *ids_dev, size_t count, float scale,
                        float *out_dev, void *stream);
 
+/* ---- Op::Argmax: greedy token choice behind the lm_head matmul -----------------------
+ * Replaces the graph op of src/arch/auto_graph_fragments/build_graph.inc.rs:2661 with the
+ * semantics of argmax_token (src/engine/executor_step.rs:48-55; its unit tests :2191-2325):
+ * token_dev[r] = index of the largest entry of row r that is not NaN; of equal maxima the
+ * LAST one wins; GLLMQ_ARGMAX_NONE when the row is empty or all NaN (the reference's None).
+ * logits_dev is [rows][ld] f32 with n <= ld entries used per row; value_dev (may be NULL)
+ * receives the winning logit (NaN for no token).  Scratch between the two launches lives
+ * in the context: calls on one context must not overlap in time. */
+#define GLLMQ_ARGMAX_NONE 0xFFFFFFFFu
+int gllmq_argmax(gllmq_ctx *ctx, const float *logits_dev, size_t rows, size_t n, size_t ld,
+                 uint32_t *token_dev, float *value_dev, void *stream);
+
 /* ---- Backend::quantized_matmul ----------------------------------------------------
  * y[m x n] = x[m x k] . W[n x k]^T.  w_bytes must be at least n * gllmq_row_bytes(dtype,k).
  * Alignment: w_dev 16 bytes for Q4_K/Q5_K, 2 bytes for Q6_K/Q8_0; x_dev 16, y_dev 4.

@@ -133,6 +133,14 @@ public:
                     "quant_gather");
     }
 
+    // Op::Argmax over device logits [rows][ld] (argmax_token, src/engine/executor_step.rs:48-55).
+    BackendError argmax_device(const float *logits_dev, size_t rows, size_t n, size_t ld, uint32_t *token_dev,
+                               float *value_dev = nullptr, void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_argmax(ctx_, logits_dev, rows, n, ld, token_dev, value_dev, stream), "argmax");
+    }
+
     // Expert FFN over a route table (ExpertRouteTable, src/moe/routing.rs:100-173).
     BackendError moe_matvec_device(const void *gate_up_dev, QuantType t_gate_up, const void *down_dev, QuantType t_down,
                                    const float *x_dev, float *out_dev, size_t tokens, size_t hidden, size_t ffn,

@@ -53,6 +53,8 @@ def lib() -> C.CDLL:
         L.gq_dequantize.argtypes = [u8p, sz, f32p, sz, C.c_uint32]
         L.gq_quant_gather.restype = C.c_int
         L.gq_quant_gather.argtypes = [u8p, C.c_uint32, sz, sz, u32p, sz, C.c_float, C.c_int, f32p]
+        L.gq_argmax_token.restype = C.c_int64
+        L.gq_argmax_token.argtypes = [f32p, sz]
         L.gq_quantized_matmul.restype = C.c_int
         L.gq_quantized_matmul.argtypes = [u8p, f32p, f32p, C.c_uint32, sz, sz, sz, C.c_int, C.c_int]
         L.gq_quantized_matmul_bf16.restype = C.c_int
@@ -132,6 +134,13 @@ def dequantize(raw, dtype: int, n_out: int | None = None) -> np.ndarray:
     if rc != OK:
         raise NotImplementedError(f"dequantize: rc={rc}")
     return out
+
+
+def argmax_token(logits):
+    """argmax_token of the reference: None for an empty or all-NaN vector."""
+    a = np.ascontiguousarray(logits, np.float32).reshape(-1)
+    r = lib().gq_argmax_token(_f32(a), a.size)
+    return None if r < 0 else int(r)
 
 
 def quant_gather(table, dtype: int, vocab: int, hidden: int, ids, scale: float | None = None) -> np.ndarray:

@@ -239,6 +239,19 @@ int gq_quant_gather(const uint8_t *table, uint32_t t, size_t vocab, size_t hidde
     return GQ_OK;
 }
 
+/* argmax_token, src/engine/executor_step.rs:48-55: entries that are NaN are filtered out, then
+ * Iterator::max_by(partial_cmp), which keeps the LAST of several equal maxima (-0.0 == +0.0).
+ * Returns -1 for the reference's None (empty or all NaN). */
+int64_t gq_argmax_token(const float *logits, size_t n)
+{
+    int64_t best = -1;
+    for (size_t i = 0; i < n; ++i) {
+        if (logits[i] != logits[i]) continue;
+        if (best < 0 || !(logits[i] < logits[best])) best = (int64_t)i; /* >= : a later equal entry replaces */
+    }
+    return best;
+}
+
 /* ------------------------------------------------------------------- matmul */
 typedef struct {
     const uint8_t *w;

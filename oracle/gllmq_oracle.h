@@ -34,6 +34,8 @@
  *                                         applied is PARITY UNPINNED (the op runs in generated
  *                                         code of gllm-kernels, no test of the reference holds
  *                                         a value)
+ *   gq_argmax_token                     : pinned by the reference's unit-test vectors
+ *                                         (src/engine/executor_step.rs:2191-2325)
  *   gq_moe_ffn                          : PARITY UNPINNED beyond routing + combine rule
  *                                         (the reference's quantized expert template is
  *                                         unfinished, build_graph.inc.rs:2922-2942)
@@ -97,6 +99,10 @@ int gq_dequantize(const uint8_t *blocks, size_t n_bytes, float *out, size_t n_ou
  * for an id >= vocab. */
 int gq_quant_gather(const uint8_t *table, uint32_t ggml_dtype, size_t vocab, size_t hidden,
                     const uint32_t *ids, size_t count, float scale, int scaled, float *out);
+
+/* argmax_token (src/engine/executor_step.rs:48-55): index of the largest entry that is not
+ * NaN, the last one of equal maxima; -1 when there is none. */
+int64_t gq_argmax_token(const float *logits, size_t n);
 
 /* Backend::quantized_matmul: y[m x n] = x[m x k] . W[n x k]^T, W as n rows of
  * gq_row_bytes(dtype,k) bytes.  threads <= 1 runs on the calling thread. */

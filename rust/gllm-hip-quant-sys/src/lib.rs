@@ -59,6 +59,8 @@ extern "C" {
                             tokens: usize, hidden: usize, ffn: usize, experts: usize, top_k: usize,
                             route_expert_dev: *const u32, route_weight_dev: *const f32,
                             route_len_dev: *const u32, relu_gate: c_int, stream: *mut c_void) -> c_int;
+    pub fn gllmq_argmax(ctx: *mut gllmq_ctx, logits_dev: *const f32, rows: usize, n: usize, ld: usize,
+                        token_dev: *mut u32, value_dev: *mut f32, stream: *mut c_void) -> c_int;
     pub fn gllmq_quant_gather(ctx: *mut gllmq_ctx, table_dev: *const c_void, table_bytes: usize, ggml_dtype: u32,
                               vocab: usize, hidden: usize, ids_dev: *const u32, count: usize, scale: f32,
                               out_dev: *mut f32, stream: *mut c_void) -> c_int;
@@ -156,6 +158,16 @@ impl HipQuant {
                                       scale: Option<f32>, out: *mut f32, stream: *mut c_void) -> Result<(), QuantError> {
         self.check(gllmq_quant_gather(self.ctx, table, table_bytes, ggml_dtype, vocab_size, hidden_dim, ids, count,
                                       scale.unwrap_or(1.0), out, stream), "quant_gather")
+    }
+
+    /// `Op::Argmax` over device logits `[rows][ld]` (argmax_token, src/engine/executor_step.rs:48-55):
+    /// `token[r]` is `u32::MAX` where the reference returns `None`.
+    ///
+    /// # Safety
+    /// `logits` must hold `rows * ld` f32, `token` `rows` u32, `value` null or `rows` f32, on this device.
+    pub unsafe fn argmax_device(&self, logits: *const f32, rows: usize, n: usize, ld: usize, token: *mut u32,
+                                value: *mut f32, stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_argmax(self.ctx, logits, rows, n, ld, token, value, stream), "argmax")
     }
 
     /// The same lookup with host slices (table uploaded, rows downloaded).
