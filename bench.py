@@ -15,6 +15,7 @@ and bracketed by events on that stream.  Prints one JSON line.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -102,12 +103,17 @@ def run_other(args):
     steps = min(args.steps, 400)
 
     def timed(fn, reps):
-        torch.cuda.synchronize()
-        start.record()
-        for _ in range(reps):
-            fn()
-        stop.record()
-        torch.cuda.synchronize()
+        gc.collect()  # no pass of Python's garbage collector inside the timed region
+        gc.disable()
+        try:
+            torch.cuda.synchronize()
+            start.record()
+            for _ in range(reps):
+                fn()
+            stop.record()
+            torch.cuda.synchronize()
+        finally:
+            gc.enable()
         return start.elapsed_time(stop) * 1e3 / reps  # us
 
     def cpu_time(fn, budget_s=8.0):
@@ -222,6 +228,40 @@ def run_other(args):
             sec *= 8.0
             sample = f"{creps} decodes of an eighth of the matrix ({n // 8} x {k}) on one thread in {cdt:.1f} s, scaled by 8"
             threads = 1
+    elif name in ("ffn_m1", "ffn_m4", "ffn_m32"):
+        # dense feed-forward block of the layer mix: gate and up Q4_K 4096 -> 14336, SwiGLU, down Q6_K
+        # 14336 -> 4096; algorithmic bytes = the three matrices once + x in + out (the intermediates
+        # are the implementation's own traffic)
+        mm = int(name.split("_m")[1])
+        H, F = 4096, 14336
+        copies = 3
+        sets = []
+        for _ in range(copies):
+            gu = device_weight_any(torch, g, 12, 2 * F, H)
+            half = gu.numel() // 2
+            sets.append((gu[:half], gu[half:], device_weight_any(torch, g, 14, H, F),
+                         torch.randn(mm, H, device="cuda", generator=g), torch.empty(mm, H, device="cuda")))
+        it = [0]
+
+        def run():
+            ga, up_, dn, xx, oo = sets[it[0] % copies]
+            it[0] += 1
+            hip.ffn_swiglu(ga, up_, 12, dn, 14, xx, oo, mm, H, F)
+        run()
+        us = timed(run, max(8, steps // 2))
+        byts = 2 * F * row_bytes(12, H) + H * row_bytes(14, F) + 2 * mm * H * 4
+        flops = 2 * mm * (2 * F * H + H * F)
+        desc = f"dense FFN M={mm}: gate/up Q4_K {H}->{F}, SwiGLU, down Q6_K {F}->{H}, rotating over {copies} weight sets"
+        if args.no_cpu:
+            sec, sample = None, None
+        else:
+            Fc = F // 8  # an eighth of the intermediate size: an eighth of every matrix
+            hg, hu = random_weight(12, Fc, H, seed=1), random_weight(12, Fc, H, seed=2)
+            hd = random_weight(14, H, Fc, seed=3)
+            hx = random_activations(mm, H, seed=4)
+            sec, creps, cdt = cpu_time(lambda: cref.ffn_swiglu(hg, hu, 12, hd, 14, hx, mm, H, Fc, acc=cref.ACC_F32, threads=threads))
+            sec *= 8.0
+            sample = f"{creps} passes at an eighth of the intermediate size ({Fc}) in {cdt:.1f} s, scaled by 8"
     elif name.startswith("gather_"):
         # Op::QuantGather: 2048 token ids (a prefill) into a 32000 x 4096 embedding table;
         # algorithmic bytes = the looked-up rows' block bytes + the ids in, 4 bytes per element out
@@ -310,7 +350,7 @@ def main():
     ap.add_argument("--no-context", action="store_true",
                     help="skip the cache-resident and streaming-read context runs (profiling: only the timed kernel launches)")
     ap.add_argument("--workload", default="gemv_q4k",
-                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, lm_head_q6k, moe, "
+                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, lm_head_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
                          "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch plain device-to-device copies of one 33 MB weight buffer (counter calibration)")
@@ -347,11 +387,19 @@ def main():
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
     def timed(batch):
-        torch.cuda.synchronize()
-        start.record()
-        hip.quantized_matmul_batch(batch)
-        stop.record()
-        torch.cuda.synchronize()
+        # The launches are enqueued by host code that allocates Python objects; a full pass of
+        # Python's cyclic garbage collector in the middle of that (tens of ms with torch
+        # loaded) would starve the GPU and be counted as kernel time.
+        gc.collect()
+        gc.disable()
+        try:
+            torch.cuda.synchronize()
+            start.record()
+            hip.quantized_matmul_batch(batch)
+            stop.record()
+            torch.cuda.synchronize()
+        finally:
+            gc.enable()
         return start.elapsed_time(stop)  # ms
 
     if args.copy_probe:

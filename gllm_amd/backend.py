@@ -95,6 +95,8 @@ def load_library() -> C.CDLL:
     L.gllmq_moe_matvec.argtypes = [vp, vp, u32, vp, u32, vp, vp, sz, sz, sz, sz, sz, vp, vp, vp, C.c_int, vp]
     L.gllmq_quant_gather.restype = C.c_int
     L.gllmq_quant_gather.argtypes = [vp, vp, sz, u32, sz, sz, vp, sz, C.c_float, vp, vp]
+    L.gllmq_ffn_swiglu.restype = C.c_int
+    L.gllmq_ffn_swiglu.argtypes = [vp, vp, vp, sz, u32, vp, sz, u32, vp, vp, sz, sz, sz, C.c_int, vp]
     L.gllmq_argmax.restype = C.c_int
     L.gllmq_argmax.argtypes = [vp, vp, sz, sz, sz, vp, vp, vp]
     L.gllmq_stream_read.restype = C.c_int
@@ -113,7 +115,7 @@ EXPORTED_SYMBOLS = [
     "gllmq_init", "gllmq_destroy", "gllmq_last_error", "gllmq_status_string", "gllmq_version",
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
-    "gllmq_moe_matvec", "gllmq_argmax", "gllmq_quant_gather", "gllmq_stream_read", "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
+    "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_quant_gather", "gllmq_stream_read", "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
 ]
 
 
@@ -258,6 +260,26 @@ class HipBackend:
                                           1.0 if scale is None else float(scale), output.data_ptr(), self._stream())
         if rc != OK:
             self._raise(rc, "quant_gather")
+
+    def ffn_swiglu(self, gate, up, dtype_gate_up, down, dtype_down, x, out, m: int, hidden: int, ffn: int,
+                   relu_gate: bool = False) -> None:
+        """Dense feed-forward block on device tensors: ``out = (silu(x gate^T) * (x up^T)) down^T``;
+        ``gate`` and ``up`` are ``[ffn x hidden]`` blocks of ``dtype_gate_up`` (``up`` may be the second
+        half of one stacked tensor), ``down`` is ``[hidden x ffn]`` of ``dtype_down``."""
+        for t in (gate, up, down, x, out):
+            if not (_is_torch(t) and t.is_cuda):
+                raise OtherError("ffn_swiglu: tensors must live on the GPU")
+        if x.dtype != self._torch.float32 or out.dtype != self._torch.float32:
+            raise OtherError("ffn_swiglu: x and out must be f32")
+        if x.numel() < m * hidden or out.numel() < m * hidden:
+            raise OtherError("ffn_swiglu: x/out shorter than m * hidden")
+        gb, ub = gate.numel() * gate.element_size(), up.numel() * up.element_size()
+        rc = self._lib.gllmq_ffn_swiglu(self._ctx, gate.data_ptr(), up.data_ptr(), min(gb, ub), _dtype_id(dtype_gate_up),
+                                        down.data_ptr(), down.numel() * down.element_size(), _dtype_id(dtype_down),
+                                        x.data_ptr(), out.data_ptr(), m, hidden, ffn, 1 if relu_gate else 0,
+                                        self._stream())
+        if rc != OK:
+            self._raise(rc, "ffn_swiglu")
 
     def argmax(self, logits, token, value=None) -> None:
         """Op::Argmax with the semantics of the reference's ``argmax_token``: ``token[r]`` = index of

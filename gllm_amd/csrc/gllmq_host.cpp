@@ -102,11 +102,11 @@ int mm8_kind(uint32_t dtype)
 
 // Bytes of LDS the int8 matrix-core kernels need: Q6_K keeps 16 sub-block sums per block
 // instead of 8, Q8_0 none, and the weight stage of a wave differs by format.
-uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs, int kind = MM8_Q4K)
+uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs, int kind = MM8_Q4K, bool glu = false)
 {
     const uint32_t stage = kind == MM8_Q6K ? gq::MM8Q6_STAGE_BYTES : kind == MM8_Q8_0 ? gq::MM8Q8_STAGE_BYTES
                          : kind == MM8_Q5K ? gq::Mm8Format<1>::STAGE : gq::Mm8Format<0>::STAGE;
-    return gq::mm8_lds_layout(groups, m, pairs, kind == MM8_Q6K ? 16u : kind == MM8_Q8_0 ? 0u : 8u, stage).total;
+    return gq::mm8_lds_layout(groups, m, pairs, kind == MM8_Q6K ? 16u : kind == MM8_Q8_0 ? 0u : 8u, stage, glu ? 4u : 2u).total;
 }
 
 } // namespace
@@ -116,6 +116,14 @@ struct gllmq_ctx {
     hipModule_t module = nullptr;
     hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
     hipFunction_t gather[kNumFormats][2] = {};  // quantized embedding lookup [format][0 = scalar stores, 1 = float4 stores]
+    // gated form of the int8 kernels (gate and up rows in one launch, act(gate) * up out):
+    // [0 = Q4_K, 1 = Q5_K][pairs 1,2,4][early steps 1,2,4] and the register-operand variants
+    hipFunction_t mm8_glu[2][3][3] = {};
+    hipFunction_t mm8_glu_areg[2][2][3][2] = {};
+    hipFunction_t glu_act = nullptr;            // act(gate) * up as a kernel of its own
+    bool ffn_fused = true;                      // GLLMQ_FFN_FUSED=0: gllmq_ffn_swiglu never uses the gated kernels
+    void *ffn_scratch = nullptr;                // gate/up results and the gated activations of gllmq_ffn_swiglu
+    size_t ffn_scratch_bytes = 0;
     hipFunction_t argmax_part = nullptr, argmax_final = nullptr;
     uint64_t *argmax_keys = nullptr;            // [ARGMAX_MAX_ROWS][ARGMAX_MAX_PARTS] scratch of gllmq_argmax
     hipFunction_t dequant_wave = nullptr;       // Q4_K with 16-byte aligned blocks and outputs: one block per wave
@@ -309,13 +317,19 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
 // its rows' digit planes in LDS and reads the weights once).  Returns -1 when the shape does
 // not fit the kernel (LDS for the prepared activations, alignment), so that the caller
 // takes the GEMV kernels.
+// `w2` != null selects the gated form: `w` holds the n gate rows, `w2` the n up rows, and
+// y = act(gate . x) * (up . x) (Q4_K and Q5_K, one pass only).
 int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
-            size_t k, bool act_bf16, void *stream, bool one_pass_only = false)
+            size_t k, bool act_bf16, void *stream, bool one_pass_only = false, const uint8_t *w2 = nullptr,
+            bool glu_relu = false)
 {
     const int kind = mm8_kind(f.dtype);
     if (!ctx->use_mm8 || kind < 0) return -1;
+    const bool glu = w2 != nullptr;
+    if (glu && kind != MM8_Q4K && kind != MM8_Q5K) return -1;
+    if (glu) one_pass_only = true;
     if (kind == MM8_Q6K && (ctx->mm8_q6k_min_m == 0 || m < ctx->mm8_q6k_min_m)) return -1;
-    if (kind == MM8_Q5K && (ctx->mm8_q5k_min_m == 0 || m < ctx->mm8_q5k_min_m)) return -1;
+    if (kind == MM8_Q5K && !glu && (ctx->mm8_q5k_min_m == 0 || m < ctx->mm8_q5k_min_m)) return -1;
     if (kind == MM8_Q8_0 && (ctx->mm8_q8_0_min_m == 0 || m < ctx->mm8_q8_0_min_m)) return -1;
     if (kind == MM8_Q8_0 && k < 256) return -1; // its fetch window is one whole group of 8 blocks
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
@@ -323,7 +337,7 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     // Rows per pass: as many as the prepared activations leave room for in the 160 KiB of LDS.
     auto pairs_for = [](uint32_t rows) { return rows <= 2 ? 1u : (rows <= 4 ? 2u : 4u); };
     uint32_t rows_per_pass = static_cast<uint32_t>(std::min<size_t>(m, 8));
-    while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass), kind) > 160u * 1024u)
+    while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass), kind, glu) > 160u * 1024u)
         --rows_per_pass;
     if (rows_per_pass == 0) return -1;
     if (one_pass_only && rows_per_pass < m) return -1;
@@ -331,8 +345,10 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(rows_per_pass, m - m0));
         const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
         const uint32_t pairs = 1u << pi;
-        const uint32_t lds = mm8_lds_bytes(groups, mm, pairs, kind);
+        const uint32_t lds = mm8_lds_bytes(groups, mm, pairs, kind, glu);
         Mm8Params P{};
+        P.w2 = w2;
+        P.glu_relu = glu_relu ? 1u : 0u;
         P.w = w;
         P.x = x + m0 * k;
         P.y = y + m0 * n;
@@ -350,11 +366,13 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         const uint32_t ppt = (groups + 7u) / 8u, steps = ((ppt + 1u) / 2u) * mm;
         int ei = steps <= 1 ? 0 : (steps <= 2 ? 1 : 2);
         while (ei < 2 && !ctx->mm8[kind][pi][ei]) ++ei; // not every (pairs, early) pair is built
+        const int gi = kind == MM8_Q5K ? 1 : 0;
         uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
         if (ctx->tune_mm8_grid) grid = std::min<uint32_t>(P.tiles, ctx->tune_mm8_grid);
         P.grid = grid;
-        hipFunction_t fn = ctx->mm8[kind][pi][ei];
-        if (pi <= 1 && ppt <= 2 && ctx->mm8_areg_on) fn = ctx->mm8_areg[kind][pi][ei][ppt - 1];
+        hipFunction_t fn = glu ? ctx->mm8_glu[gi][pi][ei] : ctx->mm8[kind][pi][ei];
+        if (pi <= 1 && ppt <= 2 && ctx->mm8_areg_on)
+            fn = glu ? ctx->mm8_glu_areg[gi][pi][ei][ppt - 1] : ctx->mm8_areg[kind][pi][ei][ppt - 1];
         int rc = launch(ctx, fn, grid, 512, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }
@@ -446,6 +464,24 @@ int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
         }
     }
     return GLLMQ_OK;
+}
+
+// One quantized matmul on validated arguments: the kernel family by format, rows and shape.
+int dispatch_matmul(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
+                    size_t k, bool bf16, void *stream)
+{
+    int rc = run_mmf(ctx, f, w, x, y, m, n, k, bf16, stream);
+    if (rc >= 0) return rc;
+    // up to 8 rows: the int8 kernel when one pass over the weights does it, else the GEMM
+    rc = run_mm8(ctx, f, w, x, y, m, n, k, bf16, stream, true);
+    if (rc >= 0) return rc;
+    if (ctx->mmf_small_min_m > 0) {
+        rc = run_mmf(ctx, f, w, x, y, m, n, k, bf16, stream, ctx->mmf_small_min_m);
+        if (rc >= 0) return rc;
+    }
+    rc = run_mm8(ctx, f, w, x, y, m, n, k, bf16, stream);
+    if (rc >= 0) return rc;
+    return run_gemv(ctx, f, w, x, y, m, n, k, bf16, stream);
 }
 
 } // namespace
@@ -587,7 +623,16 @@ int gllmq_init(gllmq_ctx **out, int device)
                     snprintf(name, sizeof name, "gq_mm8_%s_%s_a%d", kMm8Format[q], k.tag, a);
                     rc = get_function(ctx, &ctx->mm8_areg[q][k.pi][k.ei][a - 1], name);
                 }
+                if (q != MM8_Q4K && q != MM8_Q5K) continue;
+                const int gi = q == MM8_Q5K ? 1 : 0;
+                snprintf(name, sizeof name, "gq_mm8_glu_%s_%s", kMm8Format[q], k.tag);
+                if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_glu[gi][k.pi][k.ei], name);
+                for (int a = 1; a <= 2 && k.pi <= 1 && rc == GLLMQ_OK; ++a) {
+                    snprintf(name, sizeof name, "gq_mm8_glu_%s_%s_a%d", kMm8Format[q], k.tag, a);
+                    rc = get_function(ctx, &ctx->mm8_glu_areg[gi][k.pi][k.ei][a - 1], name);
+                }
             }
+        if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->glu_act, "gq_glu_act");
     }
     if (rc != GLLMQ_OK) {
         fprintf(stderr, "gllmq_init: %s\n", ctx->err.c_str());
@@ -599,6 +644,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (const char *v = getenv("GLLMQ_GEMV_F32")) ctx->gemv_f32 = (v[0] == '1');
     if (const char *v = getenv("GLLMQ_MM8")) ctx->use_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MMF")) ctx->use_mmf = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_FFN_FUSED")) ctx->ffn_fused = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MMF_SMALL_MIN_M")) ctx->mmf_small_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
     auto tune = [](const char *name) { const char *v = getenv(name); return v ? static_cast<uint32_t>(std::max(0, atoi(v))) : 0u; };
     ctx->tune_mm8_grid = tune("GLLMQ_MM8_GRID");
@@ -627,6 +673,7 @@ void gllmq_destroy(gllmq_ctx *ctx)
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->identity_rows) (void)hipFree(ctx->identity_rows);
     if (ctx->argmax_keys) (void)hipFree(ctx->argmax_keys);
+    if (ctx->ffn_scratch) (void)hipFree(ctx->ffn_scratch);
     if (ctx->mmf_partial) (void)hipFree(ctx->mmf_partial);
     if (ctx->module) (void)hipModuleUnload(ctx->module);
     delete ctx;
@@ -736,18 +783,85 @@ int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, con
     const bool bf16 = act_mode == GLLMQ_ACT_BF16;
     if (bf16 && ctx->gemv_f32)
         return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "quantized_matmul: bf16 activations are not built for GLLMQ_GEMV_F32=1");
-    rc = run_mmf(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
+    return dispatch_matmul(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
+}
+
+int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_t gate_up_bytes_each, uint32_t dtype_gate_up,
+                     const void *down_w, size_t down_bytes, uint32_t dtype_down, const float *x, float *out, size_t m,
+                     size_t hidden, size_t ffn, int relu_gate, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    const Format *fg = find_format(dtype_gate_up), *fd = find_format(dtype_down);
+    if (!fg || !fd)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
+                    "ffn_swiglu: ggml dtype %u / %u is not covered (supported: Q8_0=8, Q4_K=12, Q5_K=13, Q6_K=14)",
+                    dtype_gate_up, dtype_down);
+    if (m == 0 || hidden == 0) return GLLMQ_OK;
+    if (ffn == 0) return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "ffn_swiglu: ffn = 0");
+    if (!up_w) return fail(ctx, GLLMQ_ERR_INVALID, "ffn_swiglu: NULL device pointer");
+    // the three matrices are checked as the matmuls they are (the intermediate buffers stand in
+    // for the activations that are not the caller's)
+    int rc = check_matmul_args(ctx, fg, gate_w, gate_up_bytes_each, x, out, dtype_gate_up, m, ffn, hidden);
     if (rc >= 0) return rc;
-    // up to 8 rows: the int8 kernel when one pass over the weights does it, else the GEMM
-    rc = run_mm8(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream, true);
+    rc = check_matmul_args(ctx, fg, up_w, gate_up_bytes_each, x, out, dtype_gate_up, m, ffn, hidden);
     if (rc >= 0) return rc;
-    if (ctx->mmf_small_min_m > 0) {
-        rc = run_mmf(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream, ctx->mmf_small_min_m);
-        if (rc >= 0) return rc;
+    rc = check_matmul_args(ctx, fd, down_w, down_bytes, x, out, dtype_down, m, hidden, ffn);
+    if (rc >= 0) return rc;
+    if (ffn > 0x7FFFFFFFu / 2u) return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "ffn_swiglu: ffn exceeds 2^30-1");
+
+    // scratch: h [m][ffn], then gate/up results [m][2 ffn] for the form with three steps
+    const size_t h_bytes = ((m * ffn * sizeof(float)) + 255) & ~size_t(255);
+    const size_t need = h_bytes + m * 2 * ffn * sizeof(float);
+    {
+        std::lock_guard<std::mutex> guard(ctx->workspace_mutex);
+        GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
+        if (ctx->ffn_scratch_bytes < need) {
+            if (ctx->ffn_scratch) {
+                GLLMQ_HIP(ctx, hipDeviceSynchronize()); // earlier calls may still be using it
+                GLLMQ_HIP(ctx, hipFree(ctx->ffn_scratch));
+                ctx->ffn_scratch = nullptr;
+                ctx->ffn_scratch_bytes = 0;
+            }
+            GLLMQ_HIP(ctx, hipMalloc(&ctx->ffn_scratch, need));
+            ctx->ffn_scratch_bytes = need;
+        }
     }
-    rc = run_mm8(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
-    if (rc >= 0) return rc;
-    return run_gemv(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
+    float *h = static_cast<float *>(ctx->ffn_scratch);
+    float *gu = reinterpret_cast<float *>(static_cast<uint8_t *>(ctx->ffn_scratch) + h_bytes);
+    const uint8_t *gw = static_cast<const uint8_t *>(gate_w), *uw = static_cast<const uint8_t *>(up_w);
+
+    // gate and up in one launch with the activation in its epilogue (Q4_K / Q5_K, up to 8 rows)
+    rc = -1;
+    if (ctx->ffn_fused && m <= 8) rc = run_mm8(ctx, *fg, gw, x, h, m, ffn, hidden, false, stream, true, uw, relu_gate != 0);
+    if (rc > 0) return rc;
+    if (rc < 0) {
+        // three steps: the two products (one matmul when the up rows follow the gate rows in
+        // memory), the activation, the down projection
+        const size_t rb = gllmq_row_bytes(dtype_gate_up, hidden);
+        const bool stacked = uw == gw + ffn * rb;
+        gq::GluActParams A{};
+        A.h = h;
+        A.m = static_cast<uint32_t>(m);
+        A.ffn = static_cast<uint32_t>(ffn);
+        A.relu_gate = relu_gate ? 1u : 0u;
+        if (stacked) {
+            rc = dispatch_matmul(ctx, *fg, gw, x, gu, m, 2 * ffn, hidden, false, stream);
+            A.g = gu;
+            A.u = gu + ffn;
+            A.ld = static_cast<uint32_t>(2 * ffn);
+        } else {
+            rc = dispatch_matmul(ctx, *fg, gw, x, gu, m, ffn, hidden, false, stream);
+            if (rc == GLLMQ_OK) rc = dispatch_matmul(ctx, *fg, uw, x, gu + m * ffn, m, ffn, hidden, false, stream);
+            A.g = gu;
+            A.u = gu + m * ffn;
+            A.ld = static_cast<uint32_t>(ffn);
+        }
+        if (rc != GLLMQ_OK) return rc;
+        rc = launch2d(ctx, ctx->glu_act, static_cast<uint32_t>((ffn + 255) / 256),
+                      static_cast<uint32_t>(std::min<size_t>(m, 65535)), 256, 0, stream, &A, sizeof A);
+        if (rc != GLLMQ_OK) return rc;
+    }
+    return dispatch_matmul(ctx, *fd, static_cast<const uint8_t *>(down_w), h, out, m, hidden, ffn, false, stream);
 }
 
 int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y,

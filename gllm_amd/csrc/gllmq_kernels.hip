@@ -18,4 +18,5 @@
 #include "mmf_q8_0.hip.inc"
 #include "moe.hip.inc"
 #include "argmax.hip.inc"
+#include "ffn.hip.inc"
 #include "probe.hip.inc"

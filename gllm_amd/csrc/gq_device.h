@@ -40,6 +40,14 @@ __device__ __forceinline__ T load_unaligned(const void *p)
     return v;
 }
 
+// Gate activation of the feed-forward block: SiLU, behind a ReLU when `relu`
+// (reference: Op::SwiGlu, silu(gate) * up, src/arch/auto_graph_fragments/build_graph.inc.rs:1977-1984).
+__device__ __forceinline__ float glu_act(float g, bool relu)
+{
+    if (relu) g = g > 0.0f ? g : 0.0f;
+    return g / (1.0f + expf(-g));
+}
+
 // (sc, m) pair j of the 12-byte field held as three little-endian dwords s0,s1,s2
 // (bytes 0-3, 4-7, 8-11).  Reference: quant-kquant-iq-proprietary.md:45-50.
 __device__ __forceinline__ void scale_min_k4(int j, uint32_t s0, uint32_t s1, uint32_t s2,

@@ -97,6 +97,24 @@ int gllmq_quant_gather(gllmq_ctx *ctx, const void *table_dev, size_t table_bytes
                        size_t vocab, size_t hidden, const uint32_t *ids_dev, size_t count, float scale,
                        float *out_dev, void *stream);
 
+/* ---- Dense feed-forward block: gate/up projections, SwiGLU, down projection -------------
+ * Replaces the op sequence the reference emits per layer (QuantGemm gate_proj, QuantGemm
+ * up_proj, Op::SwiGlu, QuantGemm down_proj: src/arch/auto_graph_fragments/
+ * build_graph.inc.rs:1957-1995; formula down(silu(gate x) * (up x)), SPEC 04-OPERATORS.md:114):
+ *   out[m x hidden] = ( act(x . Wgate^T) * (x . Wup^T) ) . Wdown^T,   act = SiLU
+ * (relu_gate != 0: SiLU behind a ReLU).  Wgate and Wup are [ffn x hidden] of dtype_gate_up,
+ * each of gate_up_bytes_each bytes; Wdown is [hidden x ffn] of dtype_down; x and out are f32.
+ * Q4_K / Q5_K gate and up with up to 8 rows run as ONE launch of the int8 matrix-core kernel
+ * with the activation in its epilogue (a workgroup runs the gate tile and the up tile of a
+ * row range back to back); other shapes run the two products (one matmul when the up rows
+ * follow the gate rows in memory), an activation kernel and the down projection, each with
+ * the kernels gllmq_quantized_matmul would pick.  Intermediates live in the context: calls on
+ * one context must not overlap in time. */
+int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_dev, const void *up_dev, size_t gate_up_bytes_each,
+                     uint32_t dtype_gate_up, const void *down_dev, size_t down_bytes, uint32_t dtype_down,
+                     const float *x_dev, float *out_dev, size_t m, size_t hidden, size_t ffn, int relu_gate,
+                     void *stream);
+
 /* ---- Op::Argmax: greedy token choice behind the lm_head matmul -----------------------
  * Replaces the graph op of src/arch/auto_graph_fragments/build_graph.inc.rs:2661 with the
  * semantics of argmax_token (src/engine/executor_step.rs:48-55; its unit tests :2191-2325):

@@ -133,6 +133,20 @@ public:
                     "quant_gather");
     }
 
+    // Dense feed-forward block over device buffers: gate_proj, up_proj, Op::SwiGlu, down_proj
+    // (src/arch/auto_graph_fragments/build_graph.inc.rs:1957-1995).
+    BackendError ffn_swiglu_device(const void *gate_dev, const void *up_dev, size_t gate_up_bytes_each, QuantType t_gate_up,
+                                   const void *down_dev, size_t down_bytes, QuantType t_down, const float *x_dev,
+                                   float *out_dev, size_t m, size_t hidden, size_t ffn, bool relu_gate = false,
+                                   void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_ffn_swiglu(ctx_, gate_dev, up_dev, gate_up_bytes_each, static_cast<uint32_t>(t_gate_up), down_dev,
+                                     down_bytes, static_cast<uint32_t>(t_down), x_dev, out_dev, m, hidden, ffn,
+                                     relu_gate ? 1 : 0, stream),
+                    "ffn_swiglu");
+    }
+
     // Op::Argmax over device logits [rows][ld] (argmax_token, src/engine/executor_step.rs:48-55).
     BackendError argmax_device(const float *logits_dev, size_t rows, size_t n, size_t ld, uint32_t *token_dev,
                                float *value_dev = nullptr, void *stream = nullptr) const

@@ -53,6 +53,8 @@ def lib() -> C.CDLL:
         L.gq_dequantize.argtypes = [u8p, sz, f32p, sz, C.c_uint32]
         L.gq_quant_gather.restype = C.c_int
         L.gq_quant_gather.argtypes = [u8p, C.c_uint32, sz, sz, u32p, sz, C.c_float, C.c_int, f32p]
+        L.gq_ffn_swiglu.restype = C.c_int
+        L.gq_ffn_swiglu.argtypes = [u8p, u8p, C.c_uint32, u8p, C.c_uint32, f32p, f32p, sz, sz, sz, C.c_int, C.c_int, C.c_int]
         L.gq_argmax_token.restype = C.c_int64
         L.gq_argmax_token.argtypes = [f32p, sz]
         L.gq_quantized_matmul.restype = C.c_int
@@ -133,6 +135,21 @@ def dequantize(raw, dtype: int, n_out: int | None = None) -> np.ndarray:
     rc = lib().gq_dequantize(_u8(b), b.size, _f32(out), n_out, dtype)
     if rc != OK:
         raise NotImplementedError(f"dequantize: rc={rc}")
+    return out
+
+
+def ffn_swiglu(gate, up, dtype_gu: int, down, dtype_dn: int, x, m: int, hidden: int, ffn: int,
+               relu_gate: bool = False, acc: int = 1, threads: int = 1) -> np.ndarray:
+    """Dense feed-forward block: (silu(x gate^T) * (x up^T)) down^T; ``acc`` as in quantized_matmul."""
+    g, u, d = _bytes_arr(gate), _bytes_arr(up), _bytes_arr(down)
+    xx = np.ascontiguousarray(x, np.float32).reshape(m, hidden)
+    out = np.zeros((m, hidden), np.float32)
+    rc = lib().gq_ffn_swiglu(_u8(g), _u8(u), dtype_gu, _u8(d), dtype_dn, _f32(xx), _f32(out), m, hidden, ffn,
+                             1 if relu_gate else 0, acc, threads)
+    if rc == 1:
+        raise NotImplementedError(f"ffn_swiglu: ggml dtype {dtype_gu}/{dtype_dn}")
+    if rc != OK:
+        raise ValueError(f"ffn_swiglu: rc={rc}")
     return out
 
 

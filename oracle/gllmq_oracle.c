@@ -508,3 +508,26 @@ int gq_moe_ffn(const uint8_t *gate_up, uint32_t t_gu, const uint8_t *down, uint3
     free(o);
     return GQ_OK;
 }
+
+/* Dense feed-forward block (src/arch/auto_graph_fragments/build_graph.inc.rs:1957-1995): the
+ * gate and up products, h = silu(gate) * up in f32 (Op::SwiGlu), the down product.  The
+ * products are gq_quantized_matmul's (same accumulation modes). */
+int gq_ffn_swiglu(const uint8_t *gate, const uint8_t *up, uint32_t t_gu, const uint8_t *down, uint32_t t_dn,
+                  const float *x, float *out, size_t m, size_t hidden, size_t ffn, int relu_gate, int acc, int threads)
+{
+    float *g = (float *)malloc(sizeof(float) * m * ffn * 2);
+    if (!g) return GQ_ERR_BAD_SHAPE;
+    float *u = g + m * ffn;
+    int rc = gq_quantized_matmul(gate, x, g, t_gu, m, ffn, hidden, acc, threads);
+    if (rc == GQ_OK) rc = gq_quantized_matmul(up, x, u, t_gu, m, ffn, hidden, acc, threads);
+    if (rc == GQ_OK) {
+        for (size_t i = 0; i < m * ffn; ++i) {
+            float gv = g[i];
+            if (relu_gate && !(gv > 0.0f)) gv = 0.0f;
+            g[i] = silu(gv) * u[i];
+        }
+        rc = gq_quantized_matmul(down, g, out, t_dn, m, hidden, ffn, acc, threads);
+    }
+    free(g);
+    return rc;
+}

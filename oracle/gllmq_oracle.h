@@ -36,6 +36,10 @@
  *                                         a value)
  *   gq_argmax_token                     : pinned by the reference's unit-test vectors
  *                                         (src/engine/executor_step.rs:2191-2325)
+ *   gq_ffn_swiglu                       : the formula down(silu(gate x) * (up x)) is the reference's
+ *                                         (04-OPERATORS.md:114); pinned against a float64 numpy
+ *                                         evaluation of it; the products inherit gq_quantized_matmul's
+ *                                         status
  *   gq_moe_ffn                          : PARITY UNPINNED beyond routing + combine rule
  *                                         (the reference's quantized expert template is
  *                                         unfinished, build_graph.inc.rs:2922-2942)
@@ -134,6 +138,11 @@ size_t gq_route(const float *logits, size_t tokens, size_t experts, size_t top_k
  * gate_up: per expert 2*ffn rows of dtype_gu over hidden (gate rows first, then up rows);
  * down:    per expert hidden rows of dtype_dn over ffn.
  * relu_gate != 0 applies max(g,0) before silu (BUG-KNOWLEDGE.md:1434-1440). */
+/* Dense feed-forward block: out[m x hidden] = (silu(x . gate^T) * (x . up^T)) . down^T; gate and up
+ * are [ffn x hidden] of dtype_gu, down is [hidden x ffn] of dtype_dn; relu_gate: ReLU ahead of the SiLU. */
+int gq_ffn_swiglu(const uint8_t *gate, const uint8_t *up, uint32_t dtype_gu, const uint8_t *down, uint32_t dtype_dn,
+                  const float *x, float *out, size_t m, size_t hidden, size_t ffn, int relu_gate, int acc, int threads);
+
 int gq_moe_ffn(const uint8_t *gate_up, uint32_t dtype_gu, const uint8_t *down, uint32_t dtype_dn,
                const float *x, float *out, size_t tokens, size_t hidden, size_t ffn,
                size_t experts, size_t top_k, const uint32_t *route_expert,

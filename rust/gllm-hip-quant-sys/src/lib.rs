@@ -59,6 +59,10 @@ extern "C" {
                             tokens: usize, hidden: usize, ffn: usize, experts: usize, top_k: usize,
                             route_expert_dev: *const u32, route_weight_dev: *const f32,
                             route_len_dev: *const u32, relu_gate: c_int, stream: *mut c_void) -> c_int;
+    pub fn gllmq_ffn_swiglu(ctx: *mut gllmq_ctx, gate_dev: *const c_void, up_dev: *const c_void,
+                            gate_up_bytes_each: usize, dtype_gate_up: u32, down_dev: *const c_void, down_bytes: usize,
+                            dtype_down: u32, x_dev: *const f32, out_dev: *mut f32, m: usize, hidden: usize,
+                            ffn: usize, relu_gate: c_int, stream: *mut c_void) -> c_int;
     pub fn gllmq_argmax(ctx: *mut gllmq_ctx, logits_dev: *const f32, rows: usize, n: usize, ld: usize,
                         token_dev: *mut u32, value_dev: *mut f32, stream: *mut c_void) -> c_int;
     pub fn gllmq_quant_gather(ctx: *mut gllmq_ctx, table_dev: *const c_void, table_bytes: usize, ggml_dtype: u32,
@@ -158,6 +162,20 @@ impl HipQuant {
                                       scale: Option<f32>, out: *mut f32, stream: *mut c_void) -> Result<(), QuantError> {
         self.check(gllmq_quant_gather(self.ctx, table, table_bytes, ggml_dtype, vocab_size, hidden_dim, ids, count,
                                       scale.unwrap_or(1.0), out, stream), "quant_gather")
+    }
+
+    /// The dense feed-forward block of a layer over device tensors (gate_proj, up_proj, `Op::SwiGlu`,
+    /// down_proj: src/arch/auto_graph_fragments/build_graph.inc.rs:1957-1995).
+    ///
+    /// # Safety
+    /// All pointers must be valid device allocations of the stated sizes on this context's device.
+    #[allow(clippy::too_many_arguments)]
+    pub unsafe fn ffn_swiglu_device(&self, gate: *const c_void, up: *const c_void, gate_up_bytes_each: usize,
+                                    dtype_gate_up: u32, down: *const c_void, down_bytes: usize, dtype_down: u32,
+                                    x: *const f32, out: *mut f32, m: usize, hidden: usize, ffn: usize,
+                                    stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_ffn_swiglu(self.ctx, gate, up, gate_up_bytes_each, dtype_gate_up, down, down_bytes, dtype_down,
+                                    x, out, m, hidden, ffn, 0, stream), "ffn_swiglu")
     }
 
     /// `Op::Argmax` over device logits `[rows][ld]` (argmax_token, src/engine/executor_step.rs:48-55):

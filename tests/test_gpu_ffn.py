@@ -1,0 +1,128 @@
+"""GPU parity of the dense feed-forward block (gllmq_ffn_swiglu through the C ABI) against the
+oracle's float64-accumulated evaluation: rel-L2 <= 1e-4 and |err| <= 1e-3 max|y|, the matmul bar."""
+import numpy as np
+import pytest
+
+from gllm_amd.synth import random_activations, random_weight
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+ALL = [Q8_0, Q4_K, Q5_K, Q6_K]
+GUARD = 4096
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from gllm_amd.backend import HipBackend
+    return HipBackend(0)
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+    return torch
+
+
+def dev_bytes(torch, host):
+    flat = torch.from_numpy(np.asarray(host).view(np.uint8).reshape(-1))
+    buf = torch.full((flat.numel() + GUARD,), 0xFF, dtype=torch.uint8, device="cuda")
+    buf[:flat.numel()] = flat.cuda()
+    return buf[:flat.numel()]
+
+
+def run_ffn(hip, torch, gate, up, t_gu, down, t_dn, x, m, hidden, ffn, relu=False, stacked=False):
+    if stacked:  # up rows right behind the gate rows, as one [2 ffn x hidden] tensor
+        both = dev_bytes(torch, np.concatenate([np.asarray(gate).view(np.uint8).reshape(-1),
+                                                np.asarray(up).view(np.uint8).reshape(-1)]))
+        half = both.numel() // 2
+        gd, ud = both[:half], both[half:]
+    else:
+        gd, ud = dev_bytes(torch, gate), dev_bytes(torch, up)
+    dd = dev_bytes(torch, down)
+    xbuf = torch.full((m * hidden + GUARD,), float("nan"), dtype=torch.float32, device="cuda")
+    xbuf[:m * hidden] = torch.from_numpy(np.ascontiguousarray(x, np.float32).reshape(-1)).cuda()
+    obuf = torch.full((m * hidden + GUARD,), float("nan"), dtype=torch.float32, device="cuda")
+    obuf[m * hidden:] = 7.0
+    hip.ffn_swiglu(gd, ud, t_gu, dd, t_dn, xbuf[:m * hidden], obuf[:m * hidden], m, hidden, ffn, relu_gate=relu)
+    torch.cuda.synchronize()
+    assert bool(torch.all(obuf[m * hidden:] == 7.0)), "write past the end of the output"
+    return obuf[:m * hidden].cpu().numpy().reshape(m, hidden)
+
+
+def check(got, want, what):
+    got, want = got.astype(np.float64), want.astype(np.float64)
+    rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-300)
+    worst = np.abs(got - want).max() / max(np.abs(want).max(), 1e-300)
+    assert rel <= 1e-4 and worst <= 1e-3, f"{what}: rel_l2={rel:.3e} max_err/max|y|={worst:.3e}"
+
+
+@pytest.mark.parametrize("t_gu", ALL)
+@pytest.mark.parametrize("t_dn", [Q6_K, Q4_K, Q8_0])
+def test_ffn_all_format_pairs(hip, torch, oracle, t_gu, t_dn):
+    hidden, ffn = 1024, 1536
+    gate, up = random_weight(t_gu, ffn, hidden, seed=1), random_weight(t_gu, ffn, hidden, seed=2)
+    down = random_weight(t_dn, hidden, ffn, seed=3)
+    for m in (1, 2, 5, 8, 9, 33):
+        print(f"ffn gate/up={t_gu} down={t_dn} m={m}", flush=True)
+        x = random_activations(m, hidden, seed=10 + m)
+        want = oracle.ffn_swiglu(gate, up, t_gu, down, t_dn, x, m, hidden, ffn, acc=oracle.ACC_F64, threads=4)
+        got = run_ffn(hip, torch, gate, up, t_gu, down, t_dn, x, m, hidden, ffn, stacked=(m % 2 == 1))
+        check(got, want, f"gu={t_gu} dn={t_dn} m={m}")
+
+
+@pytest.mark.parametrize("t_gu", [Q4_K, Q5_K])
+def test_ffn_ragged_shapes_and_relu_gate(hip, torch, oracle, t_gu):
+    # ffn not a multiple of 32 (a partial last tile in both halves), hidden with 2 and 3 passes per tile
+    for hidden, ffn, m, relu in [(2560, 1000, 1, False), (4096, 776, 2, True), (6144, 520, 4, False), (512, 33, 7, True)]:
+        print(f"ffn ragged gate/up={t_gu} hidden={hidden} ffn={ffn} m={m} relu={relu}", flush=True)
+        gate, up = random_weight(t_gu, ffn, hidden, seed=ffn), random_weight(t_gu, ffn, hidden, seed=ffn + 1)
+        down = random_weight(Q8_0, hidden, ffn, seed=ffn + 2)
+        x = random_activations(m, hidden, seed=m)
+        want = oracle.ffn_swiglu(gate, up, t_gu, down, Q8_0, x, m, hidden, ffn, relu_gate=relu, acc=oracle.ACC_F64, threads=4)
+        got = run_ffn(hip, torch, gate, up, t_gu, down, Q8_0, x, m, hidden, ffn, relu=relu)
+        check(got, want, f"gu={t_gu} hidden={hidden} ffn={ffn} m={m}")
+
+
+def test_ffn_layer_shape(hip, torch, oracle):
+    """The decode shape of the layer mix: Q4_K gate/up 4096 -> 14336, Q6_K down 14336 -> 4096."""
+    hidden, ffn = 4096, 14336
+    print("ffn 4096/14336", flush=True)
+    gate, up = random_weight(Q4_K, ffn, hidden, seed=21), random_weight(Q4_K, ffn, hidden, seed=22)
+    down = random_weight(Q6_K, hidden, ffn, seed=23)
+    for m in (1, 16):
+        x = random_activations(m, hidden, seed=24 + m)
+        want = oracle.ffn_swiglu(gate, up, Q4_K, down, Q6_K, x, m, hidden, ffn, acc=oracle.ACC_F64, threads=16)
+        got = run_ffn(hip, torch, gate, up, Q4_K, down, Q6_K, x, m, hidden, ffn, stacked=True)
+        check(got, want, f"layer shape m={m}")
+
+
+def test_ffn_three_step_form(torch, oracle, monkeypatch):
+    """GLLMQ_FFN_FUSED=0: the two products, the activation kernel, the down projection."""
+    from gllm_amd.backend import HipBackend
+    monkeypatch.setenv("GLLMQ_FFN_FUSED", "0")
+    hip2 = HipBackend(0)
+    hidden, ffn = 1024, 800
+    gate, up = random_weight(Q4_K, ffn, hidden, seed=1), random_weight(Q4_K, ffn, hidden, seed=2)
+    down = random_weight(Q6_K, hidden, ffn, seed=3)
+    for m, stacked in [(1, True), (1, False), (4, True), (70, False)]:
+        print(f"ffn three steps m={m} stacked={stacked}", flush=True)
+        x = random_activations(m, hidden, seed=m)
+        want = oracle.ffn_swiglu(gate, up, Q4_K, down, Q6_K, x, m, hidden, ffn, acc=oracle.ACC_F64, threads=4)
+        got = run_ffn(hip2, torch, gate, up, Q4_K, down, Q6_K, x, m, hidden, ffn, stacked=stacked)
+        check(got, want, f"three steps m={m}")
+
+
+def test_ffn_argument_errors(hip, torch):
+    from gllm_amd.backend import BackendError, Unimplemented
+    print("ffn errors", flush=True)
+    w = torch.zeros(144 * 64, dtype=torch.uint8, device="cuda")
+    x = torch.zeros(256, device="cuda")
+    out = torch.full((256,), 7.0, device="cuda")
+    with pytest.raises(Unimplemented):
+        hip.ffn_swiglu(w, w, 2, w, Q4_K, x, out, 1, 256, 256)      # Q4_0 gate/up
+    with pytest.raises(BackendError):
+        hip.ffn_swiglu(w[:100], w, Q4_K, w, Q4_K, x, out, 1, 256, 64)  # gate shorter than 64 rows
+    hip.ffn_swiglu(w, w, Q4_K, w, Q4_K, x, out, 0, 256, 64)       # no rows: nothing written
+    torch.cuda.synchronize()
+    assert bool(torch.all(out == 7.0))
