@@ -143,6 +143,8 @@ struct gllmq_ctx {
     uint32_t mm8_q8_0_min_m = 3;                // the same for Q8_0 (GLLMQ_MM8_Q8_0_MIN_M)
     bool moe_mm8 = true;                        // GLLMQ_MOE_MM8=0 keeps the MoE expert rows on the GEMV kernels
     bool moe_mm8_q6k = true;                    // GLLMQ_MOE_MM8_Q6K=0 keeps Q6_K expert rows there
+    bool moe_glu = true;                        // GLLMQ_MOE_GLU=0: gate/up results to memory, activation as a kernel of its own
+    hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
     bool moe_mm8_rows = true;                   // GLLMQ_MOE_MM8_ROWS=0: no wave-per-tile kernel for short Q6_K rows
     // development overrides of launch shapes, read once at init (0 = the library's own choice):
     // GLLMQ_MM8_GRID, GLLMQ_MMF_KSPLIT, GLLMQ_MMF_ROWS, GLLMQ_MOE_JOB_WAVES, GLLMQ_MOE_SLICES
@@ -596,6 +598,10 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[2][0], "gq_moe_mm8_q5k_a1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[2][1], "gq_moe_mm8_q5k_a2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_q6k_rows, "gq_moe_mm8_q6k_rows");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_glu_fn[MM8_Q4K][0], "gq_moe_mm8_glu_q4k_a1");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_glu_fn[MM8_Q4K][1], "gq_moe_mm8_glu_q4k_a2");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_glu_fn[MM8_Q5K][0], "gq_moe_mm8_glu_q5k_a1");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_glu_fn[MM8_Q5K][1], "gq_moe_mm8_glu_q5k_a2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->dequant_wave, "gq_dequant_q4k_wave");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->argmax_part, "gq_argmax_part");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->argmax_final, "gq_argmax_final");
@@ -659,6 +665,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (const char *v = getenv("GLLMQ_MOE_MM8")) ctx->moe_mm8 = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MOE_MM8_Q6K")) ctx->moe_mm8_q6k = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_MOE_MM8_ROWS")) ctx->moe_mm8_rows = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_MOE_GLU")) ctx->moe_glu = (v[0] != '0');
     if (const char *v = getenv("GLLMQ_GEMV_WAVES")) {
         long w = strtol(v, nullptr, 10);
         if (w >= 4 && w <= 65536) ctx->gemv_waves = static_cast<uint32_t>(w);
@@ -988,8 +995,10 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
     // Q4_K and Q6_K with rows of at most 16 blocks go to the int8 matrix cores, every token of
     // an expert (up to eight per job) in one pass over its weights.  `by_token`: the activation
     // rows are x[token] (gate/up), else rows by sorted position (down).
+    // `glu`: n counts the gate rows of an expert, its n up rows follow them, and yout receives
+    // act(gate . x) * (up . x)
     auto grouped_mm8 = [&](const Format &f, const void *wbase, size_t rb, uint32_t n, uint32_t k, const float *xin,
-                           bool by_token, float *yout) -> int {
+                           bool by_token, float *yout, bool glu = false) -> int {
         const int kind = mm8_kind(f.dtype);
         const bool q6k = kind == MM8_Q6K;
         const uint32_t groups = (k + 255u) / 256u;
@@ -1005,15 +1014,16 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         Q.g.tiles = (n + 31u) / 32u;
         Q.jobs = jobs8;
         Q.counters = counters;
-        Q.expert_stride = static_cast<uint64_t>(n) * rb;
+        Q.expert_stride = static_cast<uint64_t>(n) * rb * (glu ? 2u : 1u);
         Q.y_stride = n;
+        Q.g.glu_relu = relu_gate ? 1u : 0u;
         Q.rows = by_token ? nullptr : ctx->identity_rows;
         // upper bound of the jobs: one per expert hit, plus one per eight further pairs
         const uint64_t max_jobs = std::min<uint64_t>(pairs, experts + pairs / 8);
         uint32_t slices = std::max<uint32_t>(1u, (3u * static_cast<uint32_t>(ctx->num_cus)) / (2u * static_cast<uint32_t>(std::min<uint64_t>(pairs, experts))));
         if (ctx->tune_moe_slices) slices = ctx->tune_moe_slices;
         const uint32_t ppt = (groups + 7u) / 8u;
-        hipFunction_t fn = ctx->moe_mm8_fn[kind][ppt - 1];
+        hipFunction_t fn = glu ? ctx->moe_mm8_glu_fn[kind][ppt - 1] : ctx->moe_mm8_fn[kind][ppt - 1];
         uint32_t units = Q.g.tiles; // what the slices of a job share: tiles, or groups of eight tiles
         if (q6k && groups <= 8 && ctx->moe_mm8_rows) {
             fn = ctx->moe_mm8_q6k_rows;
@@ -1021,23 +1031,27 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         }
         slices = std::min(slices, units);
         Q.slices = slices;
-        return launch(ctx, fn, static_cast<uint32_t>(max_jobs * slices), 512, mm8_lds_bytes(groups, 8, 4, kind), stream,
+        return launch(ctx, fn, static_cast<uint32_t>(max_jobs * slices), 512, mm8_lds_bytes(groups, 8, 4, kind, glu), stream,
                       &Q, sizeof Q);
     };
-    auto fits_mm8 = [&](const Format &f, size_t k) {
+    auto fits_mm8 = [&](const Format &f, size_t k, bool glu = false) {
         const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
         const int kind = mm8_kind(f.dtype);
+        if (glu && !(ctx->moe_glu && (kind == MM8_Q4K || kind == MM8_Q5K))) return false;
         if (!(fast && ctx->use_mm8 && ctx->moe_mm8) || kind < 0 || kind >= MM8_MOE_KINDS || groups > 16 || k % 8 != 0) return false;
         if (kind == MM8_Q6K && !ctx->moe_mm8_q6k) return false;
-        return mm8_lds_bytes(groups, 8, 4, kind) <= 160u * 1024u;
+        return mm8_lds_bytes(groups, 8, 4, kind, glu) <= 160u * 1024u;
     };
     int rc = GLLMQ_OK;
-    if (fits_mm8(*fg, hidden))
+    const bool gated = fits_mm8(*fg, hidden, true); // gate, up and the activation in one launch
+    if (gated)
+        rc = grouped_mm8(*fg, gate_up, rb_gu, static_cast<uint32_t>(ffn), static_cast<uint32_t>(hidden), x, true, h, true);
+    else if (fits_mm8(*fg, hidden))
         rc = grouped_mm8(*fg, gate_up, rb_gu, static_cast<uint32_t>(2 * ffn), static_cast<uint32_t>(hidden), x, true, gu);
     else
         rc = grouped(*fg, gate_up, rb_gu, static_cast<uint32_t>(2 * ffn), static_cast<uint32_t>(hidden), x, true, gu);
     if (rc != GLLMQ_OK) return rc;
-    {
+    if (!gated) {
         MoeActParams P{ gu, h, counters, static_cast<uint32_t>(ffn), relu_gate ? 1u : 0u };
         rc = launch2d(ctx, ctx->moe_act, static_cast<uint32_t>((ffn + 255) / 256), static_cast<uint32_t>(pairs), 256, 0,
                       stream, &P, sizeof P);

@@ -173,14 +173,15 @@ def test_moe_more_than_eight_tokens_per_expert(hip, torch, oracle, hidden, ffn):
 
 def test_moe_grouped_kernel_alternatives(torch, oracle, monkeypatch):
     """The grouped kernels the default dispatch does not pick for this shape: Q6_K down rows on
-    the tile-split matrix-core kernel and on the integer-dot GEMV."""
+    the tile-split matrix-core kernel and on the integer-dot GEMV, gate/up results through memory
+    with the activation as a kernel of its own."""
     from gllm_amd.backend import HipBackend
     experts, tokens, top_k, hidden, ffn = 6, 20, 3, 512, 1024
     gu, dn = expert_weights(Q4_K, Q6_K, experts, hidden, ffn, seed=95)
     x = random_activations(tokens, hidden, seed=96)
     r = oracle.route(random_gate_logits(tokens, experts, seed=97), top_k, capacity_factor=float(experts))
     want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
-    for env in ({"GLLMQ_MOE_MM8_ROWS": "0"}, {"GLLMQ_MOE_MM8_Q6K": "0"}, {"GLLMQ_MOE_MM8": "0"}):
+    for env in ({"GLLMQ_MOE_MM8_ROWS": "0"}, {"GLLMQ_MOE_MM8_Q6K": "0"}, {"GLLMQ_MOE_MM8": "0"}, {"GLLMQ_MOE_GLU": "0"}):
         print(f"moe alternatives {env}", flush=True)
         with monkeypatch.context() as mp:
             for k_, v_ in env.items():
