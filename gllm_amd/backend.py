@@ -116,6 +116,11 @@ EXPORTED_SYMBOLS = [
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
     "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_quant_gather", "gllmq_stream_read", "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
+    "gllmq_gguf_open", "gllmq_gguf_parse", "gllmq_gguf_close", "gllmq_gguf_version", "gllmq_gguf_tensor_count",
+    "gllmq_gguf_kv_count", "gllmq_gguf_alignment", "gllmq_gguf_data_offset", "gllmq_gguf_tensor_at",
+    "gllmq_gguf_find_tensor", "gllmq_gguf_tensor_data", "gllmq_gguf_meta_type", "gllmq_gguf_meta_u64",
+    "gllmq_gguf_meta_i64", "gllmq_gguf_meta_f64", "gllmq_gguf_meta_bool", "gllmq_gguf_meta_str", "gllmq_gguf_meta_array",
+    "gllmq_gguf_meta_array_str", "gllmq_gguf_upload",
 ]
 
 

@@ -4,7 +4,7 @@
 
 Two steps, both plain compiler invocations (no cmake, no JIT cache):
   1. hipcc --genco --offload-arch=gfx950   csrc/gllmq_kernels.hip -> csrc/build/gllmq_kernels.hsaco
-  2. hipcc (host only)                     csrc/gllmq_host.cpp + the code object embedded with
+  2. hipcc (host only)                     csrc/gllmq_host.cpp, csrc/gguf_reader.cpp + the code object embedded with
                                            .incbin                -> gllm_amd/libgllm_hip_quant.so
 """
 from __future__ import annotations
@@ -46,7 +46,7 @@ def build_host() -> str:
     _run([HIPCC, "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
           "-D__HIP_PLATFORM_AMD__=1", f'-DGLLMQ_HSACO_PATH="{HSACO}"',
           "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROCM, "include"),
-          os.path.join(CSRC, "gllmq_host.cpp"), "-o", LIB,
+          "-I", CSRC, os.path.join(CSRC, "gllmq_host.cpp"), os.path.join(CSRC, "gguf_reader.cpp"), "-o", LIB,
           "-L", os.path.join(ROCM, "lib"), "-lamdhip64", f"-Wl,-rpath,{os.path.join(ROCM, 'lib')}"])
     return LIB
 

@@ -4,6 +4,7 @@
 // (src/compat/hip_backend.rs:211-238), except that the module is loaded and every
 // function resolved once per context instead of once per launch.
 #include "gllm_hip_quant.h"
+#include "gq_host_internal.h"
 #include "gq_params.h"
 
 #include <hip/hip_runtime_api.h>
@@ -194,6 +195,15 @@ int fail(gllmq_ctx *ctx, int code, const char *fmt, ...)
     }
     return code;
 }
+
+} // namespace
+
+extern "C" int gq_ctx_set_error(gllmq_ctx *ctx, int status, const char *message)
+{
+    return fail(ctx, status, "%s", message ? message : "");
+}
+
+namespace {
 
 #define GLLMQ_HIP(ctx, call)                                                                  \
     do {                                                                                      \

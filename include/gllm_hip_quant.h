@@ -191,6 +191,69 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up_dev, uint32_t dtype_gat
                      const uint32_t *route_expert_dev, const float *route_weight_dev,
                      const uint32_t *route_len_dev, int relu_gate, void *stream);
 
+/* ---- GGUF reader and tensor upload ---------------------------------------------------
+ * The file side of the path: what the reference's loader accepts and rejects
+ * (src/loader/gguf/reader.rs:38-187): magic "GGUF", version 3 only, key/value metadata,
+ * tensor infos, `general.alignment` (default 32, 0 is an error), tensor data from the aligned
+ * end of the infos, every tensor inside the file, no duplicate names; a tensor's bytes are
+ * ceil(ne0 / block) * block_bytes * ne1 * ... for all 36 dtype ids of
+ * src/loader/gguf/types.rs:57-94,152-236,443-472.  The file is mapped read-only and the
+ * tensor data is uploaded straight from the mapping.  Host only: needs no GPU except
+ * gllmq_gguf_upload.  Strings handed out are NOT zero-terminated views into the file
+ * (length returned beside them) except tensor names. */
+typedef struct gllmq_gguf gllmq_gguf;
+
+enum {
+    GLLMQ_GGUF_OK = 0,
+    GLLMQ_GGUF_ERR_IO = 1,       /* GgufError::Io */
+    GLLMQ_GGUF_ERR_MAGIC = 2,    /* GgufError::InvalidMagic */
+    GLLMQ_GGUF_ERR_VERSION = 3,  /* GgufError::UnsupportedVersion */
+    GLLMQ_GGUF_ERR_PARSE = 4,    /* GgufError::ParseError (truncated file, overflow, duplicate name, ...) */
+    GLLMQ_GGUF_ERR_METADATA = 5, /* GgufError::InvalidMetadata */
+    GLLMQ_GGUF_ERR_BOUNDS = 6,   /* GgufError::TensorOutOfBounds */
+    GLLMQ_GGUF_ERR_DTYPE = 7,    /* a ggml dtype id outside the table */
+    GLLMQ_GGUF_ERR_UTF8 = 8      /* GgufError::Utf8: a key, string value or tensor name that is not UTF-8 */
+};
+
+typedef struct gllmq_gguf_tensor {
+    const char *name;     /* zero-terminated, owned by the reader */
+    uint32_t ggml_dtype;
+    uint32_t n_dims;      /* 0..4 */
+    uint64_t shape[4];    /* outermost first, as the reference hands shapes to its consumers
+                             (reader.rs:593-598): a [n x k] weight reads {n, k} */
+    uint64_t ne[4];       /* as stored: ne[0] innermost */
+    size_t offset;        /* absolute position in the file */
+    size_t nbytes;
+} gllmq_gguf_tensor;
+
+int gllmq_gguf_open(const char *path, gllmq_gguf **out, char *err, size_t err_len);
+/* the same over an image in memory, which must outlive the reader */
+int gllmq_gguf_parse(const void *bytes, size_t len, gllmq_gguf **out, char *err, size_t err_len);
+void gllmq_gguf_close(gllmq_gguf *g);
+uint32_t gllmq_gguf_version(const gllmq_gguf *g);
+size_t gllmq_gguf_tensor_count(const gllmq_gguf *g);
+size_t gllmq_gguf_kv_count(const gllmq_gguf *g);
+size_t gllmq_gguf_alignment(const gllmq_gguf *g);
+size_t gllmq_gguf_data_offset(const gllmq_gguf *g);
+int gllmq_gguf_tensor_at(const gllmq_gguf *g, size_t index, gllmq_gguf_tensor *out);
+long gllmq_gguf_find_tensor(const gllmq_gguf *g, const char *name); /* -1: no such tensor */
+const void *gllmq_gguf_tensor_data(const gllmq_gguf *g, size_t index);
+/* metadata: the GgufValueType id (0..12) of a key or -1; the getters return 1 when the key
+ * exists and converts (gllmq_gguf_meta_u64 like GgufValue::as_u64: unsigned kinds, and signed
+ * kinds that are not negative), else 0 */
+int gllmq_gguf_meta_type(const gllmq_gguf *g, const char *key);
+int gllmq_gguf_meta_u64(const gllmq_gguf *g, const char *key, uint64_t *out);
+int gllmq_gguf_meta_i64(const gllmq_gguf *g, const char *key, int64_t *out);
+int gllmq_gguf_meta_f64(const gllmq_gguf *g, const char *key, double *out);
+int gllmq_gguf_meta_bool(const gllmq_gguf *g, const char *key, int *out);
+const char *gllmq_gguf_meta_str(const gllmq_gguf *g, const char *key, size_t *len);
+int gllmq_gguf_meta_array(const gllmq_gguf *g, const char *key, uint32_t *item_type, uint64_t *count);
+const char *gllmq_gguf_meta_array_str(const gllmq_gguf *g, const char *key, uint64_t index, size_t *len);
+/* tensor `index` into device memory (dst_bytes >= its nbytes), as the file stores it: the
+ * layout gllmq_quantized_matmul, gllmq_quant_gather and gllmq_ffn_swiglu take */
+int gllmq_gguf_upload(gllmq_ctx *ctx, const gllmq_gguf *g, size_t index, void *dst_dev, size_t dst_bytes,
+                      void *stream);
+
 /* ---- calibration ------------------------------------------------------------------
  * No counterpart in the reference.  Reads `n_bytes` (multiple of 16, 16-byte aligned) of
  * device memory once with a pure streaming kernel; timing it gives the read bandwidth a

@@ -71,6 +71,14 @@ extern "C" {
     pub fn gllmq_quant_gather_host(ctx: *mut gllmq_ctx, table: *const c_void, table_bytes: usize, ggml_dtype: u32,
                                    vocab: usize, hidden: usize, ids: *const u32, count: usize, scale: f32,
                                    out: *mut f32) -> c_int;
+    // GGUF reader (src/loader/gguf/reader.rs:38-187) and upload; the reader is an opaque handle
+    pub fn gllmq_gguf_open(path: *const c_char, out: *mut *mut c_void, err: *mut c_char, err_len: usize) -> c_int;
+    pub fn gllmq_gguf_close(g: *mut c_void);
+    pub fn gllmq_gguf_tensor_count(g: *const c_void) -> usize;
+    pub fn gllmq_gguf_find_tensor(g: *const c_void, name: *const c_char) -> std::os::raw::c_long;
+    pub fn gllmq_gguf_tensor_data(g: *const c_void, index: usize) -> *const c_void;
+    pub fn gllmq_gguf_upload(ctx: *mut gllmq_ctx, g: *const c_void, index: usize, dst_dev: *mut c_void,
+                             dst_bytes: usize, stream: *mut c_void) -> c_int;
     pub fn gllmq_dequantize_host(ctx: *mut gllmq_ctx, blocks: *const c_void, n_bytes: usize, out: *mut f32,
                                  n_out: usize, ggml_dtype: u32) -> c_int;
     pub fn gllmq_quantized_matmul_host(ctx: *mut gllmq_ctx, w: *const c_void, w_bytes: usize, x: *const f32,

@@ -1,0 +1,173 @@
+"""The GGUF reader against what the reference's reader accepts, rejects and hands out
+(src/loader/gguf/reader.rs:38-187 and its unit tests; src/loader/gguf/types.rs:443-472).
+Host only: no GPU."""
+import os
+
+import numpy as np
+import pytest
+
+from gllm_amd.gguf import GgufError, GgufFile
+from gllm_amd.synth import random_weight
+from tests import gguf_writer as W
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+
+
+def simple(**kw):
+    meta = [("general.architecture", W.STR, "llama"), ("llama.block_count", W.U32, 2)]
+    a = np.arange(32, dtype=np.float32).reshape(4, 8)
+    return W.build(kw.pop("metadata", meta), kw.pop("tensors", [W.f32_tensor("a.weight", a)]), **kw)
+
+
+def test_header_counts_and_default_alignment():
+    g = GgufFile(image=simple())
+    assert (g.version, g.tensor_count, g.kv_count, g.alignment) == (3, 1, 2, 32)  # default alignment 32 (reader.rs:102-107)
+    assert g.data_offset % 32 == 0
+    assert g.meta("general.architecture") == "llama" and g.meta("llama.block_count") == 2
+    assert g.meta("no.such.key") is None
+
+
+def test_shapes_are_reversed_to_outermost_first():
+    """reader.rs tests iter_tensors_yields_reversed_shapes ([8,4] -> [4,8]), the 3-D case
+    ([8,4,2] -> [2,4,8]) and tensor_provider_1d_shape_not_reversed."""
+    t2 = ("m", [8, 4], 0, np.zeros(32, np.float32).tobytes())
+    t3 = ("c", [8, 4, 2], 0, np.zeros(64, np.float32).tobytes())
+    t1 = ("v", [8], 0, np.zeros(8, np.float32).tobytes())
+    g = GgufFile(image=simple(tensors=[t2, t3, t1]))
+    assert g.tensor("m").shape == (4, 8) and g.tensor("m").ne == (8, 4)
+    assert g.tensor("c").shape == (2, 4, 8)
+    assert g.tensor("v").shape == (8,)
+    assert [t.name for t in g.tensors()] == ["m", "c", "v"]
+
+
+def test_tensor_bytes_pad_rows_to_whole_blocks():
+    # types.rs:443-472; the documented example: Q4_0 [33, 2] is 2 blocks x 18 bytes x 2 rows = 72
+    cases = [(2, [33, 2], 72), (2, [33], 36), (Q8_0, [33], 68), (Q4_K, [256, 4], 576), (Q6_K, [256, 4], 840),
+             (Q4_K, [300, 3], 2 * 144 * 3), (0, [5, 7], 140), (30, [6], 12), (15, [256], 292), (39, [64], 34)]
+    tensors = [(f"t{i}", ne, dt, bytes(n)) for i, (dt, ne, n) in enumerate(cases)]
+    g = GgufFile(image=simple(tensors=tensors))
+    for i, (dt, ne, n) in enumerate(cases):
+        assert g.tensor(f"t{i}").nbytes == n, (dt, ne)
+    # every tensor starts on a multiple of the alignment behind the data offset
+    assert all((t.offset - g.data_offset) % 32 == 0 for t in g.tensors())
+
+
+def test_tensor_data_is_what_was_written_and_alignment_key_is_honoured():
+    w = random_weight(Q4_K, 5, 512, seed=1)
+    a = np.arange(12, dtype=np.float32)
+    meta = [("general.alignment", W.U32, 64), ("x", W.F32, 1.5)]
+    g = GgufFile(image=simple(metadata=meta, tensors=[("w", [512, 5], Q4_K, np.asarray(w).tobytes()), W.f32_tensor("a", a)]))
+    assert g.alignment == 64 and g.data_offset % 64 == 0
+    assert g.tensor_bytes("w") == np.asarray(w).tobytes()
+    assert np.array_equal(np.frombuffer(g.tensor_bytes("a"), np.float32), a)
+    assert g.tensor("w").shape == (5, 512) and g.tensor("w").ggml_dtype == Q4_K
+    assert g.tensor("a").offset % 64 == 0
+
+
+def test_metadata_value_types():
+    meta = [("u8", W.U8, 42), ("i8n", W.I8, -1), ("i8p", W.I8, 100), ("u16", W.U16, 0x1234), ("i16n", W.I16, -32768),
+            ("u32", W.U32, 7), ("i32", W.I32, -5), ("f32", W.F32, 0.25), ("yes", W.BOOL, 1), ("no", W.BOOL, 0),
+            ("s", W.STR, "中文测试"), ("empty", W.STR, ""), ("u64", W.U64, 2 ** 63 + 5), ("i64", W.I64, -2 ** 62),
+            ("f64", W.F64, 1e100), ("toks", W.ARR, (W.STR, ["<s>", "</s>", "hello"])), ("nums", W.ARR, (W.I32, [1, 2, 3])),
+            ("nest", W.ARR, (W.ARR, [(W.U8, [1, 2]), (W.U8, [])]))]
+    g = GgufFile(image=simple(metadata=meta))
+    assert g.kv_count == len(meta)
+    # GgufValue::as_u64 (reader.rs tests parse_value_uint8 / _int8 / _int8_positive / _uint16 / _int16_negative)
+    assert g.meta_u64("u8") == 42 and g.meta_u64("i8n") is None and g.meta_u64("i8p") == 100
+    assert g.meta_u64("u16") == 0x1234 and g.meta_u64("i16n") is None and g.meta_u64("s") is None
+    assert g.meta("i8n") == -1 and g.meta("i16n") == -32768 and g.meta("i32") == -5 and g.meta("i64") == -2 ** 62
+    assert g.meta("u64") == 2 ** 63 + 5 and g.meta("f32") == 0.25 and g.meta("f64") == 1e100
+    assert g.meta("yes") is True and g.meta("no") is False
+    assert g.meta("s") == "中文测试" and g.meta("empty") == ""   # read_string_utf8_cjk, read_string_empty
+    assert g.meta("toks") == ["<s>", "</s>", "hello"] and g.meta("nums") == (W.I32, 3) and g.meta("nest") == (W.ARR, 2)
+
+
+def test_rejections():
+    def kind(image):
+        with pytest.raises(GgufError) as e:
+            GgufFile(image=image)
+        return e.value.kind
+    assert kind(simple(magic=0x46554746)) == "InvalidMagic"
+    assert kind(simple(version=2)) == "UnsupportedVersion" and kind(simple(version=4)) == "UnsupportedVersion"
+    assert kind(simple(metadata=[("general.alignment", W.U32, 0)], alignment=32)) == "InvalidMetadata"
+    assert kind(b"GGUF") == "ParseError" and kind(b"") == "ParseError"
+    whole = simple()
+    for cut in (10, 24, 40, len(whole) - 130):       # inside the header, a key, a value, the tensor infos
+        assert kind(whole[:cut]) == "ParseError", cut
+    assert kind(whole[:-1]) == "TensorOutOfBounds"    # the last tensor loses a byte
+    assert kind(simple(offsets=[1 << 40])) == "TensorOutOfBounds"
+    # a count that claims one more tensor info than the file holds reads padding as an info: rejected one way or the other
+    assert kind(simple(tensor_count=2)) in ("ParseError", "TensorOutOfBounds", "UnknownDType")
+    two = [W.f32_tensor("same", np.zeros(4)), W.f32_tensor("same", np.ones(4))]
+    assert kind(simple(tensors=two)) == "ParseError"  # duplicate tensor name
+    assert kind(simple(tensors=[("t", [4], 4, bytes(16))])) == "UnknownDType"   # id 4 is a hole in the table
+    assert kind(simple(tensors=[("t", [1 << 62, 1 << 62], 0, b"")])) == "ParseError"  # byte size overflow
+    assert kind(simple(metadata=[("k", 13, 0)])) == "ParseError"               # value type outside 0..12
+    assert kind(simple(metadata=[("s", W.STR, b"ab\xff")])) == "Utf8"            # str::from_utf8 of the reference
+    assert kind(simple(metadata=[("s", W.STR, b"\xed\xa0\x80")])) == "Utf8"     # a surrogate
+    assert kind(simple(metadata=[("s", W.STR, b"\xc0\x80")])) == "Utf8"         # an overlong form
+    assert kind(simple(tensors=[(b"t\xfe", [4], 0, bytes(16))])) == "Utf8"
+    # an array that claims 2^40 items in a file of a few hundred bytes
+    img = bytearray(simple(metadata=[("a", W.ARR, (W.U32, [1, 2]))]))
+    at = img.index(b"a" + (W.ARR).to_bytes(4, "little") + (W.U32).to_bytes(4, "little")) + 9
+    img[at:at + 8] = (1 << 40).to_bytes(8, "little")
+    assert kind(bytes(img)) == "ParseError"
+
+
+def test_a_key_that_repeats_keeps_the_later_value_and_odd_alignment_types_fall_back():
+    g = GgufFile(image=simple(metadata=[("k", W.U32, 1), ("k", W.U32, 2)]))
+    assert g.meta("k") == 2 and g.kv_count == 2
+    # a general.alignment that is not an unsigned number reads as absent: the default 32
+    g = GgufFile(image=simple(metadata=[("general.alignment", W.STR, "64")], alignment=32))
+    assert g.alignment == 32
+
+
+def test_open_from_a_file(tmp_path):
+    path = os.path.join(tmp_path, "m.gguf")
+    w = random_weight(Q6_K, 3, 256, seed=2)
+    with open(path, "wb") as f:
+        f.write(simple(tensors=[("blk.0.ffn_down.weight", [256, 3], Q6_K, np.asarray(w).tobytes())]))
+    g = GgufFile(path)
+    assert g.tensor("blk.0.ffn_down.weight").shape == (3, 256)
+    assert g.tensor_bytes(0) == np.asarray(w).tobytes()
+    with pytest.raises(KeyError):
+        g.tensor("blk.1.ffn_down.weight")
+    g.close()
+    with pytest.raises(GgufError) as e:
+        GgufFile(os.path.join(tmp_path, "missing.gguf"))
+    assert e.value.kind == "Io"
+
+
+def test_mutated_files_never_crash_the_reader():
+    """Two thousand seeded mutations (byte flips, truncations, length fields blown up) of a valid
+    file: each either opens or raises GgufError; tensor views stay inside the image."""
+    meta = [("general.architecture", W.STR, "llama"), ("toks", W.ARR, (W.STR, ["a", "bc"])), ("n", W.U64, 5),
+            ("nest", W.ARR, (W.ARR, [(W.U8, [1, 2]), (W.U8, [3])]))]
+    base = W.build(meta, [W.f32_tensor("a", np.arange(16).reshape(2, 8)), ("q", [64, 2], Q8_0, bytes(136))])
+    rng = np.random.default_rng(0)
+    opened = 0
+    for i in range(2000):
+        img = bytearray(base)
+        how = i % 4
+        if how == 0:
+            for _ in range(int(rng.integers(1, 4))):
+                img[int(rng.integers(0, len(img)))] = int(rng.integers(0, 256))
+        elif how == 1:
+            img = img[:int(rng.integers(0, len(img)))]
+        elif how == 2:
+            at = int(rng.integers(0, max(1, len(img) - 8)))
+            img[at:at + 8] = int(rng.integers(0, 1 << 63)).to_bytes(8, "little")
+        else:
+            at = int(rng.integers(0, max(1, len(img) - 4)))
+            img[at:at + 4] = b"\xff\xff\xff\xff"
+        try:
+            g = GgufFile(image=bytes(img))
+        except GgufError:
+            continue
+        opened += 1
+        for t in g.tensors():
+            assert t.offset + t.nbytes <= len(img)
+            assert len(g.tensor_bytes(t.index)) == t.nbytes
+        for key in ("general.architecture", "toks", "n", "nest"):
+            g.meta(key)
+    assert opened > 0
