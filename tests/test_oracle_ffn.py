@@ -17,7 +17,8 @@ def numpy_ffn(gate, up, t_gu, down, t_dn, x, hidden, ffn, relu=False):
     g = x.astype(np.float64) @ wg.T
     if relu:
         g = np.maximum(g, 0.0)
-    h = g / (1.0 + np.exp(-g)) * (x.astype(np.float64) @ wu.T)
+    with np.errstate(over="ignore"):  # exp(-g) overflows to inf for very negative gates: silu is -0 there
+        h = g / (1.0 + np.exp(-g)) * (x.astype(np.float64) @ wu.T)
     return h @ wd.T
 
 
