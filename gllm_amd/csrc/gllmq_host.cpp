@@ -103,11 +103,11 @@ int mm8_kind(uint32_t dtype)
 
 // Bytes of LDS the int8 matrix-core kernels need: Q6_K keeps 16 sub-block sums per block
 // instead of 8, Q8_0 none, and the weight stage of a wave differs by format.
-uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs, int kind = MM8_Q4K, bool glu = false)
+uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs, int kind = MM8_Q4K)
 {
     const uint32_t stage = kind == MM8_Q6K ? gq::MM8Q6_STAGE_BYTES : kind == MM8_Q8_0 ? gq::MM8Q8_STAGE_BYTES
                          : kind == MM8_Q5K ? gq::Mm8Format<1>::STAGE : gq::Mm8Format<0>::STAGE;
-    return gq::mm8_lds_layout(groups, m, pairs, kind == MM8_Q6K ? 16u : kind == MM8_Q8_0 ? 0u : 8u, stage, glu ? 4u : 2u).total;
+    return gq::mm8_lds_layout(groups, m, pairs, kind == MM8_Q6K ? 16u : kind == MM8_Q8_0 ? 0u : 8u, stage).total;
 }
 
 } // namespace
@@ -340,16 +340,21 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     const bool glu = w2 != nullptr;
     if (glu && kind != MM8_Q4K && kind != MM8_Q5K) return -1;
     if (glu) one_pass_only = true;
-    if (kind == MM8_Q6K && (ctx->mm8_q6k_min_m == 0 || m < ctx->mm8_q6k_min_m)) return -1;
+    // The row thresholds below say where the GEMV kernels are as fast; that holds while a GEMV
+    // workgroup's prepared activations (848 bytes per row and 256 elements) leave room for
+    // several workgroups per CU.  Two rows of more than 9728 elements do not (one workgroup of
+    // four waves per CU: 35 against 25 us for Q6_K 14336 -> 4096), so they come here.
+    const bool gemv_cramped = 848u * m * ((k + 255) / 256) > 64u * 1024u;
+    if (kind == MM8_Q6K && (ctx->mm8_q6k_min_m == 0 || (m < ctx->mm8_q6k_min_m && !gemv_cramped))) return -1;
     if (kind == MM8_Q5K && !glu && (ctx->mm8_q5k_min_m == 0 || m < ctx->mm8_q5k_min_m)) return -1;
-    if (kind == MM8_Q8_0 && (ctx->mm8_q8_0_min_m == 0 || m < ctx->mm8_q8_0_min_m)) return -1;
+    if (kind == MM8_Q8_0 && (ctx->mm8_q8_0_min_m == 0 || (m < ctx->mm8_q8_0_min_m && !gemv_cramped))) return -1;
     if (kind == MM8_Q8_0 && k < 256) return -1; // its fetch window is one whole group of 8 blocks
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
     // Rows per pass: as many as the prepared activations leave room for in the 160 KiB of LDS.
     auto pairs_for = [](uint32_t rows) { return rows <= 2 ? 1u : (rows <= 4 ? 2u : 4u); };
     uint32_t rows_per_pass = static_cast<uint32_t>(std::min<size_t>(m, 8));
-    while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass), kind, glu) > 160u * 1024u)
+    while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass), kind) > 160u * 1024u)
         --rows_per_pass;
     if (rows_per_pass == 0) return -1;
     if (one_pass_only && rows_per_pass < m) return -1;
@@ -357,7 +362,7 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(rows_per_pass, m - m0));
         const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
         const uint32_t pairs = 1u << pi;
-        const uint32_t lds = mm8_lds_bytes(groups, mm, pairs, kind, glu);
+        const uint32_t lds = mm8_lds_bytes(groups, mm, pairs, kind);
         Mm8Params P{};
         P.w2 = w2;
         P.glu_relu = glu_relu ? 1u : 0u;
@@ -1041,7 +1046,7 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         }
         slices = std::min(slices, units);
         Q.slices = slices;
-        return launch(ctx, fn, static_cast<uint32_t>(max_jobs * slices), 512, mm8_lds_bytes(groups, 8, 4, kind, glu), stream,
+        return launch(ctx, fn, static_cast<uint32_t>(max_jobs * slices), 512, mm8_lds_bytes(groups, 8, 4, kind), stream,
                       &Q, sizeof Q);
     };
     auto fits_mm8 = [&](const Format &f, size_t k, bool glu = false) {
@@ -1050,7 +1055,7 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         if (glu && !(ctx->moe_glu && (kind == MM8_Q4K || kind == MM8_Q5K))) return false;
         if (!(fast && ctx->use_mm8 && ctx->moe_mm8) || kind < 0 || kind >= MM8_MOE_KINDS || groups > 16 || k % 8 != 0) return false;
         if (kind == MM8_Q6K && !ctx->moe_mm8_q6k) return false;
-        return mm8_lds_bytes(groups, 8, 4, kind, glu) <= 160u * 1024u;
+        return mm8_lds_bytes(groups, 8, 4, kind) <= 160u * 1024u;
     };
     int rc = GLLMQ_OK;
     const bool gated = fits_mm8(*fg, hidden, true); // gate, up and the activation in one launch

@@ -75,7 +75,7 @@ struct Mm8Lds {
     uint32_t planes;       // offset of [3 * m][plane_stride]
     uint32_t sums;         // offset of float [m][groups][8]: sum of X per sub-block
     uint32_t scales;       // offset of float [m][groups]: 2^e per block (NaN if poisoned)
-    uint32_t red;          // offset of float [red_bufs][MM8_WAVES][PAIRS][64]
+    uint32_t red;          // offset of float [2][MM8_WAVES][PAIRS][64]
     uint32_t stage;        // offset of [MM8_WAVES][MM8_STAGE_BYTES]: one weight block tile per wave
     uint32_t total;
 };
@@ -83,7 +83,7 @@ struct Mm8Lds {
 // `subs`: sub-block sums kept per 256-element block (8 of 32 elements for Q4_K, 16 of 16 for
 // Q6_K, none for Q8_0); `stage_bytes`: one wave's weight stage.
 GQ_HD inline Mm8Lds mm8_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, uint32_t subs = 8u,
-                                   uint32_t stage_bytes = MM8_STAGE_BYTES, uint32_t red_bufs = 2u)
+                                   uint32_t stage_bytes = MM8_STAGE_BYTES)
 {
     Mm8Lds L;
     L.plane_stride = groups * 256u + 16u; // +16 staggers the planes over the LDS banks
@@ -91,7 +91,7 @@ GQ_HD inline Mm8Lds mm8_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, 
     L.sums = L.planes + 3u * m * L.plane_stride;
     L.scales = L.sums + m * groups * subs * 4u;
     L.red = (L.scales + m * groups * 4u + 15u) & ~15u;
-    L.stage = L.red + red_bufs * MM8_WAVES * pairs * 64u * 4u;
+    L.stage = L.red + 2u * MM8_WAVES * pairs * 64u * 4u;
     L.total = L.stage + MM8_WAVES * stage_bytes;
     return L;
 }
