@@ -331,6 +331,21 @@ def test_q8_0_matrix_core_shapes(hip, torch, oracle):
         check_close(got, want, f"q8_0 m={m} n={n} k={k}")
 
 
+@pytest.mark.parametrize("dtype", ALL)
+def test_long_rows_one_and_two_activation_rows(hip, torch, oracle, dtype):
+    """Long rows with one and two activation rows (the waves of a GEMV workgroup share a row, rows
+    past 16384 elements take several launches; two rows past 9728 elements take the 8-row kernel):
+    whole groups, a partial last group, ragged n, up to 65536 elements."""
+    step = 32 if dtype == Q8_0 else 256
+    for n, k in [(257, 8192), (70, 14336), (33, 11008), (5, 8448 + step), (129, 16384 + 4 * step - 8), (64, 65536)]:
+        for m in (1, 2):
+            print(f"long rows dtype={dtype} n={n} k={k} m={m}", flush=True)
+            w, x = random_weight(dtype, n, k, seed=n + m), random_activations(m, k, seed=k % 1000)
+            want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+            got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+            check_close(got, want, f"dtype={dtype} n={n} k={k} m={m}")
+
+
 def test_empty_shapes_are_no_ops(hip, torch):
     print("empty shapes", flush=True)
     w = torch.zeros(144 * 16, dtype=torch.uint8, device="cuda")
