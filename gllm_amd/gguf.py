@@ -172,6 +172,32 @@ class GgufFile:
         v = C.c_uint64()
         return v.value if self._lib.gllmq_gguf_meta_u64(self._h, key.encode(), C.byref(v)) else None
 
+    def layer_table(self) -> dict:
+        """``{layer: {projection: TensorInfo}}`` over the per-layer weights ``blk.{layer}.{projection}.weight``
+        (attn_q, attn_k, attn_v, attn_output, ffn_gate, ffn_up, ffn_down, ...): the (layer, projection) ->
+        dtype table a host walks to call the kernels with each matrix's own format, as `*_K_M` files
+        mix Q4_K / Q5_K with Q6_K from layer to layer."""
+        table: dict = {}
+        for t in self.tensors():
+            parts = t.name.split(".")
+            if len(parts) == 4 and parts[0] == "blk" and parts[1].isdigit() and parts[3] == "weight":
+                table.setdefault(int(parts[1]), {})[parts[2]] = t
+        return dict(sorted(table.items()))
+
+    def mixed_quant_groups(self):
+        """Layers grouped by their dtype signature (sorted ``(projection, dtype)`` pairs), or None when
+        every layer has the same one: what the reference's graph builder detects before it emits
+        per-group matmul ops (src/arch/auto_graph_fragments/build_graph.inc.rs:388-470).  Groups come
+        in a fixed order: by signature, then by first layer."""
+        sigs = {layer: tuple(sorted((proj, t.ggml_dtype) for proj, t in projs.items()))
+                for layer, projs in self.layer_table().items()}
+        if len(set(sigs.values())) <= 1:
+            return None
+        groups: dict = {}
+        for layer, sig in sigs.items():
+            groups.setdefault(sig, []).append(layer)
+        return sorted(groups.items(), key=lambda kv: (kv[0], kv[1][0]))
+
     def upload(self, hip: "backend.HipBackend", key, dst) -> TensorInfo:
         """Copies the tensor's bytes, as stored, into the device uint8 tensor ``dst``."""
         t = self.tensor(key)

@@ -171,3 +171,32 @@ def test_mutated_files_never_crash_the_reader():
         for key in ("general.architecture", "toks", "n", "nest"):
             g.meta(key)
     assert opened > 0
+
+
+def k_m_style_file(layers=4, hidden=256, ffn=512, down_q6k=(0, 3)):
+    """Per-layer weights as a Q4_K_M file lays them out: ffn_down is Q6_K in some layers, Q4_K in the rest."""
+    tensors, host = [], {}
+    for layer in range(layers):
+        for proj, (n, k) in (("ffn_gate", (ffn, hidden)), ("ffn_up", (ffn, hidden)), ("ffn_down", (hidden, ffn))):
+            dt = Q6_K if (proj == "ffn_down" and layer in down_q6k) else Q4_K
+            w = random_weight(dt, n, k, seed=100 * layer + len(proj))
+            name = f"blk.{layer}.{proj}.weight"
+            tensors.append((name, [k, n], dt, np.asarray(w).tobytes()))
+            host[name] = (dt, n, k, w)
+    tensors.append(W.f32_tensor("output_norm.weight", np.ones(hidden)))
+    meta = [("general.architecture", W.STR, "llama"), ("llama.block_count", W.U32, layers)]
+    return W.build(meta, tensors), host
+
+
+def test_layer_table_and_mixed_quant_groups():
+    image, host = k_m_style_file()
+    g = GgufFile(image=image)
+    table = g.layer_table()
+    assert list(table) == [0, 1, 2, 3] and sorted(table[2]) == ["ffn_down", "ffn_gate", "ffn_up"]
+    assert [table[i]["ffn_down"].ggml_dtype for i in range(4)] == [Q6_K, Q4_K, Q4_K, Q6_K]
+    assert all(table[i]["ffn_gate"].ggml_dtype == Q4_K and table[i]["ffn_gate"].shape == (512, 256) for i in range(4))
+    groups = g.mixed_quant_groups()
+    assert [layers for _, layers in groups] == [[1, 2], [0, 3]]          # by signature (dtype 12 before 14), then first layer
+    assert dict(groups[1][0])["ffn_down"] == Q6_K
+    uniform, _ = k_m_style_file(down_q6k=())
+    assert GgufFile(image=uniform).mixed_quant_groups() is None          # the reference's plan is None for uniform models

@@ -85,3 +85,37 @@ def test_gguf_to_tokens(hip, torch, oracle, tmp_path):
     assert tok.cpu().numpy().tolist() == [oracle.argmax_token(got[r]) for r in range(m)]
     for r in range(m):
         assert el[r, int(tok[r])] >= el[r].max() - 2e-3 * np.abs(el[r]).max()
+
+
+def test_mixed_quant_layers_from_the_layer_table(hip, torch, oracle, tmp_path):
+    """A Q4_K_M-style file (ffn_down Q6_K in layers 0 and 3, Q4_K in 1 and 2): the host walks the
+    layer table and calls the same entry point with each matrix's own dtype."""
+    from tests.test_gguf_reader import k_m_style_file
+    print("mixed-quant layers", flush=True)
+    image, host = k_m_style_file()
+    path = os.path.join(tmp_path, "km.gguf")
+    with open(path, "wb") as f:
+        f.write(image)
+    g = GgufFile(path)
+    assert [layers for _, layers in g.mixed_quant_groups()] == [[1, 2], [0, 3]]
+    hidden, ffn, m = 256, 512, 2
+    x = np.random.default_rng(0).standard_normal((m, hidden)).astype(np.float32)
+    xd, want = torch.from_numpy(x).cuda(), x
+    for layer, projs in g.layer_table().items():
+        dev = {}
+        for proj, t in projs.items():
+            dev[proj] = torch.empty(t.nbytes, dtype=torch.uint8, device="cuda")
+            g.upload(hip, t.name, dev[proj])
+        out = torch.empty(m, hidden, device="cuda")
+        hip.ffn_swiglu(dev["ffn_gate"], dev["ffn_up"], projs["ffn_gate"].ggml_dtype, dev["ffn_down"],
+                       projs["ffn_down"].ggml_dtype, xd, out, m, hidden, ffn)
+        torch.cuda.synchronize()
+        names = [f"blk.{layer}.{p}.weight" for p in ("ffn_gate", "ffn_up", "ffn_down")]
+        want = oracle.ffn_swiglu(host[names[0]][3], host[names[1]][3], host[names[0]][0], host[names[2]][3],
+                                 host[names[2]][0], want, m, hidden, ffn, acc=oracle.ACC_F64, threads=4)
+        got = out.cpu().numpy()
+        rel = np.linalg.norm(got - want) / np.linalg.norm(want)
+        assert rel <= 1e-4, (layer, rel)
+        # the next layer continues from the GPU's own output, normalised so that magnitudes stay put
+        scale = float(np.abs(got).max())
+        xd, want = out / scale, (got / np.float32(scale)).astype(np.float32)
