@@ -126,9 +126,10 @@ def run_other(args):
             if dt > budget_s or reps >= 200:
                 return dt / reps, reps, dt
 
-    if name in ("gemv_q4k_4096", "gemv_q6k", "gemm_m16", "gemm_m32", "gemm_m64", "layer_mix", "layer_mix_m32", "lm_head_q6k"):
+    if name in ("gemv_q4k_4096", "gemv_q6k", "gemm_m16", "gemm_m32", "gemm_m64", "layer_mix", "layer_mix_m4", "layer_mix_m32",
+                "lm_head_q6k"):
         if name.startswith("layer_mix"):
-            mm = 32 if name.endswith("_m32") else 1  # decode, or batched decode of 32 sequences
+            mm = int(name.split("_m")[2]) if name.count("_m") == 2 else 1  # decode, or batched decode of 4 / 32 sequences
             ops = [(12, 6144, 4096, mm), (12, 4096, 4096, mm), (12, 2 * 14336, 4096, mm), (14, 4096, 14336, mm)]
             copies = 3
         else:
@@ -350,7 +351,7 @@ def main():
     ap.add_argument("--no-context", action="store_true",
                     help="skip the cache-resident and streaming-read context runs (profiling: only the timed kernel launches)")
     ap.add_argument("--workload", default="gemv_q4k",
-                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, lm_head_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
+                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m4, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, lm_head_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
                          "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch plain device-to-device copies of one 33 MB weight buffer (counter calibration)")

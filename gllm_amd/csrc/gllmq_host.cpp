@@ -168,6 +168,12 @@ struct gllmq_ctx {
     hipFunction_t moe_mm8_fn[MM8_KINDS][2] = {}; // grouped int8 matrix-core kernels [Mm8Kind][passes per tile - 1]
     hipFunction_t moe_mm8_q6k_rows = nullptr;   // Q6_K rows of at most 8 blocks: a wave per 32-row tile
     uint32_t *identity_rows = nullptr;          // device: 0..7, the activation rows of an ungathered matmul
+    // K split of the int8 kernels for few weight rows: slice sums and arrival counters (fixed size,
+    // allocated at init; shared by all calls on this context).  GLLMQ_MM8_KSPLIT caps the number of
+    // slices (0 or 1 = never split).
+    float *mm8_part = nullptr;
+    uint32_t *mm8_arrive = nullptr;
+    uint32_t mm8_ksplit_max = 8;
     // Device workspace of the MoE path (pair tables, jobs, intermediate activations).  It
     // grows on demand and is shared by all calls on this context: calls that use it must
     // not overlap in time.
@@ -351,10 +357,41 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     if (kind == MM8_Q8_0 && k < 256) return -1; // its fetch window is one whole group of 8 blocks
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
-    // Rows per pass: as many as the prepared activations leave room for in the 160 KiB of LDS.
+    // K split: with tiles for at most half of the CUs, 2..8 workgroups share each tile and take
+    // a slice of K each (whole passes of 8 blocks); the slices meet inside the launch.  The
+    // meeting costs about 2 us, so a slice keeps at least two passes, unless only a shorter slice
+    // lets the prepared activations of all rows fit the LDS (one pass over the weights then beats
+    // the alternatives by more than that).
+    const uint32_t tiles = static_cast<uint32_t>((n + 31) / 32), ppt_row = (groups + 7u) / 8u;
     auto pairs_for = [](uint32_t rows) { return rows <= 2 ? 1u : (rows <= 4 ? 2u : 4u); };
-    uint32_t rows_per_pass = static_cast<uint32_t>(std::min<size_t>(m, 8));
-    while (rows_per_pass > 0 && mm8_lds_bytes(groups, rows_per_pass, pairs_for(rows_per_pass), kind) > 160u * 1024u)
+    const uint32_t m_pass = static_cast<uint32_t>(std::min<size_t>(m, 8));
+    uint32_t ksplit = 1, slice_passes = ppt_row;
+    if (!glu && ctx->mm8_ksplit_max > 1 && ppt_row >= 2 && (kind != MM8_Q8_0 || k % 256 == 0)) {
+        auto fits = [&](uint32_t slices) {
+            const uint32_t passes = (ppt_row + slices - 1) / slices;
+            return mm8_lds_bytes(std::min(groups, passes * 8u), m_pass, pairs_for(m_pass), kind) <= 160u * 1024u;
+        };
+        const uint32_t most = std::min(ppt_row, ctx->mm8_ksplit_max);
+        uint32_t want = 1;
+        if (tiles * 2u <= static_cast<uint32_t>(ctx->num_cus))
+            want = std::max(1u, std::min({ static_cast<uint32_t>(ctx->num_cus) / tiles, ppt_row / 2u, most }));
+        while (want < most && !fits(want)) ++want;
+        // more workgroups than CUs run in rounds: whole rounds beat one and a half
+        const uint32_t cus = static_cast<uint32_t>(ctx->num_cus);
+        if (want > 1 && want * tiles > cus && tiles <= cus)
+            for (uint32_t w2 = want; w2 <= most; ++w2)
+                if ((w2 * tiles) % cus == 0) { want = w2; break; }
+        if (fits(want)) {
+            slice_passes = (ppt_row + want - 1) / want;
+            ksplit = (ppt_row + slice_passes - 1) / slice_passes; // every slice gets at least one pass
+        }
+        if (static_cast<size_t>(ksplit) * m_pass * n > gq::MM8_SPLIT_PART_FLOATS) ksplit = 1;
+        if (ksplit == 1) slice_passes = ppt_row;
+    }
+    const uint32_t lds_groups = ksplit > 1 ? std::min(groups, slice_passes * 8u) : groups;
+    // Rows per pass: as many as the prepared activations leave room for in the 160 KiB of LDS.
+    uint32_t rows_per_pass = m_pass;
+    while (rows_per_pass > 0 && mm8_lds_bytes(lds_groups, rows_per_pass, pairs_for(rows_per_pass), kind) > 160u * 1024u)
         --rows_per_pass;
     if (rows_per_pass == 0) return -1;
     if (one_pass_only && rows_per_pass < m) return -1;
@@ -362,8 +399,12 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(rows_per_pass, m - m0));
         const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
         const uint32_t pairs = 1u << pi;
-        const uint32_t lds = mm8_lds_bytes(groups, mm, pairs, kind);
+        const uint32_t lds = mm8_lds_bytes(lds_groups, mm, pairs, kind);
         Mm8Params P{};
+        P.ksplit = ksplit;
+        P.kslice_groups = slice_passes * 8u;
+        P.part = ctx->mm8_part;
+        P.arrive = ctx->mm8_arrive;
         P.w2 = w2;
         P.glu_relu = glu_relu ? 1u : 0u;
         P.w = w;
@@ -380,17 +421,18 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         P.act_bf16 = act_bf16 ? 1u : 0u;
         P.xrows = ctx->identity_rows;
         // preparation steps per wave: two 256-element blocks per step
-        const uint32_t ppt = (groups + 7u) / 8u, steps = ((ppt + 1u) / 2u) * mm;
+        const uint32_t ppt = slice_passes, steps = ((ppt + 1u) / 2u) * mm;
         int ei = steps <= 1 ? 0 : (steps <= 2 ? 1 : 2);
         while (ei < 2 && !ctx->mm8[kind][pi][ei]) ++ei; // not every (pairs, early) pair is built
         const int gi = kind == MM8_Q5K ? 1 : 0;
-        uint32_t grid = std::min<uint32_t>(P.tiles, static_cast<uint32_t>(ctx->num_cus));
-        if (ctx->tune_mm8_grid) grid = std::min<uint32_t>(P.tiles, ctx->tune_mm8_grid);
-        P.grid = grid;
+        uint32_t grid = std::min<uint32_t>(P.tiles, std::max(1u, static_cast<uint32_t>(ctx->num_cus) / ksplit));
+        if (ctx->tune_mm8_grid) grid = std::min<uint32_t>(P.tiles, std::max(1u, ctx->tune_mm8_grid / ksplit));
+        if (ksplit > 1) grid = std::min(grid, gq::MM8_SPLIT_MAX_LISTS);
+        P.grid = grid; // workgroups per slice: launch index = tile list * ksplit + slice
         hipFunction_t fn = glu ? ctx->mm8_glu[gi][pi][ei] : ctx->mm8[kind][pi][ei];
         if (pi <= 1 && ppt <= 2 && ctx->mm8_areg_on)
             fn = glu ? ctx->mm8_glu_areg[gi][pi][ei][ppt - 1] : ctx->mm8_areg[kind][pi][ei][ppt - 1];
-        int rc = launch(ctx, fn, grid, 512, lds, stream, &P, sizeof P);
+        int rc = launch(ctx, fn, grid * ksplit, 512, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }
     return GLLMQ_OK;
@@ -626,6 +668,12 @@ int gllmq_init(gllmq_ctx **out, int device)
         if (he != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "argmax scratch: %s", hipGetErrorString(he));
     }
     if (rc == GLLMQ_OK) {
+        hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->mm8_part), sizeof(float) * gq::MM8_SPLIT_PART_FLOATS);
+        if (he == hipSuccess) he = hipMalloc(reinterpret_cast<void **>(&ctx->mm8_arrive), sizeof(uint32_t) * gq::MM8_SPLIT_MAX_LISTS);
+        if (he == hipSuccess) he = hipMemset(ctx->mm8_arrive, 0, sizeof(uint32_t) * gq::MM8_SPLIT_MAX_LISTS);
+        if (he != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "K-split scratch: %s", hipGetErrorString(he));
+    }
+    if (rc == GLLMQ_OK) {
         static const uint32_t kRows[8] = { 0, 1, 2, 3, 4, 5, 6, 7 };
         hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->identity_rows), sizeof kRows);
         if (he == hipSuccess) he = hipMemcpy(ctx->identity_rows, kRows, sizeof kRows, hipMemcpyHostToDevice);
@@ -674,6 +722,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     ctx->tune_moe_job_waves = tune("GLLMQ_MOE_JOB_WAVES");
     ctx->tune_moe_slices = tune("GLLMQ_MOE_SLICES");
     if (const char *v = getenv("GLLMQ_MM8_AREG")) ctx->mm8_areg_on = (v[0] != '0');
+    if (const char *v = getenv("GLLMQ_MM8_KSPLIT")) ctx->mm8_ksplit_max = static_cast<uint32_t>(std::max(0, atoi(v)));
     if (const char *v = getenv("GLLMQ_MM8_Q6K_MIN_M")) ctx->mm8_q6k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
     if (const char *v = getenv("GLLMQ_MM8_Q5K_MIN_M")) ctx->mm8_q5k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
     if (const char *v = getenv("GLLMQ_MM8_Q8_0_MIN_M")) ctx->mm8_q8_0_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
@@ -694,6 +743,8 @@ void gllmq_destroy(gllmq_ctx *ctx)
     if (!ctx) return;
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->identity_rows) (void)hipFree(ctx->identity_rows);
+    if (ctx->mm8_part) (void)hipFree(ctx->mm8_part);
+    if (ctx->mm8_arrive) (void)hipFree(ctx->mm8_arrive);
     if (ctx->argmax_keys) (void)hipFree(ctx->argmax_keys);
     if (ctx->ffn_scratch) (void)hipFree(ctx->ffn_scratch);
     if (ctx->mmf_partial) (void)hipFree(ctx->mmf_partial);

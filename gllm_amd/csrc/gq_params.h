@@ -50,7 +50,17 @@ struct Mm8Params {
     // gated form only (gq_mm8_glu_*): the up rows, and whether the gate passes a ReLU ahead of the SiLU
     const uint8_t *w2;
     uint32_t glu_relu;
+    // K split (plain kernels only; 0 or 1 = off): `ksplit` consecutive workgroups share a tile list,
+    // workgroup s of them multiplies blocks [s * kslice_groups, (s + 1) * kslice_groups) of every
+    // row and writes its sums to part[s][m][n]; the one that finishes last adds the slices up in
+    // order (arrive[tile list] counts the finished ones and is left at 0).
+    uint32_t ksplit, kslice_groups;
+    float *part;
+    uint32_t *arrive;
 };
+
+constexpr uint32_t MM8_SPLIT_MAX_LISTS = 256;        // tile lists (workgroups per slice) of a K-split launch
+constexpr uint32_t MM8_SPLIT_PART_FLOATS = 1u << 20; // slices * activation rows * n of a K-split launch (4 MiB)
 
 constexpr int MM8_WAVES = 8;
 constexpr int MM8_THREADS = 64 * MM8_WAVES;

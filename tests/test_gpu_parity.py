@@ -268,7 +268,8 @@ def test_bf16_activation_mode(hip, torch, oracle, dtype, m):
                                  {"GLLMQ_GEMV_F32": "1", "GLLMQ_MM8": "0", "GLLMQ_MMF": "0"},
                                  {"GLLMQ_MM8_Q6K_MIN_M": "1", "GLLMQ_MM8_Q5K_MIN_M": "1", "GLLMQ_MM8_Q8_0_MIN_M": "1"},
                                  {"GLLMQ_MM8_Q6K_MIN_M": "0", "GLLMQ_MM8_Q5K_MIN_M": "0", "GLLMQ_MM8_Q8_0_MIN_M": "0"},
-                                 {"GLLMQ_MMF_SMALL_MIN_M": "0"}])
+                                 {"GLLMQ_MMF_SMALL_MIN_M": "0"}, {"GLLMQ_MM8_KSPLIT": "0"},
+                                 {"GLLMQ_MM8_KSPLIT": "2", "GLLMQ_MMF_SMALL_MIN_M": "0"}])
 def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
     """The kernels the default dispatch does not pick: integer-dot GEMV for Q4_K, 8-row passes
     for more than 8 rows, the f32 multiply-add flavour, Q5_K and Q6_K on the matrix cores from one
@@ -314,6 +315,32 @@ def test_random_shapes_sweep(hip, torch, oracle):
         want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
         got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
         check_close(got, want, f"case {case} dtype={dtype} m={m} n={n} k={k}")
+
+
+def test_k_split_of_the_8_row_kernels(torch, oracle, monkeypatch):
+    """Few weight rows (tiles for at most half of the CUs) and at least two passes per tile: several
+    workgroups share a tile, each takes a slice of K, the last one to finish adds the slices up.
+    Every format from one row up, 2 to 8 slices, slices of unequal length, a partial last block,
+    ragged n, a repeat of every call (the arrival counters must be back at zero; the sum order is
+    fixed, so the repeat is bit-identical) with an unsplit call in between."""
+    from gllm_amd.backend import HipBackend
+    for k_ in ("GLLMQ_MM8_Q6K_MIN_M", "GLLMQ_MM8_Q5K_MIN_M", "GLLMQ_MM8_Q8_0_MIN_M"):
+        monkeypatch.setenv(k_, "1")
+    monkeypatch.setenv("GLLMQ_MMF_SMALL_MIN_M", "0")
+    hip2 = HipBackend(0)
+    cases = [(1, 4096, 4096), (2, 1024, 4096), (1, 100, 14336), (4, 512, 8192), (8, 33, 6144), (3, 2048, 2048 + 1024),
+             (5, 64, 16384), (1, 4000, 4096 + 2048), (2, 31, 4096 + 256 * 5 - 8), (8, 4096, 4096), (6, 300, 11008)]
+    for dtype in ALL:
+        for m, n, k in cases:
+            print(f"k split dtype={dtype} m={m} n={n} k={k}", flush=True)
+            w, x = random_weight(dtype, n, k, seed=m * 100 + n), random_activations(m, k, seed=k % 997)
+            want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+            got = gpu_matmul(hip2, torch, w, x, dtype, m, n, k)
+            check_close(got, want, f"k split dtype={dtype} m={m} n={n} k={k}")
+            w2, x2 = random_weight(dtype, 8200, 256, seed=5), random_activations(1, 256, seed=6)
+            gpu_matmul(hip2, torch, w2, x2, dtype, 1, 8200, 256)
+            again = gpu_matmul(hip2, torch, w, x, dtype, m, n, k)
+            assert np.array_equal(got.view(np.uint32), again.view(np.uint32)), f"repeat differs: dtype={dtype} m={m} n={n} k={k}"
 
 
 def test_q8_0_matrix_core_shapes(hip, torch, oracle):
