@@ -351,8 +351,14 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     // several workgroups per CU.  Two rows of more than 9728 elements do not (one workgroup of
     // four waves per CU: 35 against 25 us for Q6_K 14336 -> 4096), so they come here.
     const bool gemv_cramped = 848u * m * ((k + 255) / 256) > 64u * 1024u;
-    if (kind == MM8_Q6K && (ctx->mm8_q6k_min_m == 0 || (m < ctx->mm8_q6k_min_m && !gemv_cramped))) return -1;
-    if (kind == MM8_Q5K && !glu && (ctx->mm8_q5k_min_m == 0 || m < ctx->mm8_q5k_min_m)) return -1;
+    // One row of 40 blocks and more over few weight rows (a down projection): the K split below
+    // gives every CU a slice, and the Q5_K and Q6_K kernels here then beat the GEMV, which walks
+    // such a row with three or four waves (11008 -> 4096: Q6_K 15.5 against 17.6 us, Q5_K 13.2
+    // against 16.6; 14336 -> 4096: 17.5 against 17.7 and 14.5 against 15.5).
+    const bool long_single = m == 1 && (k + 255) / 256 >= 40 && ctx->mm8_ksplit_max > 1 &&
+                             ((n + 31) / 32) * 2 <= static_cast<size_t>(ctx->num_cus);
+    if (kind == MM8_Q6K && (ctx->mm8_q6k_min_m == 0 || (m < ctx->mm8_q6k_min_m && !gemv_cramped && !long_single))) return -1;
+    if (kind == MM8_Q5K && !glu && (ctx->mm8_q5k_min_m == 0 || (m < ctx->mm8_q5k_min_m && !long_single))) return -1;
     if (kind == MM8_Q8_0 && (ctx->mm8_q8_0_min_m == 0 || (m < ctx->mm8_q8_0_min_m && !gemv_cramped))) return -1;
     if (kind == MM8_Q8_0 && k < 256) return -1; // its fetch window is one whole group of 8 blocks
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors

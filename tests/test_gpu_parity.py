@@ -361,10 +361,13 @@ def test_q8_0_matrix_core_shapes(hip, torch, oracle):
 @pytest.mark.parametrize("dtype", ALL)
 def test_long_rows_one_and_two_activation_rows(hip, torch, oracle, dtype):
     """Long rows with one and two activation rows (the waves of a GEMV workgroup share a row, rows
-    past 16384 elements take several launches; two rows past 9728 elements take the 8-row kernel):
-    whole groups, a partial last group, ragged n, up to 65536 elements."""
+    past 16384 elements take several launches; two rows past 9728 elements take the 8-row kernel,
+    and so does one Q5_K or Q6_K row of 40 blocks and more over few weight rows, K split across
+    workgroups): whole groups, a partial last group, ragged n, up to 65536 elements, two down
+    projection shapes."""
     step = 32 if dtype == Q8_0 else 256
-    for n, k in [(257, 8192), (70, 14336), (33, 11008), (5, 8448 + step), (129, 16384 + 4 * step - 8), (64, 65536)]:
+    for n, k in [(257, 8192), (70, 14336), (33, 11008), (5, 8448 + step), (129, 16384 + 4 * step - 8), (64, 65536),
+                 (4096, 11008), (2000, 10240)]:
         for m in (1, 2):
             print(f"long rows dtype={dtype} n={n} k={k} m={m}", flush=True)
             w, x = random_weight(dtype, n, k, seed=n + m), random_activations(m, k, seed=k % 1000)
