@@ -318,28 +318,41 @@ def run_other(args):
     print(json.dumps(result), flush=True)
 
 
-def cpu_baseline(budget_s: float = 12.0):
-    """The oracle's reference-faithful matmul (per-block decode, f32 multiply-add) on the host
-    cores, on the same shape with the same generator, repeated for about `budget_s` seconds."""
+def cpu_baseline(budget_s: float = 12.0, simd_budget_s: float = 6.0):
+    """The oracle's reference-faithful matmul (scalar per-block decode, f32 multiply-add: what the
+    reference ships for K-quants) on the host cores, on the same shape with the same generator,
+    repeated for about `budget_s` seconds; beside it, under "avx2", the oracle's vectorised flavour
+    (AVX2 decode, eight-lane f32 sums) for `simd_budget_s` seconds where the host has AVX2."""
     from gllm_amd.ggml import row_bytes
     from gllm_amd.synth import random_activations, random_weight
     from oracle import cref
     threads = max(1, min(os.cpu_count() or 1, 16))
     w = random_weight(DTYPE, N, K_DIM, seed=0)
     x = random_activations(M, K_DIM, seed=0)
-    cref.quantized_matmul(w, x, DTYPE, M, N, K_DIM, acc=cref.ACC_F32, threads=threads)
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        cref.quantized_matmul(w, x, DTYPE, M, N, K_DIM, acc=cref.ACC_F32, threads=threads)
-        reps += 1
-        dt = time.perf_counter() - t0
-        if dt > budget_s or reps >= 20000:
-            break
     bytes_per_call = N * row_bytes(DTYPE, K_DIM) + M * K_DIM * 4 + M * N * 4
-    return {"value": round(bytes_per_call * reps / dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-            "us_per_call": round(dt / reps * 1e6, 1),
-            "sample": f"{reps} calls of the same 1x{K_DIM}x{N} Q4_K matmul (C restatement of the reference's "
-                      f"scalar decode + f32 FMA, rows split over {threads} threads) in {dt:.1f} s"}
+
+    def leg(fn, budget):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt > budget or reps >= 20000:
+                return reps, dt
+
+    reps, dt = leg(lambda: cref.quantized_matmul(w, x, DTYPE, M, N, K_DIM, acc=cref.ACC_F32, threads=threads), budget_s)
+    out = {"value": round(bytes_per_call * reps / dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+           "us_per_call": round(dt / reps * 1e6, 1),
+           "sample": f"{reps} calls of the same 1x{K_DIM}x{N} Q4_K matmul (C restatement of the reference's "
+                     f"scalar decode + f32 FMA, rows split over {threads} threads) in {dt:.1f} s"}
+    if cref.have_avx2():
+        reps, dt = leg(lambda: cref.quantized_matmul_avx2(w, x, DTYPE, M, N, K_DIM, threads=threads), simd_budget_s)
+        out["avx2"] = {"value": round(bytes_per_call * reps / dt / 1e9, 3), "unit": "GB/s", "cores": threads,
+                       "us_per_call": round(dt / reps * 1e6, 1),
+                       "sample": f"{reps} calls of the same matmul with the oracle's AVX2 decode and eight-lane f32 sums "
+                                 f"over {threads} threads in {dt:.1f} s"}
+    return out
 
 
 def main():

@@ -252,6 +252,152 @@ int64_t gq_argmax_token(const float *logits, size_t n)
     return best;
 }
 
+/* ------------------------------------------------- vectorised flavour (AVX2) */
+/* The same decoders eight elements at a time, and a dot product over eight-lane partial sums:
+ * the "AVX2 / AVX-512" side of the CPU baseline.  Every decoded value equals the scalar
+ * decoder's bit for bit (the products d*sc*q are exact in f32, so a fused multiply-subtract
+ * rounds like the scalar multiply then subtract); only the summation order of the dot product
+ * differs from GQ_ACC_F32. */
+#if defined(__AVX2__) && defined(__FMA__)
+#include <immintrin.h>
+#define GQ_HAVE_AVX2 1
+
+static inline __m256 u8x8_to_ps(__m128i bytes) { return _mm256_cvtepi32_ps(_mm256_cvtepu8_epi32(bytes)); }
+
+static void dequant_block_q4_k_avx2(const uint8_t *blk, float *out)
+{
+    const float d = gq_f16_to_f32(rd16(blk)), dmin = gq_f16_to_f32(rd16(blk + 2));
+    const __m128i low4 = _mm_set1_epi8(0x0F);
+    for (int g = 0; g < 4; ++g) {
+        uint8_t sc0, m0, sc1, m1;
+        gq_scale_min_k4(2 * g, blk + 4, &sc0, &m0);
+        gq_scale_min_k4(2 * g + 1, blk + 4, &sc1, &m1);
+        const __m256 d0 = _mm256_set1_ps(d * (float)sc0), n0 = _mm256_set1_ps(dmin * (float)m0);
+        const __m256 d1 = _mm256_set1_ps(d * (float)sc1), n1 = _mm256_set1_ps(dmin * (float)m1);
+        for (int l = 0; l < 32; l += 8) {
+            const __m128i q = _mm_loadl_epi64((const __m128i *)(blk + 16 + 32 * g + l));
+            const __m128i lo = _mm_and_si128(q, low4), hi = _mm_and_si128(_mm_srli_epi16(q, 4), low4);
+            _mm256_storeu_ps(out + 64 * g + l, _mm256_fmsub_ps(d0, u8x8_to_ps(lo), n0));
+            _mm256_storeu_ps(out + 64 * g + 32 + l, _mm256_fmsub_ps(d1, u8x8_to_ps(hi), n1));
+        }
+    }
+}
+
+static void dequant_block_q5_k_avx2(const uint8_t *blk, float *out)
+{
+    const float d = gq_f16_to_f32(rd16(blk)), dmin = gq_f16_to_f32(rd16(blk + 2));
+    const __m128i low4 = _mm_set1_epi8(0x0F), one = _mm_set1_epi8(1);
+    for (int g = 0; g < 4; ++g) {
+        uint8_t sc0, m0, sc1, m1;
+        gq_scale_min_k4(2 * g, blk + 4, &sc0, &m0);
+        gq_scale_min_k4(2 * g + 1, blk + 4, &sc1, &m1);
+        const __m256 d0 = _mm256_set1_ps(d * (float)sc0), n0 = _mm256_set1_ps(dmin * (float)m0);
+        const __m256 d1 = _mm256_set1_ps(d * (float)sc1), n1 = _mm256_set1_ps(dmin * (float)m1);
+        for (int l = 0; l < 32; l += 8) {
+            const __m128i q = _mm_loadl_epi64((const __m128i *)(blk + 48 + 32 * g + l));
+            const __m128i qh = _mm_loadl_epi64((const __m128i *)(blk + 16 + l));
+            /* bit 2g of qh is the fifth bit of the low-nibble element, bit 2g+1 of the high one */
+            const __m128i b0 = _mm_slli_epi16(_mm_and_si128(_mm_srli_epi16(qh, 2 * g), one), 4);
+            const __m128i b1 = _mm_slli_epi16(_mm_and_si128(_mm_srli_epi16(qh, 2 * g + 1), one), 4);
+            const __m128i lo = _mm_or_si128(_mm_and_si128(q, low4), b0);
+            const __m128i hi = _mm_or_si128(_mm_and_si128(_mm_srli_epi16(q, 4), low4), b1);
+            _mm256_storeu_ps(out + 64 * g + l, _mm256_fmsub_ps(d0, u8x8_to_ps(lo), n0));
+            _mm256_storeu_ps(out + 64 * g + 32 + l, _mm256_fmsub_ps(d1, u8x8_to_ps(hi), n1));
+        }
+    }
+}
+
+static void dequant_block_q6_k_avx2(const uint8_t *blk, float *out)
+{
+    const int8_t *sc = (const int8_t *)(blk + 192);
+    const float d = gq_f16_to_f32(rd16(blk + 208));
+    const __m128i low4 = _mm_set1_epi8(0x0F), two = _mm_set1_epi8(3);
+    const __m256 off = _mm256_set1_ps(32.0f);
+    for (int h = 0; h < 2; ++h)
+        for (int l = 0; l < 32; l += 8) {
+            const int is = 8 * h + l / 16;
+            const __m128i a = _mm_loadl_epi64((const __m128i *)(blk + 64 * h + l));
+            const __m128i b = _mm_loadl_epi64((const __m128i *)(blk + 64 * h + 32 + l));
+            const __m128i hb = _mm_loadl_epi64((const __m128i *)(blk + 128 + 32 * h + l));
+            const __m128i q1 = _mm_or_si128(_mm_and_si128(a, low4), _mm_slli_epi16(_mm_and_si128(hb, two), 4));
+            const __m128i q2 = _mm_or_si128(_mm_and_si128(b, low4), _mm_slli_epi16(_mm_and_si128(_mm_srli_epi16(hb, 2), two), 4));
+            const __m128i q3 = _mm_or_si128(_mm_and_si128(_mm_srli_epi16(a, 4), low4), _mm_slli_epi16(_mm_and_si128(_mm_srli_epi16(hb, 4), two), 4));
+            const __m128i q4 = _mm_or_si128(_mm_and_si128(_mm_srli_epi16(b, 4), low4), _mm_slli_epi16(_mm_and_si128(_mm_srli_epi16(hb, 6), two), 4));
+            /* d * sc * (q - 32): q - 32 is exact, both products are exact in f32 */
+            float *o = out + 128 * h + l;
+            _mm256_storeu_ps(o, _mm256_mul_ps(_mm256_set1_ps(d * (float)sc[is + 0]), _mm256_sub_ps(u8x8_to_ps(q1), off)));
+            _mm256_storeu_ps(o + 32, _mm256_mul_ps(_mm256_set1_ps(d * (float)sc[is + 2]), _mm256_sub_ps(u8x8_to_ps(q2), off)));
+            _mm256_storeu_ps(o + 64, _mm256_mul_ps(_mm256_set1_ps(d * (float)sc[is + 4]), _mm256_sub_ps(u8x8_to_ps(q3), off)));
+            _mm256_storeu_ps(o + 96, _mm256_mul_ps(_mm256_set1_ps(d * (float)sc[is + 6]), _mm256_sub_ps(u8x8_to_ps(q4), off)));
+        }
+}
+
+static void dequant_block_q8_0_avx2(const uint8_t *blk, float *out)
+{
+    const __m256 d = _mm256_set1_ps(gq_f16_to_f32(rd16(blk)));
+    for (int i = 0; i < 32; i += 8) {
+        const __m128i q = _mm_loadl_epi64((const __m128i *)(blk + 2 + i));
+        _mm256_storeu_ps(out + i, _mm256_mul_ps(d, _mm256_cvtepi32_ps(_mm256_cvtepi8_epi32(q))));
+    }
+}
+
+/* sum of w[e] * x[e], e < len: four eight-lane partial sums over whole groups of 32, the lanes
+ * added pairwise at the end, the tail one element at a time */
+static float dot_avx2(const float *w, const float *x, size_t len, float carry)
+{
+    __m256 a0 = _mm256_setzero_ps(), a1 = a0, a2 = a0, a3 = a0;
+    size_t e = 0;
+    for (; e + 32 <= len; e += 32) {
+        a0 = _mm256_fmadd_ps(_mm256_loadu_ps(w + e), _mm256_loadu_ps(x + e), a0);
+        a1 = _mm256_fmadd_ps(_mm256_loadu_ps(w + e + 8), _mm256_loadu_ps(x + e + 8), a1);
+        a2 = _mm256_fmadd_ps(_mm256_loadu_ps(w + e + 16), _mm256_loadu_ps(x + e + 16), a2);
+        a3 = _mm256_fmadd_ps(_mm256_loadu_ps(w + e + 24), _mm256_loadu_ps(x + e + 24), a3);
+    }
+    const __m256 s = _mm256_add_ps(_mm256_add_ps(a0, a1), _mm256_add_ps(a2, a3));
+    __m128 q = _mm_add_ps(_mm256_castps256_ps128(s), _mm256_extractf128_ps(s, 1));
+    q = _mm_add_ps(q, _mm_movehl_ps(q, q));
+    q = _mm_add_ss(q, _mm_shuffle_ps(q, q, 1));
+    float sum = carry + _mm_cvtss_f32(q);
+    for (; e < len; ++e) sum += w[e] * x[e];
+    return sum;
+}
+
+static block_fn codec_avx2_for(uint32_t t)
+{
+    switch (t) {
+    case GQ_TYPE_Q4_K: return dequant_block_q4_k_avx2;
+    case GQ_TYPE_Q5_K: return dequant_block_q5_k_avx2;
+    case GQ_TYPE_Q6_K: return dequant_block_q6_k_avx2;
+    case GQ_TYPE_Q8_0: return dequant_block_q8_0_avx2;
+    default: return NULL;
+    }
+}
+#else
+#define GQ_HAVE_AVX2 0
+#endif
+
+int gq_have_avx2(void)
+{
+#if GQ_HAVE_AVX2
+    return __builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma");
+#else
+    return 0;
+#endif
+}
+
+int gq_dequant_block_avx2(uint32_t t, const uint8_t *blk, float *out)
+{
+#if GQ_HAVE_AVX2
+    block_fn f = codec_avx2_for(t);
+    if (!f || !gq_have_avx2()) return GQ_ERR_UNIMPLEMENTED;
+    f(blk, out);
+    return GQ_OK;
+#else
+    (void)t; (void)blk; (void)out;
+    return GQ_ERR_UNIMPLEMENTED;
+#endif
+}
+
 /* ------------------------------------------------------------------- matmul */
 typedef struct {
     const uint8_t *w;
@@ -259,7 +405,7 @@ typedef struct {
     float *y;
     uint32_t t;
     size_t m, n, k;
-    int mode; /* GQ_ACC_F32, GQ_ACC_F64, 2 = bf16 operands + f64 sum */
+    int mode; /* GQ_ACC_F32, GQ_ACC_F64, 2 = bf16 operands + f64 sum, 3 = vectorised decode and f32 dot */
     size_t row0, row1;
 } mm_job;
 
@@ -267,6 +413,9 @@ static void *mm_worker(void *arg)
 {
     const mm_job *j = (const mm_job *)arg;
     block_fn f = codec_for(j->t);
+#if GQ_HAVE_AVX2
+    if (j->mode == 3) f = codec_avx2_for(j->t);
+#endif
     const size_t bs = gq_block_size(j->t), bb = gq_block_bytes(j->t);
     const size_t nblk = (j->k + bs - 1) / bs;
     const size_t stride = nblk * bb;
@@ -284,6 +433,12 @@ static void *mm_worker(void *arg)
                 for (size_t e = 0; e < len; ++e) tmp[e] = bf16_round(tmp[e]);
             for (size_t i = 0; i < j->m; ++i) {
                 const float *xi = j->x + i * j->k + k0;
+#if GQ_HAVE_AVX2
+                if (j->mode == 3) {
+                    accf[i] = dot_avx2(tmp, xi, len, accf[i]);
+                    continue;
+                }
+#endif
                 if (j->mode == GQ_ACC_F32) {
                     float a = accf[i];
                     for (size_t e = 0; e < len; ++e) a += tmp[e] * xi[e];
@@ -300,7 +455,7 @@ static void *mm_worker(void *arg)
             }
         }
         for (size_t i = 0; i < j->m; ++i)
-            j->y[i * j->n + r] = (j->mode == GQ_ACC_F32) ? accf[i] : (float)accd[i];
+            j->y[i * j->n + r] = (j->mode == GQ_ACC_F32 || j->mode == 3) ? accf[i] : (float)accd[i];
     }
     free(accf);
     free(accd);
@@ -348,6 +503,13 @@ int gq_quantized_matmul_bf16(const uint8_t *w, const float *x, float *y, uint32_
                              size_t n, size_t k, int threads)
 {
     return mm_run(w, x, y, t, m, n, k, 2, threads);
+}
+
+int gq_quantized_matmul_avx2(const uint8_t *w, const float *x, float *y, uint32_t t, size_t m,
+                             size_t n, size_t k, int threads)
+{
+    if (!gq_have_avx2()) return GQ_ERR_UNIMPLEMENTED;
+    return mm_run(w, x, y, t, m, n, k, 3, threads);
 }
 
 /* ---------------------------------------------------------------------- MoE */

@@ -29,6 +29,9 @@
  *                                         summation order, threading and any internal
  *                                         activation handling are PARITY UNPINNED (no
  *                                         test or fixture of the reference exercises it)
+ *   gq_quantized_matmul_avx2            : the vectorised baseline flavour; decoders pinned bitwise
+ *                                         against the scalar ones, the sum against the f64 yardstick;
+ *                                         same status as gq_quantized_matmul otherwise
  *   gq_quant_gather                     : unscaled lookups are pinned with gq_dequantize (a row
  *                                         gather of its output); where the embedding scale is
  *                                         applied is PARITY UNPINNED (the op runs in generated
@@ -116,6 +119,15 @@ int gq_quantized_matmul(const uint8_t *w, const float *x, float *y, uint32_t ggm
 /* Same contraction with both operands rounded to bf16 (round-to-nearest-even) before
  * the multiply and products summed in double: yardstick for the MFMA path. */
 int gq_quantized_matmul_bf16(const uint8_t *w, const float *x, float *y, uint32_t ggml_dtype,
+                             size_t m, size_t n, size_t k, int threads);
+
+/* The vectorised flavour of the CPU baseline: the block decoders eight elements at a time
+ * (AVX2; every decoded value equal to the scalar decoder's bit for bit) and an f32 dot product
+ * over eight-lane partial sums.  GQ_ERR_UNIMPLEMENTED when the build or the host has no AVX2+FMA.
+ * gq_dequant_block_avx2 decodes one block with those decoders (for the bit-equality test). */
+int gq_have_avx2(void);
+int gq_dequant_block_avx2(uint32_t ggml_dtype, const uint8_t *blk, float *out);
+int gq_quantized_matmul_avx2(const uint8_t *w, const float *x, float *y, uint32_t ggml_dtype,
                              size_t m, size_t n, size_t k, int threads);
 
 /* src/moe/routing.rs:290-302 */

@@ -207,3 +207,51 @@ def test_moe_ffn_equals_dense_masked_evaluation(oracle, relu_gate):
         h = (g / (1 + np.exp(-g))) * u
         want += gate_w[:, e:e + 1] * (h @ dn_f[e].T)
     assert rel_l2(got, want) < 2e-6
+
+
+# ------------------------------------------- the vectorised flavour of the CPU baseline
+@pytest.mark.parametrize("dtype", ALL)
+def test_avx2_decoders_equal_the_scalar_ones_bit_for_bit(oracle, dtype):
+    """Random blocks (every byte pattern of quants and scales; f16 scales over normal, subnormal,
+    zero and negative values) and blocks of all-0x00 / all-0xFF quants."""
+    if not oracle.have_avx2():
+        pytest.skip("host without AVX2+FMA")
+    bb = oracle.block_bytes(dtype)
+    rng = np.random.default_rng(dtype)
+    blocks = rng.integers(0, 256, (400, bb), dtype=np.uint8)
+    d_off = {Q8_0: [0], Q4_K: [0, 2], Q5_K: [0, 2], Q6_K: [208]}[dtype]
+    special = np.array([0x0000, 0x8000, 0x0001, 0x03FF, 0x0400, 0x3C00, 0xBC00, 0x7BFF, 0x2E66], np.uint16)
+    for i in range(blocks.shape[0]):
+        for off in d_off:
+            h = special[rng.integers(0, special.size)] if i % 4 == 0 else np.float16(rng.uniform(-0.05, 0.05)).view(np.uint16)
+            blocks[i, off:off + 2] = np.frombuffer(np.uint16(h).tobytes(), np.uint8)
+    blocks[1, [j for j in range(bb) if j not in sum(([o, o + 1] for o in d_off), [])]] = 0x00
+    blocks[2, [j for j in range(bb) if j not in sum(([o, o + 1] for o in d_off), [])]] = 0xFF
+    for blk in blocks:
+        want = oracle.dequantize(blk, dtype)
+        got = oracle.dequant_block_avx2(blk, dtype)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_avx2_matmul_matches_the_float64_yardstick(oracle, dtype):
+    """Whole blocks, a partial last block (the tail runs one element at a time), several activation
+    rows, threads; unit vectors return weight columns bit for bit (every other term is +-0)."""
+    if not oracle.have_avx2():
+        pytest.skip("host without AVX2+FMA")
+    step = 32 if dtype == Q8_0 else 256
+    for m, n, k in [(1, 33, 4096), (3, 17, 2 * step + step // 2 + 4), (2, 5, step)]:
+        w, x = random_weight(dtype, n, k, seed=7), random_activations(m, k, seed=8)
+        want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64)
+        for threads in (1, 3):
+            got = oracle.quantized_matmul_avx2(w, x, dtype, m, n, k, threads=threads)
+            assert rel_l2(got, want) < 1e-6
+            assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
+    n, k = 9, 512
+    w = random_weight(dtype, n, k, seed=4)
+    deq = oracle.dequantize(w, dtype).reshape(n, k)
+    for col in (0, 7, 8, 31, 255, 256, 511):
+        x = np.zeros((1, k), np.float32)
+        x[0, col] = 1.0
+        y = oracle.quantized_matmul_avx2(w, x, dtype, 1, n, k)
+        assert np.array_equal(y[0], deq[:, col])
