@@ -143,7 +143,12 @@ int gllmq_argmax(gllmq_ctx *ctx, const float *logits_dev, size_t rows, size_t n,
  * long that the prepared activations do not fit the LDS of one 8-row pass (K above about
  * 4096..12288, by format and rows).  Q5_K with one row, Q6_K and Q8_0 with one or two, and
  * Q8_0 rows shorter than 256 elements run integer-dot GEMV kernels, two activation rows per
- * pass. */
+ * pass; one Q5_K or Q6_K row of 40 blocks and more over at most 4096 weight rows takes the
+ * matrix-core kernel.  With so few weight rows that their 32-row tiles cover at most half of
+ * the CUs, the matrix-core kernels of up to 8 rows split K across the workgroups of one launch
+ * (the last workgroup of a tile adds the slice sums in slice order); slice sums and arrival
+ * counters live in the context too.  Which scratch a call uses depends on its shape: calls on
+ * one context must not overlap in time. */
 int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev,
                            float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,
                            void *stream);
