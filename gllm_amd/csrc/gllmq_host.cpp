@@ -319,6 +319,9 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
     if (n > 0x7FFFFFFFu || k > 0x7FFFFFFFu || m > 0x7FFFFFFFu)
         return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quantized_matmul: dimension exceeds 2^31-1");
     const size_t rb = gllmq_row_bytes(dtype, k);
+    // the kernels address a workgroup's rows with 32-bit byte offsets from the first of them
+    if (rb > (size_t(1) << 26))
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quantized_matmul: rows of %zu bytes (k=%zu) exceed the supported 64 MiB", rb, k);
     if (w_bytes < n * rb)
         return fail(ctx, GLLMQ_ERR_BAD_SHAPE,
                     "quantized_matmul: weight buffer has %zu bytes, n=%zu rows of k=%zu need %zu", w_bytes, n, k,
@@ -456,6 +459,8 @@ int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
     const uint32_t row_tiles = static_cast<uint32_t>((n + 255) / 256);
     if (row_tiles > kMmfMaxRowTiles) return -1;
+    // the GEMM kernels address weight rows with 32-bit byte offsets from the start of the matrix
+    if (n * gllmq_row_bytes(f.dtype, k) > 0xFFFFFFFFull) return -1;
     uint32_t ksplit = std::max(1u, static_cast<uint32_t>(ctx->num_cus) / row_tiles);
     if (ctx->tune_mmf_ksplit) ksplit = ctx->tune_mmf_ksplit;
     ksplit = std::min(ksplit, groups);

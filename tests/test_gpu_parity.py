@@ -456,3 +456,35 @@ def test_unsupported_formats_are_errors(hip, torch):
     with pytest.raises(OtherError):  # weight buffer shorter than n rows
         hip.quantized_matmul(w, x, y, Q8_0, 1, 4, 64)
     hip.quantized_matmul(w, x, y, Q8_0, 0, 4, 32)  # m = 0: nothing to do
+
+
+def test_weight_matrix_larger_than_4_gib(hip, torch, oracle):
+    """A Q8_0 matrix of 4.6 GB: rows that start past byte offset 2^32 must be addressed with
+    64-bit arithmetic on every kernel path (1, 2, 5 and 16 activation rows; the GEMM addresses rows
+    with 32-bit offsets from the start of the matrix and must leave such a matrix to the other
+    kernels).  Weights are made on the device; sampled rows on both sides of the 4 GiB line are
+    checked against the oracle."""
+    dtype, n, k = Q8_0, 132000, 32768
+    rb = (k // 32) * 34
+    assert n * rb > 2**32
+    g = torch.Generator(device="cuda")
+    g.manual_seed(77)
+    wd = torch.randint(0, 256, (n * rb,), dtype=torch.uint8, device="cuda", generator=g)
+    blocks = wd.view(-1, 34)
+    d = (torch.rand(blocks.shape[0], 1, device="cuda", generator=g) * 0.049 + 0.001).to(torch.float16)
+    blocks[:, 0:2] = d.view(torch.uint8)
+    del d
+    first_past = 2**32 // rb + 1
+    rows = [0, 1, 31, 4097, first_past - 2, first_past - 1, first_past, first_past + 1, first_past + 300, n - 33, n - 2, n - 1]
+    w_rows = torch.stack([wd[r * rb:(r + 1) * rb] for r in rows]).cpu().numpy()
+    for m in (1, 2, 5, 16):
+        print(f"4 GiB matrix m={m}", flush=True)
+        x = random_activations(m, k, seed=m)
+        xd = torch.from_numpy(x).cuda()
+        yd = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+        hip.quantized_matmul(wd, xd, yd, dtype, m, n, k)
+        torch.cuda.synchronize()
+        got = yd[:, rows].cpu().numpy()
+        want = oracle.quantized_matmul(w_rows, x, dtype, m, len(rows), k, acc=oracle.ACC_F64, threads=4)
+        check_close(got, want, f"4 GiB matrix m={m}")
+        assert not bool(torch.isnan(yd).any())
