@@ -439,7 +439,11 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         if (ksplit > 1) grid = std::min(grid, gq::MM8_SPLIT_MAX_LISTS);
         P.grid = grid; // workgroups per slice: launch index = tile list * ksplit + slice
         hipFunction_t fn = glu ? ctx->mm8_glu[gi][pi][ei] : ctx->mm8[kind][pi][ei];
-        if (pi <= 1 && ppt <= 2 && ctx->mm8_areg_on)
+        // The register-resident variants are compiled for a fixed number of passes per tile and
+        // take a tile's pass from the item's position in the register ring; a last K slice with
+        // fewer passes than the others would break that, so such a split runs the LDS variants.
+        const bool even_slices = ksplit == 1 || ppt_row % slice_passes == 0;
+        if (pi <= 1 && ppt <= 2 && ctx->mm8_areg_on && even_slices)
             fn = glu ? ctx->mm8_glu_areg[gi][pi][ei][ppt - 1] : ctx->mm8_areg[kind][pi][ei][ppt - 1];
         int rc = launch(ctx, fn, grid * ksplit, 512, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;

@@ -488,3 +488,17 @@ def test_weight_matrix_larger_than_4_gib(hip, torch, oracle):
         want = oracle.quantized_matmul(w_rows, x, dtype, m, len(rows), k, acc=oracle.ACC_F64, threads=4)
         check_close(got, want, f"4 GiB matrix m={m}")
         assert not bool(torch.isnan(yd).any())
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_k_split_with_a_shorter_last_slice(hip, torch, oracle, dtype):
+    """K slices of two passes and a last slice of one (an odd number of 8-block passes per tile),
+    several tiles per workgroup: the variants that keep a wave's activation operands in registers
+    are compiled for one number of passes per tile and must not run such a launch (they gave wrong
+    sums for every tile after a workgroup's first)."""
+    for m, n, k in [(4, 4096, 13824), (4, 4096, 14336 - 256), (3, 2048, 9728), (4, 1024, 5632), (4, 3000, 13824), (2, 4096, 13824)]:
+        print(f"uneven k slices dtype={dtype} m={m} n={n} k={k}", flush=True)
+        w, x = random_weight(dtype, n, k, seed=276), random_activations(m, k, seed=277)
+        want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+        got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+        check_close(got, want, f"uneven k slices dtype={dtype} m={m} n={n} k={k}")
