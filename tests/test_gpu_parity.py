@@ -502,3 +502,25 @@ def test_k_split_with_a_shorter_last_slice(hip, torch, oracle, dtype):
         want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
         got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
         check_close(got, want, f"uneven k slices dtype={dtype} m={m} n={n} k={k}")
+
+
+def test_few_weight_rows_long_rows_sweep(hip, torch, oracle):
+    """A hundred seeded shapes where the K split of the 8-row kernels and the long-row dispatch
+    decide: up to 5000 weight rows (among them 2048 and 4096 exactly: whole rounds of workgroups),
+    rows of 8 to 71 blocks with and without a partial last one, 1 to 33 activation rows; every
+    call twice, the repeat bit-identical (sums meet in a fixed order, counters return to zero)."""
+    rng = np.random.default_rng(23)
+    for case in range(100):
+        dtype = ALL[case % len(ALL)]
+        m = int(rng.choice([1, 1, 1, 2, 2, 3, 4, 5, 7, 8, 9, 16, 33]))
+        n = int(rng.choice([rng.integers(1, 64), rng.integers(64, 1024), rng.integers(1024, 5000), 4096, 2048]))
+        k = int(rng.integers(8, 72)) * 256
+        if rng.random() < 0.3:
+            k -= int(rng.integers(1, 8)) * (4 if dtype != Q8_0 else 32)
+        print(f"few rows sweep case {case}: dtype={dtype} m={m} n={n} k={k}", flush=True)
+        w, x = random_weight(dtype, n, k, seed=case), random_activations(m, k, seed=case + 1)
+        want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
+        got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+        check_close(got, want, f"few rows sweep case {case} dtype={dtype} m={m} n={n} k={k}")
+        again = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+        assert np.array_equal(got.view(np.uint32), again.view(np.uint32)), f"repeat differs: case {case}"
