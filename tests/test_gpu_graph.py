@@ -32,6 +32,9 @@ def test_graph_replays_match_eager(hip, torch):
     wd = dev(random_weight(Q6_K, hidden, ffn, seed=4))
     wo = dev(random_weight(Q6_K, vocab, hidden, seed=5))          # lm_head
     wb = dev(random_weight(Q5_K, 512, hidden, seed=6))            # a 16-row GEMM (prepare, GEMM, reduce)
+    ws = dev(random_weight(Q4_K, 256, 8 * hidden, seed=7))        # few rows of long rows: K split across workgroups
+    xs = torch.empty(2, 8 * hidden, device="cuda")
+    ys = torch.empty(2, 256, device="cuda")
     x = torch.empty(1, hidden, device="cuda")
     xb = torch.empty(16, hidden, device="cuda")
     qkv = torch.empty(1, 3 * hidden, device="cuda")
@@ -46,10 +49,12 @@ def test_graph_replays_match_eager(hip, torch):
         hip.quantized_matmul(wo, h, logits, Q6_K, 1, vocab, hidden)
         hip.argmax(logits, tok)
         hip.quantized_matmul(wb, xb, yb, Q5_K, 16, 512, hidden)
+        hip.quantized_matmul(ws, xs, ys, Q4_K, 2, 256, 8 * hidden)
 
     def fill(seed):
         x.copy_(torch.from_numpy(random_activations(1, hidden, seed=seed)))
         xb.copy_(torch.from_numpy(random_activations(16, hidden, seed=seed + 50)))
+        xs.copy_(torch.from_numpy(random_activations(2, 8 * hidden, seed=seed + 90)))
 
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
@@ -65,8 +70,8 @@ def test_graph_replays_match_eager(hip, torch):
         fill(seed)
         step()
         torch.cuda.synchronize()
-        want = [t.clone() for t in (qkv, h, logits, yb, tok)]
-        for t in (qkv, h, logits, yb):
+        want = [t.clone() for t in (qkv, h, logits, yb, ys, tok)]
+        for t in (qkv, h, logits, yb, ys):
             t.fill_(float("nan"))
         tok.fill_(-7)
         # eager work of the program's own between the replays
@@ -74,5 +79,5 @@ def test_graph_replays_match_eager(hip, torch):
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        for got, exp in zip((qkv, h, logits, yb, tok), want):
+        for got, exp in zip((qkv, h, logits, yb, ys, tok), want):
             assert torch.equal(got, exp), f"replay {seed} differs from the eager run"
