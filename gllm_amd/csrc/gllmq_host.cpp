@@ -128,6 +128,7 @@ struct gllmq_ctx {
     hipFunction_t argmax_part = nullptr, argmax_final = nullptr;
     uint64_t *argmax_keys = nullptr;            // [ARGMAX_MAX_ROWS][ARGMAX_MAX_PARTS] scratch of gllmq_argmax
     hipFunction_t dequant_wave = nullptr;       // Q4_K with 16-byte aligned blocks and outputs: one block per wave
+    hipFunction_t dequant_wave_q5k = nullptr;   // the same for Q5_K
     hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1], f32 multiply-add flavour
     hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
     bool gemv_f32 = false;                      // GLLMQ_GEMV_F32=1 selects the f32 flavour
@@ -675,6 +676,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_glu_fn[MM8_Q5K][0], "gq_moe_mm8_glu_q5k_a1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_glu_fn[MM8_Q5K][1], "gq_moe_mm8_glu_q5k_a2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->dequant_wave, "gq_dequant_q4k_wave");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->dequant_wave_q5k, "gq_dequant_q5k_wave");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->argmax_part, "gq_argmax_part");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->argmax_final, "gq_argmax_final");
     if (rc == GLLMQ_OK) {
@@ -791,8 +793,8 @@ int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *
     const uint32_t grid = static_cast<uint32_t>(std::min<uint64_t>(want, static_cast<uint64_t>(ctx->num_cus) * 64));
     struct { const void *b; float *o; uint64_t n; } args = { blocks, out, n_quads };
     hipFunction_t fn = ctx->dequant[format_index(dtype)][vec];
-    // (the same form for Q5_K measured slower than the per-quad kernel: 93 against 88 us)
     if (vec && aligned(blocks, 16) && dtype == T_Q4_K) fn = ctx->dequant_wave;
+    if (vec && aligned(blocks, 16) && dtype == T_Q5_K) fn = ctx->dequant_wave_q5k;
     return launch(ctx, fn, grid, 256, 0, stream, &args, sizeof args);
 }
 
