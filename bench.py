@@ -4,19 +4,28 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 Without --workload (or with gemv_q4k) it measures the headline configuration described
-below.  The other workloads are the remaining baseline configurations, timed the same way
-(one JSON line each): gemv_q4k_4096, gemv_q6k, layer_mix, gemm_m16, gemm_m32, gemm_m64, moe.
+below.  The other workloads are the remaining baseline configurations and the ops around the
+matmul, timed the same way (one JSON line each).
 
 A step is one call of the quantized matmul (m = 1) over one weight matrix.  The weights
-rotate over 16 distinct copies (528 MB) so that no cache level can serve them: every step
-streams its 33 MB from HBM.  The K timed steps are enqueued from one C call on one stream
-and bracketed by events on that stream.  Prints one JSON line.
+rotate over 16 distinct copies (504 MiB) so that no cache level can serve them: every step
+streams its 33 MB from HBM.
+
+Timing method (the same for every workload, whatever --steps and --warmup say):
+  * warm-up: at least max(W, 200) steps AND at least 50 ms of device work;
+  * then a region of exactly K steps is enqueued R times back to back on the stream the
+    kernels run on, with one event between regions (R is at least 50 and grows until the
+    regions cover about 100 ms); nothing synchronises inside that sequence;
+  * `ms_per_step` is the MEDIAN over the R regions of (region time / K); p10 and p90 of the
+    same set, R and the summed region time are printed beside it.
+So `--steps 20 --warmup 5` and the defaults give the same figure.
 """
 from __future__ import annotations
 
 import argparse
 import gc
 import json
+import math
 import os
 import sys
 import time
@@ -30,31 +39,92 @@ DTYPE = 12  # GGML Q4_K
 COPIES = 16
 HBM_PEAK_GBS = 8000.0
 
+WARMUP_MIN_STEPS = 200
+WARMUP_MIN_SECONDS = 0.05
+REGIONS_MIN = 50
+REGIONS_MAX = 500
+REGIONS_TARGET_SECONDS = 0.1
+MAX_TIMED_STEPS = 400_000
 
-# HBM bytes per launch of the timed kernel on this workload, from two counter passes
-# (FETCH_SIZE 16,255.5 KiB and WRITE_SIZE 56.0 KiB per dispatch) scaled by what the same
-# counters read for a plain 32,256 KiB copy kernel (factors 1.9985 and 1.0000).
+
+# HBM bytes per launch of the timed kernel on the headline workload: not measured by this
+# program (hardware counters need the profiler) but by two counter passes of this same command
+# under rocprofv3 (FETCH_SIZE, then WRITE_SIZE, per dispatch), each scaled by what the same
+# counter reads for a plain copy of known size; the summary sits in profiles/ beside the
+# kernel trace.
 TRAFFIC_BYTES_PER_LAUNCH = 33_323_900
+TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy (profiles/)"
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def device_weights(torch, n_rows: int, k: int, copies: int):
-    """Random Q4_K matrices generated on the device: uniform packed bytes, f16 d/dmin in (0.001, 0.05)."""
-    from gllm_amd.ggml import row_bytes
-    total = n_rows * row_bytes(DTYPE, k)
-    out = []
-    g = torch.Generator(device="cuda")
-    g.manual_seed(0)
-    for _ in range(copies):
-        w = torch.randint(0, 256, (total,), dtype=torch.uint8, device="cuda", generator=g)
-        blocks = w.view(-1, 144)
-        d = (torch.rand(blocks.shape[0], 2, device="cuda", generator=g) * 0.049 + 0.001).to(torch.float16)
-        blocks[:, 0:4] = d.view(torch.uint8).view(-1, 4)
-        out.append(w)
-    return out
+def percentile(sorted_vals, q):
+    """Linear-interpolated percentile of an ascending list."""
+    if len(sorted_vals) == 1:
+        return sorted_vals[0]
+    pos = q * (len(sorted_vals) - 1)
+    lo = int(math.floor(pos))
+    hi = min(lo + 1, len(sorted_vals) - 1)
+    return sorted_vals[lo] + (sorted_vals[hi] - sorted_vals[lo]) * (pos - lo)
+
+
+def measure(torch, enqueue_region, steps: int, warmup: int):
+    """Times regions of exactly `steps` steps.  `enqueue_region(r)` enqueues the steps of region
+    number r on torch's current stream (the stream the library launches on, so the events below
+    see exactly those kernels) and returns without synchronising.
+
+    Returns a dict: median / p10 / p90 microseconds per step, regions, timed seconds."""
+    steps = max(1, steps)
+    # warm-up floor: launches and device time, independent of the command line
+    done, t0, r = 0, time.perf_counter(), 0
+    torch.cuda.synchronize()
+    while done < max(warmup, WARMUP_MIN_STEPS) or time.perf_counter() - t0 < WARMUP_MIN_SECONDS:
+        enqueue_region(r)
+        torch.cuda.synchronize()
+        done += steps
+        r += 1
+    # one probe region sizes the number of repeats
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    enqueue_region(r)
+    e1.record()
+    torch.cuda.synchronize()
+    r += 1
+    region_s = max(e0.elapsed_time(e1) * 1e-3, 1e-7)
+    regions = int(min(REGIONS_MAX, max(REGIONS_MIN, math.ceil(REGIONS_TARGET_SECONDS / region_s))))
+    regions = max(10, min(regions, MAX_TIMED_STEPS // steps))
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(regions + 1)]
+    # The launches are enqueued by host code that allocates Python objects; a pass of Python's
+    # cyclic garbage collector in the middle of that (tens of ms with torch loaded) would starve
+    # the GPU and be counted as kernel time.
+    gc.collect()
+    gc.disable()
+    try:
+        torch.cuda.synchronize()
+        events[0].record()
+        for i in range(regions):
+            enqueue_region(r + i)
+            events[i + 1].record()
+        torch.cuda.synchronize()
+    finally:
+        gc.enable()
+    per_step_us = sorted(events[i].elapsed_time(events[i + 1]) * 1e3 / steps for i in range(regions))
+    return {"us": percentile(per_step_us, 0.5), "p10_us": percentile(per_step_us, 0.1),
+            "p90_us": percentile(per_step_us, 0.9), "regions": regions,
+            "timed_region_s": sum(per_step_us) * steps * 1e-6}
+
+
+def timing_fields(t, steps, warmup):
+    return {"steps": steps, "warmup": warmup, "ms_per_step": round(t["us"] / 1e3, 6), "us_per_call": round(t["us"], 3),
+            "p10_us": round(t["p10_us"], 3), "p90_us": round(t["p90_us"], 3), "repeats": t["regions"],
+            "timed_region_s": round(t["timed_region_s"], 4),
+            "timing": "median over `repeats` back-to-back regions of `steps` calls each, events on the launching stream; "
+                      "launch-to-launch gaps included",
+            # what rocprofv3 reports as the kernel's own duration is not visible to events on the
+            # stream; the committed kernel trace holds it
+            "kernel_us": None}
 
 
 BLOCK_BYTES = {8: 34, 12: 144, 13: 176, 14: 210}
@@ -82,9 +152,20 @@ def device_weight_any(torch, g, dtype: int, rows: int, k: int):
     return w
 
 
+def cpu_time(fn, budget_s=8.0, max_reps=200):
+    fn()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > budget_s or reps >= max_reps:
+            return dt / reps, reps, dt
+
+
 def run_other(args):
-    """The baseline configurations other than the headline one.  Same timing method: the timed
-    steps are enqueued back to back on one stream between two events, weights rotate over
+    """The baseline configurations other than the headline one, and the ops on either side of the
+    matmul.  Same timing method; weights (or outputs, for the write-dominated ops) rotate over
     enough copies to exceed the 256 MB Infinity Cache."""
     import numpy as np
     import torch
@@ -92,39 +173,24 @@ def run_other(args):
     from gllm_amd.backend import HipBackend
     from gllm_amd.ggml import row_bytes
     from gllm_amd.synth import random_activations, random_gate_logits, random_weight
-    from oracle import cref
+    from oracle import cref  # the checker, here only as the CPU baseline leg
 
     hip = HipBackend(0)
     g = torch.Generator(device="cuda")
     g.manual_seed(0)
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     threads = max(1, min(os.cpu_count() or 1, 16))
     name = args.workload
-    steps = min(args.steps, 400)
+    steps = args.steps
+    sec = sample = None
+    extra = {}
 
-    def timed(fn, reps):
-        gc.collect()  # no pass of Python's garbage collector inside the timed region
-        gc.disable()
-        try:
-            torch.cuda.synchronize()
-            start.record()
-            for _ in range(reps):
-                fn()
-            stop.record()
-            torch.cuda.synchronize()
-        finally:
-            gc.enable()
-        return start.elapsed_time(stop) * 1e3 / reps  # us
-
-    def cpu_time(fn, budget_s=8.0):
-        fn()
-        reps, t0 = 0, time.perf_counter()
-        while True:
-            fn()
-            reps += 1
-            dt = time.perf_counter() - t0
-            if dt > budget_s or reps >= 200:
-                return dt / reps, reps, dt
+    def rotating(run_one, copies):
+        """Region r runs steps number r * steps .. of an endless rotation over `copies` inputs."""
+        def region(r):
+            base = r * steps
+            for i in range(steps):
+                run_one((base + i) % copies)
+        return region
 
     if name in ("gemv_q4k_4096", "gemv_q6k", "gemm_m16", "gemm_m32", "gemm_m64", "layer_mix", "layer_mix_m4", "layer_mix_m32",
                 "lm_head_q6k"):
@@ -144,19 +210,21 @@ def run_other(args):
         for _ in range(copies):
             sets.append([(device_weight_any(torch, g, dt, n, k), torch.randn(m, k, device="cuda", generator=g),
                           torch.empty(m, n, device="cuda"), dt, m, n, k) for dt, n, k, m in ops])
-        flat = [d for st in sets for d in st]
-        hip.quantized_matmul_batch(flat)
-        reps = max(1, steps // copies)
-        us = timed(lambda: hip.quantized_matmul_batch(flat), reps) / copies
+        # one step = one call of the batch entry point over one set; a region is one C call over
+        # `steps` consecutive sets of the rotation
+        per_set = len(ops)
+        batch = hip.make_batch([d for i in range(steps + copies) for d in sets[i % copies]])
+
+        def region(r):
+            hip.run_batch(batch, ((r * steps) % copies) * per_set, steps * per_set)
         byts = sum(n * row_bytes(dt, k) + m * k * 4 + m * n * 4 for dt, n, k, m in ops)
         flops = sum(2 * m * n * k for dt, n, k, m in ops)
         desc = " + ".join(f"{TAGS[dt]} M={m} K={k} N={n}" for dt, n, k, m in ops)
-        # CPU: the oracle's reference-style path on the same shapes (bounded sample)
-        host = [(random_weight(dt, n, k, seed=i), random_activations(m, k, seed=i), dt, m, n, k)
-                for i, (dt, n, k, m) in enumerate(ops)]
-        if args.no_cpu:
-            sec, sample = None, None
-        else:
+        t = measure(torch, region, steps, args.warmup)
+        if not args.no_cpu:
+            # CPU: the oracle's reference-style path on the same shapes (bounded sample)
+            host = [(random_weight(dt, n, k, seed=i), random_activations(m, k, seed=i), dt, m, n, k)
+                    for i, (dt, n, k, m) in enumerate(ops)]
             sec, creps, cdt = cpu_time(lambda: [cref.quantized_matmul(w, x, dt, m, n, k, acc=cref.ACC_F32, threads=threads)
                                                 for w, x, dt, m, n, k in host])
             sample = f"{creps} passes of the same shapes in {cdt:.1f} s"
@@ -166,35 +234,37 @@ def run_other(args):
         dn = device_weight_any(torch, g, 14, E * H, F)
         x = torch.randn(T, H, device="cuda", generator=g)
         out = torch.empty(T, H, device="cuda")
+        # The router is the library's: logits in, route table out, once per set of logits and
+        # outside the timed region (routing is the gate's job, the metric is the expert matvec).
+        # Capacity factor = number of experts: nothing is dropped (the default 1.25 gives
+        # capacity 1 at 16 tokens over 128 experts and would drop most routes).
         tabs = []
         for s_ in range(8):
-            # capacity factor = number of experts: nothing is dropped (the default 1.25 gives
-            # capacity 1 at 16 tokens over 128 experts and would drop most routes)
-            r = cref.route(random_gate_logits(T, E, seed=s_), KK, capacity_factor=float(E))
-            tabs.append((torch.from_numpy(r["expert"].view(np.int32)).cuda(), torch.from_numpy(r["weight"]).cuda(),
-                         torch.from_numpy(r["len"].view(np.int32)).cuda(), len(np.unique(r["expert"]))))
-        it = [0]
+            logits = torch.from_numpy(random_gate_logits(T, E, seed=s_)).cuda()
+            re_ = torch.empty(T, KK, dtype=torch.int32, device="cuda")
+            rw = torch.empty(T, KK, device="cuda")
+            rl = torch.empty(T, dtype=torch.int32, device="cuda")
+            hip.moe_route(logits, KK, re_, rw, rl, capacity_factor=float(E))
+            torch.cuda.synchronize()
+            hit = len(np.unique(re_.cpu().numpy()))
+            tabs.append((re_, rw, rl, hit))
 
-        def run():
-            re_, rw, rl, _ = tabs[it[0] % len(tabs)]
-            it[0] += 1
+        def run_one(i):
+            re_, rw, rl, _ = tabs[i]
             hip.moe_matvec(gu, 12, dn, 14, x, out, H, F, E, re_, rw, rl)
-        run()
-        us = timed(run, max(8, steps // 4))
-        e_act = float(np.mean([t[3] for t in tabs]))
+        t = measure(torch, rotating(run_one, len(tabs)), steps, args.warmup)
+        e_act = float(np.mean([tb[3] for tb in tabs]))
         byts = int(e_act * (2 * F * row_bytes(12, H) + H * row_bytes(14, F)) + 128 * H * 4 + 128 * F * 8 + T * H * 4)
         flops = 128 * 2 * (2 * F * H + H * F)
         desc = (f"MoE expert matvec: {E} experts, top-{KK}, {T} tokens, gate/up Q4_K [{2 * F}x{H}], down Q6_K [{H}x{F}], "
                 f"{e_act:.1f} distinct experts hit per call on average, no capacity drop")
-        # CPU: 8 experts' worth of the same shapes (a sixteenth of the weights), 16 tokens top-2
-        Ec = 8
-        gu_h, dn_h = random_weight(12, Ec * 2 * F, H, seed=1), random_weight(14, Ec * H, F, seed=2)
-        rc_ = cref.route(random_gate_logits(T, Ec, seed=0), 2, capacity_factor=float(Ec))
-        xh = random_activations(T, H, seed=3)
-        pairs_c = int(rc_["len"].sum())
-        if args.no_cpu:
-            sec, sample = None, None
-        else:
+        if not args.no_cpu:
+            # CPU: 8 experts' worth of the same shapes (a sixteenth of the weights), 16 tokens top-2
+            Ec = 8
+            gu_h, dn_h = random_weight(12, Ec * 2 * F, H, seed=1), random_weight(14, Ec * H, F, seed=2)
+            rc_ = cref.route(random_gate_logits(T, Ec, seed=0), 2, capacity_factor=float(Ec))
+            xh = random_activations(T, H, seed=3)
+            pairs_c = int(rc_["len"].sum())
             sec, creps, cdt = cpu_time(lambda: cref.moe_ffn(gu_h, 12, dn_h, 14, xh, H, F, Ec, rc_["expert"], rc_["weight"],
                                                             rc_["len"], acc=cref.ACC_F32, threads=threads))
             sec *= 128.0 / pairs_c  # the oracle works pair by pair: scale to the 128 pairs of the workload
@@ -210,21 +280,12 @@ def run_other(args):
         copies = 3
         ws = [device_weight_any(torch, g, dtype, n, k) for _ in range(copies)]
         outs = [torch.empty(n * k, device="cuda") for _ in range(copies)]
-        it = [0]
-
-        def run():
-            i = it[0] % copies
-            it[0] += 1
-            hip.dequantize(ws[i], outs[i], dtype)
-        run()
-        us = timed(run, max(8, steps // 4))
+        t = measure(torch, rotating(lambda i: hip.dequantize(ws[i], outs[i], dtype), copies), steps, args.warmup)
         byts = n * row_bytes(dtype, k) + n * k * 4
         flops = 0
         desc = f"Backend::dequantize {TAGS[dtype]} {n} x {k} (block bytes in, f32 out), rotating over {copies} matrices"
-        host_w = random_weight(dtype, n // 8, k, seed=0)
-        if args.no_cpu:
-            sec, sample = None, None
-        else:
+        if not args.no_cpu:
+            host_w = random_weight(dtype, n // 8, k, seed=0)
             sec, creps, cdt = cpu_time(lambda: cref.dequantize(host_w, dtype))
             sec *= 8.0
             sample = f"{creps} decodes of an eighth of the matrix ({n // 8} x {k}) on one thread in {cdt:.1f} s, scaled by 8"
@@ -242,20 +303,15 @@ def run_other(args):
             half = gu.numel() // 2
             sets.append((gu[:half], gu[half:], device_weight_any(torch, g, 14, H, F),
                          torch.randn(mm, H, device="cuda", generator=g), torch.empty(mm, H, device="cuda")))
-        it = [0]
 
-        def run():
-            ga, up_, dn, xx, oo = sets[it[0] % copies]
-            it[0] += 1
+        def run_one(i):
+            ga, up_, dn, xx, oo = sets[i]
             hip.ffn_swiglu(ga, up_, 12, dn, 14, xx, oo, mm, H, F)
-        run()
-        us = timed(run, max(8, steps // 2))
+        t = measure(torch, rotating(run_one, copies), steps, args.warmup)
         byts = 2 * F * row_bytes(12, H) + H * row_bytes(14, F) + 2 * mm * H * 4
         flops = 2 * mm * (2 * F * H + H * F)
         desc = f"dense FFN M={mm}: gate/up Q4_K {H}->{F}, SwiGLU, down Q6_K {F}->{H}, rotating over {copies} weight sets"
-        if args.no_cpu:
-            sec, sample = None, None
-        else:
+        if not args.no_cpu:
             Fc = F // 8  # an eighth of the intermediate size: an eighth of every matrix
             hg, hu = random_weight(12, Fc, H, seed=1), random_weight(12, Fc, H, seed=2)
             hd = random_weight(14, H, Fc, seed=3)
@@ -275,23 +331,15 @@ def run_other(args):
         copies = 12  # 12 x 33.5 MB of outputs rotate past the Infinity Cache
         ids = [torch.randint(0, vocab, (count,), generator=g, device="cuda", dtype=torch.int32) for _ in range(copies)]
         outs = [torch.empty(count * hidden, device="cuda") for _ in range(copies)]
-        it = [0]
-
-        def run():
-            i = it[0] % copies
-            it[0] += 1
-            hip.quant_gather(table, dtype, vocab, hidden, ids[i], outs[i])
-        run()
-        us = timed(run, max(8, steps // 4))
+        t = measure(torch, rotating(lambda i: hip.quant_gather(table, dtype, vocab, hidden, ids[i], outs[i]), copies),
+                    steps, args.warmup)
         byts = count * row_bytes(dtype, hidden) + count * 4 + count * hidden * 4
         flops = 0
         desc = (f"Op::QuantGather {TAGS[dtype]}: {count} ids into a {vocab} x {hidden} table (row blocks in, f32 rows out), "
                 f"rotating over {copies} id sets and outputs")
-        host_t = random_weight(dtype, 1024, hidden, seed=0)
-        host_ids = np.random.default_rng(0).integers(0, 1024, count // 8).astype(np.uint32)
-        if args.no_cpu:
-            sec, sample = None, None
-        else:
+        if not args.no_cpu:
+            host_t = random_weight(dtype, 1024, hidden, seed=0)
+            host_ids = np.random.default_rng(0).integers(0, 1024, count // 8).astype(np.uint32)
             sec, creps, cdt = cpu_time(lambda: cref.quant_gather(host_t, dtype, 1024, hidden, host_ids))
             sec *= 8.0
             sample = f"{creps} lookups of {count // 8} ids in a 1024-row table on one thread in {cdt:.1f} s, scaled by 8"
@@ -300,29 +348,32 @@ def run_other(args):
         log(f"bench.py: unknown workload {name}")
         sys.exit(2)
 
+    us = t["us"]
     gbs = byts / us / 1e3
     result = {
-        "metric": f"{name}: achieved HBM GB/s", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps,
-        "warmup": args.warmup, "ms_per_step": round(us / 1e3, 6), "us_per_call": round(us, 3),
+        "metric": f"{name}: achieved HBM GB/s", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        **timing_fields(t, steps, args.warmup),
         "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 2), "tflops": round(flops / us / 1e6, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16" if name.startswith("gemm") else ("f32" if name.startswith(("dequant", "gather")) else "i8"), "data": "synthetic",
-        "config": {"workload": desc, "bytes_per_call": byts},
+        "config": {"workload": desc, "bytes_per_call": byts, **extra},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
     }
     if sec is not None:
         result["cpu_baseline"] = {"value": round(byts / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
                                   "us_per_call": round(sec * 1e6, 1), "sample": sample}
-    log(f"{name}: {us:.2f} us/call, {gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS * 100:.1f}% of 8 TB/s)")
+    log(f"{name}: {us:.2f} us/call (p10 {t['p10_us']:.2f}, p90 {t['p90_us']:.2f}, {t['regions']} regions of {steps}), "
+        f"{gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS * 100:.1f}% of 8 TB/s)")
     print(json.dumps(result), flush=True)
 
 
-def cpu_baseline(budget_s: float = 12.0, simd_budget_s: float = 6.0):
+def cpu_baseline(budget_s: float = 12.0, simd_budget_s: float = 5.0):
     """The oracle's reference-faithful matmul (scalar per-block decode, f32 multiply-add: what the
     reference ships for K-quants) on the host cores, on the same shape with the same generator,
-    repeated for about `budget_s` seconds; beside it, under "avx2", the oracle's vectorised flavour
-    (AVX2 decode, eight-lane f32 sums) for `simd_budget_s` seconds where the host has AVX2."""
+    repeated for about `budget_s` seconds; beside it the oracle's vectorised flavours (AVX2, and
+    AVX-512 where the host has it: block decode and f32 sums in vector registers) for
+    `simd_budget_s` seconds each."""
     from gllm_amd.ggml import row_bytes
     from gllm_amd.synth import random_activations, random_weight
     from oracle import cref
@@ -346,23 +397,26 @@ def cpu_baseline(budget_s: float = 12.0, simd_budget_s: float = 6.0):
            "us_per_call": round(dt / reps * 1e6, 1),
            "sample": f"{reps} calls of the same 1x{K_DIM}x{N} Q4_K matmul (C restatement of the reference's "
                      f"scalar decode + f32 FMA, rows split over {threads} threads) in {dt:.1f} s"}
-    if cref.have_avx2():
-        reps, dt = leg(lambda: cref.quantized_matmul_avx2(w, x, DTYPE, M, N, K_DIM, threads=threads), simd_budget_s)
-        out["avx2"] = {"value": round(bytes_per_call * reps / dt / 1e9, 3), "unit": "GB/s", "cores": threads,
-                       "us_per_call": round(dt / reps * 1e6, 1),
-                       "sample": f"{reps} calls of the same matmul with the oracle's AVX2 decode and eight-lane f32 sums "
-                                 f"over {threads} threads in {dt:.1f} s"}
+    for tag, have, fn in (("avx2", cref.have_avx2, cref.quantized_matmul_avx2),
+                          ("avx512", getattr(cref, "have_avx512", lambda: False), getattr(cref, "quantized_matmul_avx512", None))):
+        if fn is None or not have():
+            continue
+        reps, dt = leg(lambda: fn(w, x, DTYPE, M, N, K_DIM, threads=threads), simd_budget_s)
+        out[tag] = {"value": round(bytes_per_call * reps / dt / 1e9, 3), "unit": "GB/s", "cores": threads,
+                    "us_per_call": round(dt / reps * 1e6, 1),
+                    "sample": f"{reps} calls of the same matmul with the oracle's {tag.upper()} decode and vector f32 sums "
+                              f"over {threads} threads in {dt:.1f} s"}
     return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-context", action="store_true",
-                    help="skip the cache-resident and streaming-read context runs (profiling: only the timed kernel launches)")
+                    help="skip the cache-resident and copy-rate context runs (profiling: only the timed kernel launches)")
     ap.add_argument("--workload", default="gemv_q4k",
                     help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m4, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, lm_head_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
                          "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
@@ -372,6 +426,9 @@ def main():
     if args.gpus != 1:
         log("bench.py: this build measures one GPU; the quantized matmul path has no multi-GPU part "
             "(rows would shard by N with no collective). Run with --gpus 1.")
+        sys.exit(2)
+    if args.steps < 1:
+        log("bench.py: --steps must be at least 1")
         sys.exit(2)
 
     import torch
@@ -386,35 +443,20 @@ def main():
         run_other(args)
         return
     hip = HipBackend(0)
-    ws = device_weights(torch, N, K_DIM, COPIES)
     g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    ws = [device_weight_any(torch, g, DTYPE, N, K_DIM) for _ in range(COPIES)]
     g.manual_seed(1)
     x = torch.randn(M, K_DIM, device="cuda", generator=g)
     ys = [torch.empty(M, N, device="cuda") for _ in range(COPIES)]
     nb = ws[0].numel()
     bytes_per_call = N * row_bytes(DTYPE, K_DIM) + M * K_DIM * 4 + M * N * 4  # 33,103,872
+    steps = args.steps
 
-    def descs(count, single=False):
-        return [(ws[0 if single else i % COPIES], x, ys[0 if single else i % COPIES], DTYPE, M, N, K_DIM)
-                for i in range(count)]
-
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-
-    def timed(batch):
-        # The launches are enqueued by host code that allocates Python objects; a full pass of
-        # Python's cyclic garbage collector in the middle of that (tens of ms with torch
-        # loaded) would starve the GPU and be counted as kernel time.
-        gc.collect()
-        gc.disable()
-        try:
-            torch.cuda.synchronize()
-            start.record()
-            hip.quantized_matmul_batch(batch)
-            stop.record()
-            torch.cuda.synchronize()
-        finally:
-            gc.enable()
-        return start.elapsed_time(stop)  # ms
+    # One list of steps + COPIES descriptors; region r is one C call over `steps` consecutive
+    # entries starting where region r - 1 stopped in the rotation.
+    rotating = hip.make_batch([(ws[i % COPIES], x, ys[i % COPIES], DTYPE, M, N, K_DIM) for i in range(steps + COPIES)])
+    resident = hip.make_batch([(ws[0], x, ys[0], DTYPE, M, N, K_DIM)] * steps)
 
     if args.copy_probe:
         # A plain copy kernel of known size: 33,030,144 bytes read and as many written per launch.
@@ -422,44 +464,34 @@ def main():
         for i in range(8):
             dst.copy_(ws[i % COPIES])
         torch.cuda.synchronize()
-    hip.quantized_matmul_batch(descs(args.warmup))
-    torch.cuda.synchronize()
-    ms = timed(descs(args.steps))
-    us_per_call = ms * 1e3 / args.steps
+
+    t = measure(torch, lambda r: hip.run_batch(rotating, (r * steps) % COPIES, steps), steps, args.warmup)
+    us_per_call = t["us"]
     gbs = bytes_per_call / (us_per_call * 1e-6) / 1e9
 
-    # context figures (stderr): cache-resident weights, and the device's streaming-read rate
+    # context figures: cache-resident weights, and the rate of a plain device-to-device copy
     context = None
     if not args.no_context:
-        ms1 = timed(descs(min(args.steps, 1000), single=True))
-        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
-        for i in range(32):
-            hip.stream_read(ws[i % COPIES], sink)
-        torch.cuda.synchronize()
-        start.record()
-        for i in range(400):
-            hip.stream_read(ws[i % COPIES], sink)
-        stop.record()
-        torch.cuda.synchronize()
-        probe_us = start.elapsed_time(stop) * 1e3 / 400
-        context = {"cache_resident_us_per_call": round(ms1 * 1e3 / min(args.steps, 1000), 3),
-                   "stream_read_probe_gbs": round(nb / probe_us / 1e3, 1)}
-    log(f"Q4_K GEMV 1x{K_DIM}x{N}: {us_per_call:.2f} us/call, {gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS * 100:.1f}% of 8 TB/s), "
+        t1 = measure(torch, lambda r: hip.run_batch(resident, 0, steps), steps, args.warmup)
+        dsts = [torch.empty_like(ws[0]) for _ in range(4)]
+        tc = measure(torch, lambda r: [dsts[i % 4].copy_(ws[(r * 20 + i) % COPIES]) for i in range(20)], 20, 20)
+        context = {"cache_resident_us_per_call": round(t1["us"], 3),
+                   "device_copy_gbs_read_plus_write": round(2 * nb / tc["us"] / 1e3, 1)}
+    log(f"Q4_K GEMV 1x{K_DIM}x{N}: {us_per_call:.2f} us/call (p10 {t['p10_us']:.2f}, p90 {t['p90_us']:.2f}; "
+        f"{t['regions']} regions of {steps} calls), {gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS * 100:.1f}% of 8 TB/s), "
         f"{2 * N * K_DIM / (us_per_call * 1e-6) / 1e12:.2f} TFLOP/s")
     if context:
         log(f"  same weights every call (cache resident): {context['cache_resident_us_per_call']:.2f} us/call")
-        log(f"  streaming-read probe over the same 33 MB buffers: {context['stream_read_probe_gbs']:.0f} GB/s")
+        log(f"  plain device-to-device copy of the same 33 MB buffers: {context['device_copy_gbs_read_plus_write']:.0f} GB/s read+write")
 
     result = {
         "metric": "Q4_K GEMV 1x4096x14336: achieved HBM GB/s",
         "value": round(gbs, 1),
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(us_per_call / 1e3, 6),
-        "us_per_call": round(us_per_call, 3),
+        **timing_fields(t, steps, args.warmup),
         "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 2),
+        "target_pct_of_hbm_peak": 70.0,
         "tflops": round(2 * N * K_DIM / (us_per_call * 1e-6) / 1e12, 3),
         "higher_is_better": True,
         "scaling": "weak",
@@ -469,10 +501,11 @@ def main():
         "config": {"workload": f"Q4_K dequant-GEMV M=1 K={K_DIM} N={N} (GGUF 144-byte super-blocks), f32 activations "
                                f"~N(0,1) as 23-bit block fixed point, int8 MFMA with i32 accumulation, f32 scales; "
                                f"weights rotate over {COPIES} copies ({COPIES * nb >> 20} MiB) so every call reads HBM",
-                   "bytes_per_call": bytes_per_call, "kernel": "gq_mm8_q4k_p1_e1_a2"},
+                   "bytes_per_call": bytes_per_call, "kernel": hip.last_kernel_name()},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-                     "note": "achieved = 33,103,872 algorithmic bytes / (event time over the timed region / steps); "
+                     "traffic_source": TRAFFIC_SOURCE,
+                     "note": "achieved = 33,103,872 algorithmic bytes / median event time per call; "
                              "the event time includes the gap between back-to-back launches"},
     }
     if context:

@@ -92,15 +92,30 @@ def load_library() -> C.CDLL:
     L.gllmq_quantized_matmul_batch.restype = C.c_int
     L.gllmq_quantized_matmul_batch.argtypes = [vp, C.POINTER(MatmulDesc), sz, vp]
     L.gllmq_moe_matvec.restype = C.c_int
-    L.gllmq_moe_matvec.argtypes = [vp, vp, u32, vp, u32, vp, vp, sz, sz, sz, sz, sz, vp, vp, vp, C.c_int, vp]
+    L.gllmq_moe_matvec.argtypes = [vp, vp, sz, sz, vp, sz, sz, u32, vp, sz, sz, u32, vp, vp, sz, sz, sz, sz, sz, vp, vp, vp,
+                                   C.c_int, vp]
+    L.gllmq_moe_route.restype = C.c_int
+    L.gllmq_moe_route.argtypes = [vp, vp, sz, sz, sz, C.c_float, vp, vp, vp, vp, vp, vp, vp]
+    L.gllmq_set_option.restype = C.c_int
+    L.gllmq_set_option.argtypes = [vp, C.c_char_p, C.c_long]
+    L.gllmq_last_kernel_name.restype = C.c_char_p
+    L.gllmq_last_kernel_name.argtypes = [vp]
+    L.gllmq_reserve_matmul.restype = C.c_int
+    L.gllmq_reserve_matmul.argtypes = [vp, u32, sz, sz, sz, vp]
+    L.gllmq_reserve_ffn.restype = C.c_int
+    L.gllmq_reserve_ffn.argtypes = [vp, u32, u32, sz, sz, sz, vp]
+    L.gllmq_reserve_moe.restype = C.c_int
+    L.gllmq_reserve_moe.argtypes = [vp, sz, sz, sz, sz, vp]
+    L.gllmq_weights_forget.restype = None
+    L.gllmq_weights_forget.argtypes = [vp, vp]
+    L.gllmq_weight_uploads.restype = C.c_uint64
+    L.gllmq_weight_uploads.argtypes = [vp]
     L.gllmq_quant_gather.restype = C.c_int
     L.gllmq_quant_gather.argtypes = [vp, vp, sz, u32, sz, sz, vp, sz, C.c_float, vp, vp]
     L.gllmq_ffn_swiglu.restype = C.c_int
     L.gllmq_ffn_swiglu.argtypes = [vp, vp, vp, sz, u32, vp, sz, u32, vp, vp, sz, sz, sz, C.c_int, vp]
     L.gllmq_argmax.restype = C.c_int
     L.gllmq_argmax.argtypes = [vp, vp, sz, sz, sz, vp, vp, vp]
-    L.gllmq_stream_read.restype = C.c_int
-    L.gllmq_stream_read.argtypes = [vp, vp, sz, vp, vp]
     L.gllmq_dequantize_host.restype = C.c_int
     L.gllmq_dequantize_host.argtypes = [vp, vp, sz, vp, sz, u32]
     L.gllmq_quant_gather_host.restype = C.c_int
@@ -115,7 +130,9 @@ EXPORTED_SYMBOLS = [
     "gllmq_init", "gllmq_destroy", "gllmq_last_error", "gllmq_status_string", "gllmq_version",
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
-    "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_quant_gather", "gllmq_stream_read", "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
+    "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_quant_gather", "gllmq_moe_route", "gllmq_set_option", "gllmq_last_kernel_name",
+    "gllmq_reserve_matmul", "gllmq_reserve_ffn", "gllmq_reserve_moe", "gllmq_weights_forget", "gllmq_weight_uploads",
+    "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
     "gllmq_gguf_open", "gllmq_gguf_parse", "gllmq_gguf_close", "gllmq_gguf_version", "gllmq_gguf_tensor_count",
     "gllmq_gguf_kv_count", "gllmq_gguf_alignment", "gllmq_gguf_data_offset", "gllmq_gguf_tensor_at",
     "gllmq_gguf_find_tensor", "gllmq_gguf_tensor_data", "gllmq_gguf_meta_type", "gllmq_gguf_meta_u64",
@@ -143,7 +160,9 @@ def _host_bytes(buf) -> np.ndarray:
 class HipBackend:
     """The MI355X backend for ``Op::QuantGemm``: quantized weights x f32 activations."""
 
-    def __init__(self, device: int = 0):
+    def __init__(self, device: int = 0, options: dict | None = None):
+        """``options``: kernel-family choices by name (``gllmq_set_option``), used by the tests to
+        reach the kernels the default dispatch does not pick."""
         self._lib = load_library()
         import torch
         if not torch.cuda.is_available():
@@ -155,6 +174,41 @@ class HipBackend:
         if rc != OK:
             raise HipError(f"gllmq_init(device={device}): {self._lib.gllmq_status_string(rc).decode()}")
         self._ctx = ctx
+        for name, value in (options or {}).items():
+            self.set_option(name, value)
+
+    def set_option(self, name: str, value: int) -> None:
+        rc = self._lib.gllmq_set_option(self._ctx, name.encode(), int(value))
+        if rc != OK:
+            self._raise(rc, "set_option")
+
+    def last_kernel_name(self) -> str:
+        """Name of the kernel this context launched last."""
+        return self._lib.gllmq_last_kernel_name(self._ctx).decode()
+
+    def weight_uploads(self) -> int:
+        """Host-to-device weight copies the host-slice calls of this context have made."""
+        return int(self._lib.gllmq_weight_uploads(self._ctx))
+
+    def weights_forget(self, host_array=None) -> None:
+        ptr = None if host_array is None else _host_bytes(host_array).ctypes.data
+        self._lib.gllmq_weights_forget(self._ctx, ptr)
+
+    def reserve_matmul(self, quant_type, m: int, n: int, k: int) -> None:
+        rc = self._lib.gllmq_reserve_matmul(self._ctx, _dtype_id(quant_type), m, n, k, self._stream())
+        if rc != OK:
+            self._raise(rc, "reserve_matmul")
+
+    def reserve_ffn(self, dtype_gate_up, dtype_down, m: int, hidden: int, ffn: int) -> None:
+        rc = self._lib.gllmq_reserve_ffn(self._ctx, _dtype_id(dtype_gate_up), _dtype_id(dtype_down), m, hidden, ffn,
+                                         self._stream())
+        if rc != OK:
+            self._raise(rc, "reserve_ffn")
+
+    def reserve_moe(self, tokens: int, top_k: int, hidden: int, ffn: int) -> None:
+        rc = self._lib.gllmq_reserve_moe(self._ctx, tokens, top_k, hidden, ffn, self._stream())
+        if rc != OK:
+            self._raise(rc, "reserve_moe")
 
     def close(self) -> None:
         if getattr(self, "_ctx", None):
@@ -234,16 +288,29 @@ class HipBackend:
             self._raise(rc, "dequantize")
 
     # --------------------------------------------------------------- extensions
-    def quantized_matmul_batch(self, descs) -> None:
-        """descs: iterable of (w, x, y, quant_type, m, n, k) device tensors; one C call."""
+    def make_batch(self, descs):
+        """A descriptor array for ``run_batch``; descs: iterable of (w, x, y, quant_type, m, n, k)
+        device tensors, which must stay alive while the array is used."""
         items = list(descs)
         arr = (MatmulDesc * len(items))()
         for i, (w, x, y, qt, m, n, k) in enumerate(items):
             arr[i] = MatmulDesc(w.data_ptr(), w.numel() * w.element_size(), x.data_ptr(), y.data_ptr(),
                                 _dtype_id(qt), 0, m, n, k)
-        rc = self._lib.gllmq_quantized_matmul_batch(self._ctx, arr, len(items), self._stream())
+        return arr
+
+    def run_batch(self, arr, start: int = 0, count: int | None = None) -> None:
+        """One C call over ``count`` descriptors of ``arr`` from ``start``."""
+        count = len(arr) - start if count is None else count
+        if start < 0 or count < 0 or start + count > len(arr):
+            raise OtherError("run_batch: range outside the descriptor array")
+        first = C.cast(C.byref(arr, start * C.sizeof(MatmulDesc)), C.POINTER(MatmulDesc))
+        rc = self._lib.gllmq_quantized_matmul_batch(self._ctx, first, count, self._stream())
         if rc != OK:
             self._raise(rc, "quantized_matmul_batch")
+
+    def quantized_matmul_batch(self, descs) -> None:
+        """descs: iterable of (w, x, y, quant_type, m, n, k) device tensors; one C call."""
+        self.run_batch(self.make_batch(descs))
 
     def quant_gather(self, table, quant_type, vocab_size: int, hidden_dim: int, token_ids, output,
                      scale: float | None = None) -> None:
@@ -304,18 +371,44 @@ class HipBackend:
         if rc != OK:
             self._raise(rc, "argmax")
 
-    def stream_read(self, buf, sink) -> None:
-        """Calibration: one streaming read of ``buf`` (device tensor, 16-byte multiple)."""
-        rc = self._lib.gllmq_stream_read(self._ctx, buf.data_ptr(), buf.numel() * buf.element_size(),
-                                         sink.data_ptr(), self._stream())
+    def moe_route(self, logits, top_k: int, route_expert, route_weight, route_len, capacity_factor: float = 1.25,
+                  route_pos=None, expert_counts=None, overflow=None) -> None:
+        """ExpertRouteTable::from_gate_logits on device tensors: ``logits`` f32 ``[tokens, experts]``;
+        outputs ``route_expert`` (32-bit int) and ``route_weight`` (f32) ``[tokens, top_k]``,
+        ``route_len`` ``[tokens]``; optional ``route_pos`` ``[tokens, top_k]``, ``expert_counts``
+        ``[experts]``, ``overflow`` ``[1]``.  The reference's default capacity factor is 1.25."""
+        tokens, experts = logits.shape
+        if logits.dtype != self._torch.float32 or not logits.is_cuda or not logits.is_contiguous():
+            raise OtherError("moe_route: logits must be a contiguous device f32 tensor")
+        if route_expert.numel() < tokens * top_k or route_weight.numel() < tokens * top_k or route_len.numel() < tokens:
+            raise OtherError("moe_route: outputs shorter than tokens * top_k / tokens")
+        opt = [t.data_ptr() if t is not None else None for t in (route_pos, expert_counts, overflow)]
+        rc = self._lib.gllmq_moe_route(self._ctx, logits.data_ptr(), tokens, experts, top_k, float(capacity_factor),
+                                       route_expert.data_ptr(), route_weight.data_ptr(), route_len.data_ptr(),
+                                       opt[0], opt[1], opt[2], self._stream())
         if rc != OK:
-            self._raise(rc, "stream_read")
+            self._raise(rc, "moe_route")
 
     def moe_matvec(self, gate_up, dtype_gate_up, down, dtype_down, x, out, hidden: int, ffn: int,
-                   experts: int, route_expert, route_weight, route_len, relu_gate: bool = False) -> None:
+                   experts: int, route_expert, route_weight, route_len, relu_gate: bool = False,
+                   up=None) -> None:
+        """Expert matvec over a route table.  ``gate_up``: per expert ``ffn`` gate rows followed by
+        ``ffn`` up rows (one stacked tensor), or, with ``up`` given, the gate rows of all experts
+        (``[experts, ffn, hidden]``) with ``up`` holding the up rows the same way (GGUF's layout);
+        ``down``: ``[experts, hidden, ffn]``."""
         tokens, top_k = route_expert.shape
+        dgu, ddn = _dtype_id(dtype_gate_up), _dtype_id(dtype_down)
+        each = ffn * self._lib.gllmq_row_bytes(dgu, hidden)  # 0 for a dtype the library does not cover
+        gbytes = gate_up.numel() * gate_up.element_size()
+        if up is None:
+            gate_ptr, gate_b, gate_st = gate_up.data_ptr(), max(gbytes - each, 0), 2 * each
+            up_ptr, up_b, up_st = gate_up.data_ptr() + each, max(gbytes - each, 0), 2 * each
+        else:
+            gate_ptr, gate_b, gate_st = gate_up.data_ptr(), gbytes, each
+            up_ptr, up_b, up_st = up.data_ptr(), up.numel() * up.element_size(), each
         rc = self._lib.gllmq_moe_matvec(
-            self._ctx, gate_up.data_ptr(), _dtype_id(dtype_gate_up), down.data_ptr(), _dtype_id(dtype_down),
+            self._ctx, gate_ptr, gate_b, gate_st, up_ptr, up_b, up_st, dgu,
+            down.data_ptr(), down.numel() * down.element_size(), hidden * self._lib.gllmq_row_bytes(ddn, ffn), ddn,
             x.data_ptr(), out.data_ptr(), tokens, hidden, ffn, experts, top_k, route_expert.data_ptr(),
             route_weight.data_ptr(), route_len.data_ptr(), int(relu_gate), self._stream())
         if rc != OK:

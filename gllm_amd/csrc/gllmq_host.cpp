@@ -10,12 +10,14 @@
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 // The code object built from gllmq_kernels.hip, placed in .rodata by the assembler.
@@ -112,6 +114,41 @@ uint32_t mm8_lds_bytes(uint32_t groups, uint32_t m, uint32_t pairs, int kind = M
 
 } // namespace
 
+// Device memory beyond the inputs and outputs that the kernels of one call may use.  Every stream
+// a context is used on gets its own set, so calls on different streams never share scratch and
+// calls on one stream are ordered by the stream itself.
+struct Scratch {
+    hipStream_t stream = nullptr;
+    uint64_t last_use = 0;
+    bool fixed = false;          // carved from a block of fixed size: a call that needs more fails
+    // K split of the int8 kernels: slice sums, and arrival counters that every launch leaves at 0
+    float *mm8_part = nullptr;   // [MM8_SPLIT_PART_FLOATS]
+    uint32_t *mm8_arrive = nullptr; // [MM8_SPLIT_MAX_LISTS]
+    uint64_t *argmax_keys = nullptr; // [ARGMAX_MAX_ROWS][ARGMAX_MAX_PARTS]
+    void *base = nullptr;        // the allocation that holds the three above
+    void *mmf = nullptr;         // GEMM: activation images, then partial sums of K-split workgroups
+    size_t mmf_bytes = 0;
+    void *ffn = nullptr;         // gllmq_ffn_swiglu: gated activations, then gate/up results
+    size_t ffn_bytes = 0;
+    void *moe = nullptr;         // gllmq_moe_matvec: pair tables, jobs, intermediate activations
+    size_t moe_bytes = 0;
+};
+
+constexpr size_t kScratchArriveBytes = 4096; // MM8_SPLIT_MAX_LISTS words, padded
+constexpr size_t kScratchKeysBytes = sizeof(uint64_t) * gq::ARGMAX_MAX_ROWS * gq::ARGMAX_MAX_PARTS;
+constexpr size_t kScratchPartBytes = sizeof(float) * gq::MM8_SPLIT_PART_FLOATS;
+constexpr size_t kScratchFixedBytes = kScratchArriveBytes + kScratchKeysBytes + kScratchPartBytes;
+constexpr size_t kMaxScratchSlots = 16;
+
+// Weights that a host-slice call uploaded, kept for the next call with the same slice
+// (the reference keeps its uploaded weight blob the same way, src/compat/hip_backend.rs:141-156).
+struct CachedWeights {
+    const void *host = nullptr;
+    size_t bytes = 0;
+    void *dev = nullptr;
+    uint64_t last_use = 0;
+};
+
 struct gllmq_ctx {
     int device = 0;
     hipModule_t module = nullptr;
@@ -122,65 +159,53 @@ struct gllmq_ctx {
     hipFunction_t mm8_glu[2][3][3] = {};
     hipFunction_t mm8_glu_areg[2][2][3][2] = {};
     hipFunction_t glu_act = nullptr;            // act(gate) * up as a kernel of its own
-    bool ffn_fused = true;                      // GLLMQ_FFN_FUSED=0: gllmq_ffn_swiglu never uses the gated kernels
-    void *ffn_scratch = nullptr;                // gate/up results and the gated activations of gllmq_ffn_swiglu
-    size_t ffn_scratch_bytes = 0;
     hipFunction_t argmax_part = nullptr, argmax_final = nullptr;
-    uint64_t *argmax_keys = nullptr;            // [ARGMAX_MAX_ROWS][ARGMAX_MAX_PARTS] scratch of gllmq_argmax
     hipFunction_t dequant_wave = nullptr;       // Q4_K with 16-byte aligned blocks and outputs: one block per wave
     hipFunction_t dequant_wave_q5k = nullptr;   // the same for Q5_K
     hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1], f32 multiply-add flavour
     hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
-    bool gemv_f32 = false;                      // GLLMQ_GEMV_F32=1 selects the f32 flavour
     // int8 matrix-core kernels [Mm8Kind][pairs 1,2,4][early steps 1,2,4], and the same with
     // register-resident activation operands [Mm8Kind][pairs 1,2][early][passes per tile - 1]
     hipFunction_t mm8[MM8_KINDS][3][3] = {};
     hipFunction_t mm8_areg[MM8_KINDS][2][3][2] = {};
-    bool use_mm8 = true;                        // GLLMQ_MM8=0 falls back to the GEMV kernels
-    bool mm8_areg_on = true;                    // GLLMQ_MM8_AREG=0 keeps the activation operands in LDS
-    // Fewest activation rows that send Q6_K to the matrix-core kernel: up to two rows the GEMV
-    // kernels are as fast or faster.  GLLMQ_MM8_Q6K_MIN_M overrides (1 = always, 0 = never).
-    uint32_t mm8_q6k_min_m = 3;
-    uint32_t mm8_q5k_min_m = 2;                 // the same for Q5_K (GLLMQ_MM8_Q5K_MIN_M): one row is as fast on the GEMV
-    uint32_t mm8_q8_0_min_m = 3;                // the same for Q8_0 (GLLMQ_MM8_Q8_0_MIN_M)
-    bool moe_mm8 = true;                        // GLLMQ_MOE_MM8=0 keeps the MoE expert rows on the GEMV kernels
-    bool moe_mm8_q6k = true;                    // GLLMQ_MOE_MM8_Q6K=0 keeps Q6_K expert rows there
-    bool moe_glu = true;                        // GLLMQ_MOE_GLU=0: gate/up results to memory, activation as a kernel of its own
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
-    bool moe_mm8_rows = true;                   // GLLMQ_MOE_MM8_ROWS=0: no wave-per-tile kernel for short Q6_K rows
-    // development overrides of launch shapes, read once at init (0 = the library's own choice):
-    // GLLMQ_MM8_GRID, GLLMQ_MMF_KSPLIT, GLLMQ_MMF_ROWS, GLLMQ_MOE_JOB_WAVES, GLLMQ_MOE_SLICES
-    uint32_t tune_mm8_grid = 0, tune_mmf_ksplit = 0, tune_mmf_rows = 0, tune_moe_job_waves = 0, tune_moe_slices = 0;
-    hipFunction_t stream_read = nullptr;
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
     hipFunction_t mmf_reduce = nullptr;         // and the in-order sum of its K-split partial results
-    bool use_mmf = true;                        // GLLMQ_MMF=0 keeps m > 8 on the 8-row passes
-    // Fewest rows the GEMM takes when the 8-row kernel would need more than one pass over the
-    // weights (long rows: the prepared activations of all rows do not fit the LDS of a CU).
-    // GLLMQ_MMF_SMALL_MIN_M overrides (0 = never).
-    uint32_t mmf_small_min_m = 3;
-    // Scratch of the GEMM: activation images and partial sums of K-split workgroups.  Shared
-    // by all calls on this context, like `workspace`.
-    void *mmf_partial = nullptr;
-    size_t mmf_partial_bytes = 0;
-    hipFunction_t moe_plan = nullptr, moe_act = nullptr, moe_combine = nullptr;
+    hipFunction_t moe_plan = nullptr, moe_act = nullptr, moe_combine = nullptr, moe_route = nullptr;
     hipFunction_t moe_gemv[kNumFormats] = {};
     hipFunction_t moe_mm8_fn[MM8_KINDS][2] = {}; // grouped int8 matrix-core kernels [Mm8Kind][passes per tile - 1]
     hipFunction_t moe_mm8_q6k_rows = nullptr;   // Q6_K rows of at most 8 blocks: a wave per 32-row tile
     uint32_t *identity_rows = nullptr;          // device: 0..7, the activation rows of an ungathered matmul
-    // K split of the int8 kernels for few weight rows: slice sums and arrival counters (fixed size,
-    // allocated at init; shared by all calls on this context).  GLLMQ_MM8_KSPLIT caps the number of
-    // slices (0 or 1 = never split).
-    float *mm8_part = nullptr;
-    uint32_t *mm8_arrive = nullptr;
-    uint32_t mm8_ksplit_max = 8;
-    // Device workspace of the MoE path (pair tables, jobs, intermediate activations).  It
-    // grows on demand and is shared by all calls on this context: calls that use it must
-    // not overlap in time.
-    void *workspace = nullptr;
-    size_t workspace_bytes = 0;
-    std::mutex workspace_mutex;
+
+    // Kernel-family choices (gllmq_set_option).  The defaults are the measured best; the tests
+    // switch them to reach every kernel family through the public entry points.
+    bool gemv_f32 = false;                      // "gemv_f32": the f32 multiply-add GEMV instead of the integer-dot one
+    bool use_mm8 = true;                        // "mm8" = 0: no int8 matrix-core kernels
+    bool use_mmf = true;                        // "mmf" = 0: more than 8 rows run 8-row passes
+    bool ffn_fused = true;                      // "ffn_fused" = 0: gllmq_ffn_swiglu never uses the gated kernels
+    // Fewest activation rows that send a format to the int8 matrix-core kernel (below, the GEMV
+    // kernels are as fast or faster); 1 = always, 0 = never.
+    uint32_t mm8_q6k_min_m = 3, mm8_q5k_min_m = 2, mm8_q8_0_min_m = 3;
+    // Fewest rows the GEMM takes when the 8-row kernel would need more than one pass over the
+    // weights (long rows: the prepared activations of all rows do not fit the LDS of a CU); 0 = never.
+    uint32_t mmf_small_min_m = 3;
+    uint32_t mm8_ksplit_max = 8;                // "mm8_ksplit": most slices of the K split (0 or 1 = never split)
+    bool moe_mm8 = true;                        // "moe_mm8" = 0: expert rows stay on the GEMV kernels
+    bool moe_mm8_q6k = true;                    // "moe_mm8_q6k" = 0: Q6_K expert rows stay there
+    bool moe_glu = true;                        // "moe_glu" = 0: gate/up results to memory, activation as a kernel of its own
+    bool moe_mm8_rows = true;                   // "moe_mm8_rows" = 0: no wave-per-tile kernel for short Q6_K rows
+
+    // One lock over every enqueue on this context: calls from several threads take turns on the
+    // host (the kernels they enqueue overlap as their streams allow).
+    std::recursive_mutex call_mutex;
+    std::vector<Scratch> scratch;               // one set per stream the context has been used on
+    uint64_t use_counter = 0;
+    std::vector<CachedWeights> weights;         // host-slice calls: uploaded weights by (pointer, length)
+    size_t weights_cache_limit = size_t(64) << 30; // bytes kept before the least recently used goes
+    uint64_t weight_uploads = 0;                // how many host-to-device weight copies the cache has done
+    std::unordered_map<hipFunction_t, std::string> kernel_names;
+    hipFunction_t last_kernel = nullptr;
     int num_cus = 256;
     uint32_t gemv_waves = 2048; // waves a GEMV launch aims to put on the device
     std::mutex err_mutex;
@@ -210,6 +235,8 @@ extern "C" int gq_ctx_set_error(gllmq_ctx *ctx, int status, const char *message)
     return fail(ctx, status, "%s", message ? message : "");
 }
 
+extern "C" int gq_ctx_device(const gllmq_ctx *ctx) { return ctx ? ctx->device : -1; }
+
 namespace {
 
 #define GLLMQ_HIP(ctx, call)                                                                  \
@@ -225,6 +252,100 @@ int get_function(gllmq_ctx *ctx, hipFunction_t *f, const char *name)
     if (e != hipSuccess)
         return fail(ctx, GLLMQ_ERR_HIP, "kernel %s missing from the code object: %s", name,
                     hipGetErrorString(e));
+    ctx->kernel_names[*f] = name;
+    return GLLMQ_OK;
+}
+
+bool stream_is_capturing(void *stream)
+{
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return st != hipStreamCaptureStatusNone;
+}
+
+void carve_fixed(Scratch &S, void *base)
+{
+    uint8_t *b = static_cast<uint8_t *>(base);
+    S.mm8_arrive = reinterpret_cast<uint32_t *>(b);
+    S.argmax_keys = reinterpret_cast<uint64_t *>(b + kScratchArriveBytes);
+    S.mm8_part = reinterpret_cast<float *>(b + kScratchArriveBytes + kScratchKeysBytes);
+}
+
+void free_scratch(Scratch &S)
+{
+    if (S.fixed) return;
+    if (S.base) (void)hipFree(S.base);
+    if (S.mmf) (void)hipFree(S.mmf);
+    if (S.ffn) (void)hipFree(S.ffn);
+    if (S.moe) (void)hipFree(S.moe);
+    S = Scratch{};
+}
+
+// The scratch set of `stream` on this context (call_mutex held).  A stream the context has not
+// seen gets a new set; beyond kMaxScratchSlots streams the least recently used set is given up
+// after the device has drained.  Allocating is not possible while `stream` is being captured.
+int acquire_scratch(gllmq_ctx *ctx, void *stream, Scratch **out)
+{
+    ++ctx->use_counter;
+    for (Scratch &S : ctx->scratch)
+        if (S.stream == static_cast<hipStream_t>(stream)) {
+            S.last_use = ctx->use_counter;
+            *out = &S;
+            return GLLMQ_OK;
+        }
+    if (stream_is_capturing(stream))
+        return fail(ctx, GLLMQ_ERR_INVALID,
+                    "the context has no scratch for this stream yet and cannot allocate it during stream capture: "
+                    "call gllmq_reserve (or run the call once) on this stream before capturing");
+    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
+    if (ctx->scratch.size() >= kMaxScratchSlots) {
+        size_t lru = 0;
+        for (size_t i = 1; i < ctx->scratch.size(); ++i)
+            if (ctx->scratch[i].last_use < ctx->scratch[lru].last_use) lru = i;
+        GLLMQ_HIP(ctx, hipDeviceSynchronize()); // its stream may be gone: wait for everything
+        free_scratch(ctx->scratch[lru]);
+        ctx->scratch.erase(ctx->scratch.begin() + static_cast<long>(lru));
+    }
+    Scratch S;
+    S.stream = static_cast<hipStream_t>(stream);
+    S.last_use = ctx->use_counter;
+    GLLMQ_HIP(ctx, hipMalloc(&S.base, kScratchFixedBytes));
+    hipError_t e = hipMemset(S.base, 0, kScratchArriveBytes);
+    if (e != hipSuccess) {
+        (void)hipFree(S.base);
+        return fail(ctx, GLLMQ_ERR_HIP, "scratch: %s", hipGetErrorString(e));
+    }
+    carve_fixed(S, S.base);
+    ctx->scratch.push_back(S);
+    *out = &ctx->scratch.back();
+    return GLLMQ_OK;
+}
+
+// Makes *buf hold at least `need` bytes.  Growing waits for the stream's earlier work (which may
+// still use the old buffer; other streams have their own scratch), so it cannot happen while the
+// stream is being captured, and never happens for a set of fixed size.
+int grow_scratch(gllmq_ctx *ctx, const Scratch &S, void **buf, size_t *have, size_t need, void *stream, const char *what)
+{
+    if (*have >= need) return GLLMQ_OK;
+    if (S.fixed)
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "%s needs %zu bytes of scratch, the fixed scratch of this entry point has %zu",
+                    what, need, *have);
+    if (stream_is_capturing(stream))
+        return fail(ctx, GLLMQ_ERR_INVALID,
+                    "%s needs %zu bytes of scratch (the stream has %zu) and cannot allocate during stream capture: "
+                    "call gllmq_reserve (or run the shape once) on this stream before capturing", what, need, *have);
+    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
+    if (*buf) {
+        GLLMQ_HIP(ctx, hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+        GLLMQ_HIP(ctx, hipFree(*buf));
+        *buf = nullptr;
+        *have = 0;
+    }
+    GLLMQ_HIP(ctx, hipMalloc(buf, need));
+    *have = need;
     return GLLMQ_OK;
 }
 
@@ -235,6 +356,7 @@ int launch2d(gllmq_ctx *ctx, hipFunction_t f, uint32_t grid_x, uint32_t grid_y, 
                        &params_size, HIP_LAUNCH_PARAM_END };
     GLLMQ_HIP(ctx, hipModuleLaunchKernel(f, grid_x, grid_y, 1, block, 1, 1, lds, static_cast<hipStream_t>(stream),
                                          nullptr, config));
+    ctx->last_kernel = f;
     return GLLMQ_OK;
 }
 
@@ -341,7 +463,7 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
 // takes the GEMV kernels.
 // `w2` != null selects the gated form: `w` holds the n gate rows, `w2` the n up rows, and
 // y = act(gate . x) * (up . x) (Q4_K and Q5_K, one pass only).
-int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
+int run_mm8(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
             size_t k, bool act_bf16, void *stream, bool one_pass_only = false, const uint8_t *w2 = nullptr,
             bool glu_relu = false)
 {
@@ -413,8 +535,8 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         Mm8Params P{};
         P.ksplit = ksplit;
         P.kslice_groups = slice_passes * 8u;
-        P.part = ctx->mm8_part;
-        P.arrive = ctx->mm8_arrive;
+        P.part = S.mm8_part;
+        P.arrive = S.mm8_arrive;
         P.w2 = w2;
         P.glu_relu = glu_relu ? 1u : 0u;
         P.w = w;
@@ -436,7 +558,6 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         while (ei < 2 && !ctx->mm8[kind][pi][ei]) ++ei; // not every (pairs, early) pair is built
         const int gi = kind == MM8_Q5K ? 1 : 0;
         uint32_t grid = std::min<uint32_t>(P.tiles, std::max(1u, static_cast<uint32_t>(ctx->num_cus) / ksplit));
-        if (ctx->tune_mm8_grid) grid = std::min<uint32_t>(P.tiles, std::max(1u, ctx->tune_mm8_grid / ksplit));
         if (ksplit > 1) grid = std::min(grid, gq::MM8_SPLIT_MAX_LISTS);
         P.grid = grid; // workgroups per slice: launch index = tile list * ksplit + slice
         hipFunction_t fn = glu ? ctx->mm8_glu[gi][pi][ei] : ctx->mm8[kind][pi][ei];
@@ -444,7 +565,7 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         // take a tile's pass from the item's position in the register ring; a last K slice with
         // fewer passes than the others would break that, so such a split runs the LDS variants.
         const bool even_slices = ksplit == 1 || ppt_row % slice_passes == 0;
-        if (pi <= 1 && ppt <= 2 && ctx->mm8_areg_on && even_slices)
+        if (pi <= 1 && ppt <= 2 && even_slices)
             fn = glu ? ctx->mm8_glu_areg[gi][pi][ei][ppt - 1] : ctx->mm8_areg[kind][pi][ei][ppt - 1];
         int rc = launch(ctx, fn, grid * ksplit, 512, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
@@ -454,40 +575,43 @@ int run_mm8(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
 
 constexpr uint32_t kMmfMaxRowTiles = 16384;
 
-int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
+// Launch shape of the GEMM for one matmul, and the scratch it needs.
+struct MmfPlan {
+    uint32_t groups, row_tiles, ksplit, bps;
+    size_t img_bytes, need;
+};
+
+MmfPlan plan_mmf(const gllmq_ctx *ctx, size_t m, size_t n, size_t k)
+{
+    MmfPlan L{};
+    L.groups = static_cast<uint32_t>((k + 255) / 256);
+    L.row_tiles = static_cast<uint32_t>((n + 255) / 256);
+    uint32_t ksplit = std::max(1u, static_cast<uint32_t>(ctx->num_cus) / std::max(1u, L.row_tiles));
+    ksplit = std::min(ksplit, L.groups);
+    L.bps = (L.groups + ksplit - 1) / ksplit;
+    L.ksplit = (L.groups + L.bps - 1) / L.bps; // every workgroup gets at least one block
+    const size_t rows = std::min<size_t>(m, 64);
+    // scratch: the activation images of one pass, then the partial sums
+    L.img_bytes = static_cast<size_t>(L.groups) * mmf_image_bytes(rows <= 32 ? 1u : 2u);
+    L.need = L.img_bytes + (L.ksplit > 1 ? static_cast<size_t>(L.ksplit) * rows * n * 4 : 0);
+    return L;
+}
+
+int run_mmf(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
             size_t k, bool act_bf16, void *stream, size_t min_m = 9)
 {
     if (!ctx->use_mmf || m < min_m) return -1;
     const int fmt = f.dtype == T_Q8_0 ? 3 : f.dtype == T_Q6_K ? 2 : f.dtype == T_Q5_K ? 1 : 0;
     if (fmt == 3 && k < 256) return -1; // the Q8_0 fetch window is one whole group of 8 blocks
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
-    const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
-    const uint32_t row_tiles = static_cast<uint32_t>((n + 255) / 256);
+    const MmfPlan L = plan_mmf(ctx, m, n, k);
+    const uint32_t groups = L.groups, row_tiles = L.row_tiles, ksplit = L.ksplit, bps = L.bps;
     if (row_tiles > kMmfMaxRowTiles) return -1;
     // the GEMM kernels address weight rows with 32-bit byte offsets from the start of the matrix
     if (n * gllmq_row_bytes(f.dtype, k) > 0xFFFFFFFFull) return -1;
-    uint32_t ksplit = std::max(1u, static_cast<uint32_t>(ctx->num_cus) / row_tiles);
-    if (ctx->tune_mmf_ksplit) ksplit = ctx->tune_mmf_ksplit;
-    ksplit = std::min(ksplit, groups);
-    const uint32_t bps = (groups + ksplit - 1) / ksplit;
-    ksplit = (groups + bps - 1) / bps; // every workgroup gets at least one block
-    std::lock_guard<std::mutex> guard(ctx->workspace_mutex);
-    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
-    size_t rows_per_pass = 64;
-    if (ctx->tune_mmf_rows) rows_per_pass = ctx->tune_mmf_rows <= 32 ? 32 : 64;
-    // scratch: the activation images of one pass, then the partial sums
-    const size_t img_bytes = static_cast<size_t>(groups) * mmf_image_bytes(std::min(m, rows_per_pass) <= 32 ? 1u : 2u);
-    const size_t need = img_bytes + (ksplit > 1 ? static_cast<size_t>(ksplit) * std::min(m, rows_per_pass) * n * 4 : 0);
-    if (ctx->mmf_partial_bytes < need) {
-        if (ctx->mmf_partial) {
-            GLLMQ_HIP(ctx, hipDeviceSynchronize()); // earlier calls may still be using it
-            GLLMQ_HIP(ctx, hipFree(ctx->mmf_partial));
-            ctx->mmf_partial = nullptr;
-            ctx->mmf_partial_bytes = 0;
-        }
-        GLLMQ_HIP(ctx, hipMalloc(&ctx->mmf_partial, need));
-        ctx->mmf_partial_bytes = need;
-    }
+    const size_t rows_per_pass = 64, img_bytes = L.img_bytes;
+    int grc = grow_scratch(ctx, S, &S.mmf, &S.mmf_bytes, L.need, stream, "quantized_matmul (GEMM)");
+    if (grc != GLLMQ_OK) return grc;
     for (size_t m0 = 0; m0 < m; m0 += rows_per_pass) {
         const uint32_t mm = static_cast<uint32_t>(std::min(rows_per_pass, m - m0));
         const uint32_t mt = mm <= 32 ? 1u : 2u;
@@ -495,8 +619,8 @@ int run_mmf(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, f
         P.w = w;
         P.x = x + m0 * k;
         P.y = y + m0 * n;
-        P.ximg = static_cast<uint8_t *>(ctx->mmf_partial);
-        P.partial = reinterpret_cast<float *>(static_cast<uint8_t *>(ctx->mmf_partial) + img_bytes);
+        P.ximg = static_cast<uint8_t *>(S.mmf);
+        P.partial = reinterpret_cast<float *>(static_cast<uint8_t *>(S.mmf) + img_bytes);
         P.n = static_cast<uint32_t>(n);
         P.k = static_cast<uint32_t>(k);
         P.groups = groups;
@@ -542,21 +666,39 @@ int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
 }
 
 // One quantized matmul on validated arguments: the kernel family by format, rows and shape.
-int dispatch_matmul(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
-                    size_t k, bool bf16, void *stream)
+int dispatch_matmul(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m,
+                    size_t n, size_t k, bool bf16, void *stream)
 {
-    int rc = run_mmf(ctx, f, w, x, y, m, n, k, bf16, stream);
+    int rc = run_mmf(ctx, S, f, w, x, y, m, n, k, bf16, stream);
     if (rc >= 0) return rc;
     // up to 8 rows: the int8 kernel when one pass over the weights does it, else the GEMM
-    rc = run_mm8(ctx, f, w, x, y, m, n, k, bf16, stream, true);
+    rc = run_mm8(ctx, S, f, w, x, y, m, n, k, bf16, stream, true);
     if (rc >= 0) return rc;
     if (ctx->mmf_small_min_m > 0) {
-        rc = run_mmf(ctx, f, w, x, y, m, n, k, bf16, stream, ctx->mmf_small_min_m);
+        rc = run_mmf(ctx, S, f, w, x, y, m, n, k, bf16, stream, ctx->mmf_small_min_m);
         if (rc >= 0) return rc;
     }
-    rc = run_mm8(ctx, f, w, x, y, m, n, k, bf16, stream);
+    rc = run_mm8(ctx, S, f, w, x, y, m, n, k, bf16, stream);
     if (rc >= 0) return rc;
     return run_gemv(ctx, f, w, x, y, m, n, k, bf16, stream);
+}
+
+size_t ffn_h_bytes(size_t m, size_t ffn) { return ((m * ffn * sizeof(float)) + 255) & ~size_t(255); }
+size_t ffn_scratch_bytes(size_t m, size_t ffn) { return ffn_h_bytes(m, ffn) + m * 2 * ffn * sizeof(float); }
+
+// One validated quantized matmul with the scratch of `S` (call_mutex held).
+int matmul_on_scratch(gllmq_ctx *ctx, Scratch &S, const void *w, size_t w_bytes, const float *x, float *y, uint32_t dtype,
+                      size_t m, size_t n, size_t k, int act_mode, void *stream)
+{
+    const Format *f = find_format(dtype);
+    int rc = check_matmul_args(ctx, f, w, w_bytes, x, y, dtype, m, n, k);
+    if (rc >= 0) return rc;
+    if (act_mode != GLLMQ_ACT_F32_SPLIT && act_mode != GLLMQ_ACT_BF16)
+        return fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul: unknown activation mode %d", act_mode);
+    const bool bf16 = act_mode == GLLMQ_ACT_BF16;
+    if (bf16 && ctx->gemv_f32)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "quantized_matmul: bf16 activations are not built for the f32 GEMV flavour");
+    return dispatch_matmul(ctx, S, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
 }
 
 } // namespace
@@ -647,7 +789,7 @@ int gllmq_init(gllmq_ctx **out, int device)
             rc = get_function(ctx, &ctx->gemv_i8[i][m - 1], name);
         }
     }
-    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->stream_read, "gq_stream_read");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_route, "gq_moe_route");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[0], "gq_mmf_prep_t1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[1], "gq_mmf_prep_t2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_reduce, "gq_mmf_reduce");
@@ -679,17 +821,6 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->dequant_wave_q5k, "gq_dequant_q5k_wave");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->argmax_part, "gq_argmax_part");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->argmax_final, "gq_argmax_final");
-    if (rc == GLLMQ_OK) {
-        hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->argmax_keys),
-                                  sizeof(uint64_t) * gq::ARGMAX_MAX_ROWS * gq::ARGMAX_MAX_PARTS);
-        if (he != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "argmax scratch: %s", hipGetErrorString(he));
-    }
-    if (rc == GLLMQ_OK) {
-        hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->mm8_part), sizeof(float) * gq::MM8_SPLIT_PART_FLOATS);
-        if (he == hipSuccess) he = hipMalloc(reinterpret_cast<void **>(&ctx->mm8_arrive), sizeof(uint32_t) * gq::MM8_SPLIT_MAX_LISTS);
-        if (he == hipSuccess) he = hipMemset(ctx->mm8_arrive, 0, sizeof(uint32_t) * gq::MM8_SPLIT_MAX_LISTS);
-        if (he != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "K-split scratch: %s", hipGetErrorString(he));
-    }
     if (rc == GLLMQ_OK) {
         static const uint32_t kRows[8] = { 0, 1, 2, 3, 4, 5, 6, 7 };
         hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->identity_rows), sizeof kRows);
@@ -727,30 +858,6 @@ int gllmq_init(gllmq_ctx **out, int device)
         return rc;
     }
     ctx->gemv_waves = static_cast<uint32_t>(ctx->num_cus) * 8u;
-    if (const char *v = getenv("GLLMQ_GEMV_F32")) ctx->gemv_f32 = (v[0] == '1');
-    if (const char *v = getenv("GLLMQ_MM8")) ctx->use_mm8 = (v[0] != '0');
-    if (const char *v = getenv("GLLMQ_MMF")) ctx->use_mmf = (v[0] != '0');
-    if (const char *v = getenv("GLLMQ_FFN_FUSED")) ctx->ffn_fused = (v[0] != '0');
-    if (const char *v = getenv("GLLMQ_MMF_SMALL_MIN_M")) ctx->mmf_small_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
-    auto tune = [](const char *name) { const char *v = getenv(name); return v ? static_cast<uint32_t>(std::max(0, atoi(v))) : 0u; };
-    ctx->tune_mm8_grid = tune("GLLMQ_MM8_GRID");
-    ctx->tune_mmf_ksplit = tune("GLLMQ_MMF_KSPLIT");
-    ctx->tune_mmf_rows = tune("GLLMQ_MMF_ROWS");
-    ctx->tune_moe_job_waves = tune("GLLMQ_MOE_JOB_WAVES");
-    ctx->tune_moe_slices = tune("GLLMQ_MOE_SLICES");
-    if (const char *v = getenv("GLLMQ_MM8_AREG")) ctx->mm8_areg_on = (v[0] != '0');
-    if (const char *v = getenv("GLLMQ_MM8_KSPLIT")) ctx->mm8_ksplit_max = static_cast<uint32_t>(std::max(0, atoi(v)));
-    if (const char *v = getenv("GLLMQ_MM8_Q6K_MIN_M")) ctx->mm8_q6k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
-    if (const char *v = getenv("GLLMQ_MM8_Q5K_MIN_M")) ctx->mm8_q5k_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
-    if (const char *v = getenv("GLLMQ_MM8_Q8_0_MIN_M")) ctx->mm8_q8_0_min_m = static_cast<uint32_t>(std::max(0, atoi(v)));
-    if (const char *v = getenv("GLLMQ_MOE_MM8")) ctx->moe_mm8 = (v[0] != '0');
-    if (const char *v = getenv("GLLMQ_MOE_MM8_Q6K")) ctx->moe_mm8_q6k = (v[0] != '0');
-    if (const char *v = getenv("GLLMQ_MOE_MM8_ROWS")) ctx->moe_mm8_rows = (v[0] != '0');
-    if (const char *v = getenv("GLLMQ_MOE_GLU")) ctx->moe_glu = (v[0] != '0');
-    if (const char *v = getenv("GLLMQ_GEMV_WAVES")) {
-        long w = strtol(v, nullptr, 10);
-        if (w >= 4 && w <= 65536) ctx->gemv_waves = static_cast<uint32_t>(w);
-    }
     *out = ctx;
     return GLLMQ_OK;
 }
@@ -758,13 +865,10 @@ int gllmq_init(gllmq_ctx **out, int device)
 void gllmq_destroy(gllmq_ctx *ctx)
 {
     if (!ctx) return;
-    if (ctx->workspace) (void)hipFree(ctx->workspace);
+    for (Scratch &S : ctx->scratch) free_scratch(S);
+    for (CachedWeights &W : ctx->weights)
+        if (W.dev) (void)hipFree(W.dev);
     if (ctx->identity_rows) (void)hipFree(ctx->identity_rows);
-    if (ctx->mm8_part) (void)hipFree(ctx->mm8_part);
-    if (ctx->mm8_arrive) (void)hipFree(ctx->mm8_arrive);
-    if (ctx->argmax_keys) (void)hipFree(ctx->argmax_keys);
-    if (ctx->ffn_scratch) (void)hipFree(ctx->ffn_scratch);
-    if (ctx->mmf_partial) (void)hipFree(ctx->mmf_partial);
     if (ctx->module) (void)hipModuleUnload(ctx->module);
     delete ctx;
 }
@@ -772,13 +876,52 @@ void gllmq_destroy(gllmq_ctx *ctx)
 const char *gllmq_last_error(const gllmq_ctx *ctx)
 {
     if (!ctx) return "NULL context";
-    return ctx->err.c_str();
+    // a copy per calling thread: another thread's failing call may replace the context's string
+    static thread_local std::string copy;
+    {
+        std::lock_guard<std::mutex> g(const_cast<gllmq_ctx *>(ctx)->err_mutex);
+        copy = ctx->err;
+    }
+    return copy.c_str();
+}
+
+int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    if (!name) return fail(ctx, GLLMQ_ERR_INVALID, "set_option: NULL name");
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    const std::string n(name);
+    const uint32_t u = static_cast<uint32_t>(std::max(0l, value));
+    if (n == "gemv_f32") ctx->gemv_f32 = value != 0;
+    else if (n == "mm8") ctx->use_mm8 = value != 0;
+    else if (n == "mmf") ctx->use_mmf = value != 0;
+    else if (n == "ffn_fused") ctx->ffn_fused = value != 0;
+    else if (n == "mmf_small_min_m") ctx->mmf_small_min_m = u;
+    else if (n == "mm8_ksplit") ctx->mm8_ksplit_max = u;
+    else if (n == "mm8_q6k_min_m") ctx->mm8_q6k_min_m = u;
+    else if (n == "mm8_q5k_min_m") ctx->mm8_q5k_min_m = u;
+    else if (n == "mm8_q8_0_min_m") ctx->mm8_q8_0_min_m = u;
+    else if (n == "moe_mm8") ctx->moe_mm8 = value != 0;
+    else if (n == "moe_mm8_q6k") ctx->moe_mm8_q6k = value != 0;
+    else if (n == "moe_mm8_rows") ctx->moe_mm8_rows = value != 0;
+    else if (n == "moe_glu") ctx->moe_glu = value != 0;
+    else if (n == "weights_cache_mib") ctx->weights_cache_limit = static_cast<size_t>(u) << 20;
+    else return fail(ctx, GLLMQ_ERR_INVALID, "set_option: unknown option %s", name);
+    return GLLMQ_OK;
+}
+
+const char *gllmq_last_kernel_name(const gllmq_ctx *ctx)
+{
+    if (!ctx || !ctx->last_kernel) return "";
+    const auto it = ctx->kernel_names.find(ctx->last_kernel);
+    return it == ctx->kernel_names.end() ? "" : it->second.c_str();
 }
 
 int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *out, size_t n_out,
                      uint32_t dtype, void *stream)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     const Format *f = find_format(dtype);
     if (!f)
         return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
@@ -802,6 +945,7 @@ int gllmq_quant_gather(gllmq_ctx *ctx, const void *table, size_t table_bytes, ui
                        size_t hidden, const uint32_t *ids, size_t count, float scale, float *out, void *stream)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     const Format *f = find_format(dtype);
     if (!f)
         return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
@@ -837,14 +981,18 @@ int gllmq_argmax(gllmq_ctx *ctx, const float *logits, size_t rows, size_t n, siz
                  void *stream)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     if (rows == 0) return GLLMQ_OK;
     if ((!logits && n > 0) || !token) return fail(ctx, GLLMQ_ERR_INVALID, "argmax: NULL device pointer");
     if (n > 0xFFFFFFFEu || ld > 0xFFFFFFFFu || rows > 0x7FFFFFFFu || ld < n)
         return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "argmax: n = %zu, ld = %zu, rows = %zu out of range", n, ld, rows);
     if (!aligned(logits, 4) || !aligned(token, 4) || (value && !aligned(value, 4)))
         return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "argmax: buffers must be 4-byte aligned");
+    Scratch *S = nullptr;
+    int src = acquire_scratch(ctx, stream, &S);
+    if (src != GLLMQ_OK) return src;
     ArgmaxParams P{};
-    P.keys = ctx->argmax_keys;
+    P.keys = S->argmax_keys;
     P.n = static_cast<uint32_t>(n);
     P.ld = static_cast<uint32_t>(ld);
     P.parts = static_cast<uint32_t>(std::min<size_t>(gq::ARGMAX_MAX_PARTS, std::max<size_t>(1, (n + 4095) / 4096)));
@@ -865,15 +1013,11 @@ int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, con
                               uint32_t dtype, size_t m, size_t n, size_t k, int act_mode, void *stream)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
-    const Format *f = find_format(dtype);
-    int rc = check_matmul_args(ctx, f, w, w_bytes, x, y, dtype, m, n, k);
-    if (rc >= 0) return rc;
-    if (act_mode != GLLMQ_ACT_F32_SPLIT && act_mode != GLLMQ_ACT_BF16)
-        return fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul: unknown activation mode %d", act_mode);
-    const bool bf16 = act_mode == GLLMQ_ACT_BF16;
-    if (bf16 && ctx->gemv_f32)
-        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "quantized_matmul: bf16 activations are not built for GLLMQ_GEMV_F32=1");
-    return dispatch_matmul(ctx, *f, static_cast<const uint8_t *>(w), x, y, m, n, k, bf16, stream);
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    Scratch *S = nullptr;
+    int rc = acquire_scratch(ctx, stream, &S);
+    if (rc != GLLMQ_OK) return rc;
+    return matmul_on_scratch(ctx, *S, w, w_bytes, x, y, dtype, m, n, k, act_mode, stream);
 }
 
 int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_t gate_up_bytes_each, uint32_t dtype_gate_up,
@@ -881,6 +1025,7 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_
                      size_t hidden, size_t ffn, int relu_gate, void *stream)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     const Format *fg = find_format(dtype_gate_up), *fd = find_format(dtype_down);
     if (!fg || !fd)
         return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
@@ -900,29 +1045,21 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_
     if (ffn > 0x7FFFFFFFu / 2u) return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "ffn_swiglu: ffn exceeds 2^30-1");
 
     // scratch: h [m][ffn], then gate/up results [m][2 ffn] for the form with three steps
-    const size_t h_bytes = ((m * ffn * sizeof(float)) + 255) & ~size_t(255);
-    const size_t need = h_bytes + m * 2 * ffn * sizeof(float);
-    {
-        std::lock_guard<std::mutex> guard(ctx->workspace_mutex);
-        GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
-        if (ctx->ffn_scratch_bytes < need) {
-            if (ctx->ffn_scratch) {
-                GLLMQ_HIP(ctx, hipDeviceSynchronize()); // earlier calls may still be using it
-                GLLMQ_HIP(ctx, hipFree(ctx->ffn_scratch));
-                ctx->ffn_scratch = nullptr;
-                ctx->ffn_scratch_bytes = 0;
-            }
-            GLLMQ_HIP(ctx, hipMalloc(&ctx->ffn_scratch, need));
-            ctx->ffn_scratch_bytes = need;
-        }
-    }
-    float *h = static_cast<float *>(ctx->ffn_scratch);
-    float *gu = reinterpret_cast<float *>(static_cast<uint8_t *>(ctx->ffn_scratch) + h_bytes);
+    const size_t h_bytes = ffn_h_bytes(m, ffn);
+    const size_t need = ffn_scratch_bytes(m, ffn);
+    Scratch *Sp = nullptr;
+    rc = acquire_scratch(ctx, stream, &Sp);
+    if (rc != GLLMQ_OK) return rc;
+    Scratch &S = *Sp;
+    rc = grow_scratch(ctx, S, &S.ffn, &S.ffn_bytes, need, stream, "ffn_swiglu");
+    if (rc != GLLMQ_OK) return rc;
+    float *h = static_cast<float *>(S.ffn);
+    float *gu = reinterpret_cast<float *>(static_cast<uint8_t *>(S.ffn) + h_bytes);
     const uint8_t *gw = static_cast<const uint8_t *>(gate_w), *uw = static_cast<const uint8_t *>(up_w);
 
     // gate and up in one launch with the activation in its epilogue (Q4_K / Q5_K, up to 8 rows)
     rc = -1;
-    if (ctx->ffn_fused && m <= 8) rc = run_mm8(ctx, *fg, gw, x, h, m, ffn, hidden, false, stream, true, uw, relu_gate != 0);
+    if (ctx->ffn_fused && m <= 8) rc = run_mm8(ctx, S, *fg, gw, x, h, m, ffn, hidden, false, stream, true, uw, relu_gate != 0);
     if (rc > 0) return rc;
     if (rc < 0) {
         // three steps: the two products (one matmul when the up rows follow the gate rows in
@@ -935,13 +1072,13 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_
         A.ffn = static_cast<uint32_t>(ffn);
         A.relu_gate = relu_gate ? 1u : 0u;
         if (stacked) {
-            rc = dispatch_matmul(ctx, *fg, gw, x, gu, m, 2 * ffn, hidden, false, stream);
+            rc = dispatch_matmul(ctx, S, *fg, gw, x, gu, m, 2 * ffn, hidden, false, stream);
             A.g = gu;
             A.u = gu + ffn;
             A.ld = static_cast<uint32_t>(2 * ffn);
         } else {
-            rc = dispatch_matmul(ctx, *fg, gw, x, gu, m, ffn, hidden, false, stream);
-            if (rc == GLLMQ_OK) rc = dispatch_matmul(ctx, *fg, uw, x, gu + m * ffn, m, ffn, hidden, false, stream);
+            rc = dispatch_matmul(ctx, S, *fg, gw, x, gu, m, ffn, hidden, false, stream);
+            if (rc == GLLMQ_OK) rc = dispatch_matmul(ctx, S, *fg, uw, x, gu + m * ffn, m, ffn, hidden, false, stream);
             A.g = gu;
             A.u = gu + m * ffn;
             A.ld = static_cast<uint32_t>(ffn);
@@ -951,7 +1088,7 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_
                       static_cast<uint32_t>(std::min<size_t>(m, 65535)), 256, 0, stream, &A, sizeof A);
         if (rc != GLLMQ_OK) return rc;
     }
-    return dispatch_matmul(ctx, *fd, static_cast<const uint8_t *>(down_w), h, out, m, hidden, ffn, false, stream);
+    return dispatch_matmul(ctx, S, *fd, static_cast<const uint8_t *>(down_w), h, out, m, hidden, ffn, false, stream);
 }
 
 int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y,
@@ -963,29 +1100,106 @@ int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w, size_t w_bytes, const 
 int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs, size_t count, void *stream)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     if (count && !descs) return fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul_batch: NULL descriptor list");
+    Scratch *S = nullptr;
+    int rc = acquire_scratch(ctx, stream, &S);
+    if (rc != GLLMQ_OK) return rc;
     for (size_t i = 0; i < count; ++i) {
         const gllmq_matmul_desc &d = descs[i];
-        int rc = gllmq_quantized_matmul(ctx, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k,
-                                        stream);
+        rc = matmul_on_scratch(ctx, *S, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k,
+                               GLLMQ_ACT_F32_SPLIT, stream);
         if (rc != GLLMQ_OK) return rc;
     }
     return GLLMQ_OK;
 }
 
-int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, const void *down, uint32_t dtype_dn,
-                     const float *x, float *out, size_t tokens, size_t hidden, size_t ffn, size_t experts,
-                     size_t top_k, const uint32_t *route_expert, const float *route_weight,
-                     const uint32_t *route_len, int relu_gate, void *stream)
+int gllmq_moe_route(gllmq_ctx *ctx, const float *logits, size_t tokens, size_t experts, size_t top_k,
+                    float capacity_factor, uint32_t *route_expert, float *route_weight, uint32_t *route_len,
+                    uint32_t *route_pos, uint32_t *expert_counts, uint32_t *overflow, void *stream)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    if (tokens == 0) return GLLMQ_OK;
+    if (!logits || !route_expert || !route_weight || !route_len)
+        return fail(ctx, GLLMQ_ERR_INVALID, "moe_route: NULL device pointer");
+    if (experts == 0 || top_k == 0) return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "moe_route: experts and top_k must be positive");
+    if (experts > gq::ROUTE_MAX_EXPERTS || top_k > gq::ROUTE_MAX_TOP_K || tokens > 0x7FFFFFFFu / top_k)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "moe_route: experts = %zu (max %u), top_k = %zu (max %u) or tokens = %zu is beyond this build",
+                    experts, gq::ROUTE_MAX_EXPERTS, top_k, gq::ROUTE_MAX_TOP_K, tokens);
+    if (!aligned(logits, 4) || !aligned(route_expert, 4) || !aligned(route_weight, 4) || !aligned(route_len, 4))
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "moe_route: buffers must be 4-byte aligned");
+    gq::MoeRouteParams P{};
+    P.logits = logits;
+    P.route_expert = route_expert;
+    P.route_weight = route_weight;
+    P.route_len = route_len;
+    P.route_pos = route_pos;
+    P.expert_counts = expert_counts;
+    P.overflow = overflow;
+    P.tokens = static_cast<uint32_t>(tokens);
+    P.experts = static_cast<uint32_t>(experts);
+    P.top_k = static_cast<uint32_t>(top_k);
+    // ExpertRouteConfig::expert_capacity (src/moe/routing.rs:53-61): the same f32 arithmetic
+    float cap = std::ceil(capacity_factor * static_cast<float>(tokens) / static_cast<float>(experts));
+    if (!(cap >= 0.0f)) cap = 0.0f; // negative or NaN
+    if (cap > 1.0e9f) cap = 1.0e9f;
+    P.capacity = static_cast<uint32_t>(cap);
+    const uint32_t lds = static_cast<uint32_t>((gq::ROUTE_WAVES + 1) * experts * 4);
+    if (tokens <= gq::ROUTE_FUSED_MAX_TOKENS) {
+        P.phases = 3u;
+        return launch(ctx, ctx->moe_route, 1, gq::ROUTE_THREADS, lds, stream, &P, sizeof P);
+    }
+    P.phases = 1u;
+    const uint32_t grid = static_cast<uint32_t>(std::min<size_t>((tokens + gq::ROUTE_WAVES - 1) / gq::ROUTE_WAVES,
+                                                                 static_cast<size_t>(ctx->num_cus) * 4));
+    int rc = launch(ctx, ctx->moe_route, grid, gq::ROUTE_THREADS, lds, stream, &P, sizeof P);
+    if (rc != GLLMQ_OK) return rc;
+    P.phases = 2u;
+    return launch(ctx, ctx->moe_route, 1, gq::ROUTE_THREADS, lds, stream, &P, sizeof P);
+}
+
+namespace {
+
+// Carve-up of the MoE workspace (256-byte aligned pieces).
+struct MoeWorkspace {
+    size_t src, pos, jobs, jobs8, cnt, gu, h, o, total;
+};
+
+MoeWorkspace moe_workspace(size_t pairs, size_t hidden, size_t ffn)
+{
+    auto up256 = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+    MoeWorkspace W{};
+    size_t off = 0;
+    W.src = off; off = up256(off + pairs * 4);
+    W.pos = off; off = up256(off + pairs * 4);
+    W.jobs = off; off = up256(off + pairs * sizeof(MoeJob));
+    W.jobs8 = off; off = up256(off + pairs * sizeof(MoeJob8));
+    W.cnt = off; off = up256(off + 4 * 4);
+    W.gu = off; off = up256(off + pairs * 2 * ffn * 4);
+    W.h = off; off = up256(off + pairs * ffn * 4);
+    W.o = off; off = up256(off + pairs * hidden * 4);
+    W.total = off;
+    return W;
+}
+
+} // namespace
+
+int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate, size_t gate_bytes, size_t gate_expert_stride, const void *up,
+                     size_t up_bytes, size_t up_expert_stride, uint32_t dtype_gu, const void *down, size_t down_bytes,
+                     size_t down_expert_stride, uint32_t dtype_dn, const float *x, float *out, size_t tokens,
+                     size_t hidden, size_t ffn, size_t experts, size_t top_k, const uint32_t *route_expert,
+                     const float *route_weight, const uint32_t *route_len, int relu_gate, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     const Format *fg = find_format(dtype_gu), *fd = find_format(dtype_dn);
     if (!fg || !fd)
         return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
                     "moe_matvec: ggml dtype %u / %u is not covered (supported: Q8_0=8, Q4_K=12, Q5_K=13, Q6_K=14)",
                     dtype_gu, dtype_dn);
     if (tokens == 0 || hidden == 0) return GLLMQ_OK;
-    if (!gate_up || !down || !x || !out || !route_expert || !route_weight || !route_len)
+    if (!gate || !up || !down || !x || !out || !route_expert || !route_weight || !route_len)
         return fail(ctx, GLLMQ_ERR_INVALID, "moe_matvec: NULL device pointer");
     if (ffn == 0 || experts == 0 || top_k == 0)
         return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "moe_matvec: ffn, experts and top_k must be positive");
@@ -1002,59 +1216,55 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
     if (hidden % 4 != 0 || ffn % 4 != 0)
         return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "moe_matvec: hidden and ffn must be multiples of 4");
     const size_t rb_gu = gllmq_row_bytes(dtype_gu, hidden), rb_dn = gllmq_row_bytes(dtype_dn, ffn);
-    if (!aligned(gate_up, fg->w_align) || rb_gu % fg->w_align != 0 || !aligned(down, fd->w_align) ||
-        rb_dn % fd->w_align != 0)
-        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "moe_matvec: expert weights miss the alignment of their format");
+    // every expert's matrix must lie inside its buffer
+    const size_t gu_each = ffn * rb_gu, dn_each = hidden * rb_dn;
+    auto inside = [&](size_t bytes, size_t stride, size_t each) {
+        return stride >= each && bytes >= each && (experts - 1) <= (bytes - each) / stride;
+    };
+    if (!inside(gate_bytes, gate_expert_stride, gu_each) || !inside(up_bytes, up_expert_stride, gu_each) ||
+        !inside(down_bytes, down_expert_stride, dn_each))
+        return fail(ctx, GLLMQ_ERR_BAD_SHAPE,
+                    "moe_matvec: %zu experts of %zu (gate, up) / %zu (down) bytes at strides %zu / %zu / %zu do not fit buffers of "
+                    "%zu / %zu / %zu bytes", experts, gu_each, dn_each, gate_expert_stride, up_expert_stride, down_expert_stride,
+                    gate_bytes, up_bytes, down_bytes);
+    if (!aligned(gate, fg->w_align) || !aligned(up, fg->w_align) || rb_gu % fg->w_align != 0 ||
+        gate_expert_stride % fg->w_align != 0 || up_expert_stride % fg->w_align != 0 || !aligned(down, fd->w_align) ||
+        rb_dn % fd->w_align != 0 || down_expert_stride % fd->w_align != 0)
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "moe_matvec: expert weights or strides miss the alignment of their format");
     if (!aligned(x, 16) || !aligned(out, 4))
         return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "moe_matvec: x must be 16-byte and out 4-byte aligned");
 
-    // workspace carve-up (256-byte aligned pieces)
-    auto up256 = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
-    size_t off = 0;
-    const size_t o_src = off; off = up256(off + pairs * 4);
-    const size_t o_pos = off; off = up256(off + pairs * 4);
-    const size_t o_jobs = off; off = up256(off + pairs * sizeof(MoeJob));
-    const size_t o_jobs8 = off; off = up256(off + pairs * sizeof(MoeJob8));
-    const size_t o_cnt = off; off = up256(off + 4 * 4);
-    const size_t o_gu = off; off = up256(off + pairs * 2 * ffn * 4);
-    const size_t o_h = off; off = up256(off + pairs * ffn * 4);
-    const size_t o_o = off; off = up256(off + pairs * hidden * 4);
-    std::lock_guard<std::mutex> guard(ctx->workspace_mutex);
-    if (ctx->workspace_bytes < off) {
-        GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
-        if (ctx->workspace) {
-            GLLMQ_HIP(ctx, hipDeviceSynchronize()); // earlier calls may still be reading it
-            GLLMQ_HIP(ctx, hipFree(ctx->workspace));
-            ctx->workspace = nullptr;
-            ctx->workspace_bytes = 0;
-        }
-        GLLMQ_HIP(ctx, hipMalloc(&ctx->workspace, off));
-        ctx->workspace_bytes = off;
-    }
-    uint8_t *ws = static_cast<uint8_t *>(ctx->workspace);
-    uint32_t *pair_src = reinterpret_cast<uint32_t *>(ws + o_src);
-    uint32_t *pair_pos = reinterpret_cast<uint32_t *>(ws + o_pos);
-    MoeJob *jobs = reinterpret_cast<MoeJob *>(ws + o_jobs);
-    MoeJob8 *jobs8 = reinterpret_cast<MoeJob8 *>(ws + o_jobs8);
-    uint32_t *counters = reinterpret_cast<uint32_t *>(ws + o_cnt);
-    float *gu = reinterpret_cast<float *>(ws + o_gu);
-    float *h = reinterpret_cast<float *>(ws + o_h);
-    float *o = reinterpret_cast<float *>(ws + o_o);
+    const MoeWorkspace W = moe_workspace(pairs, hidden, ffn);
+    Scratch *Sp = nullptr;
+    int rc = acquire_scratch(ctx, stream, &Sp);
+    if (rc != GLLMQ_OK) return rc;
+    rc = grow_scratch(ctx, *Sp, &Sp->moe, &Sp->moe_bytes, W.total, stream, "moe_matvec");
+    if (rc != GLLMQ_OK) return rc;
+    uint8_t *ws = static_cast<uint8_t *>(Sp->moe);
+    uint32_t *pair_src = reinterpret_cast<uint32_t *>(ws + W.src);
+    uint32_t *pair_pos = reinterpret_cast<uint32_t *>(ws + W.pos);
+    MoeJob *jobs = reinterpret_cast<MoeJob *>(ws + W.jobs);
+    MoeJob8 *jobs8 = reinterpret_cast<MoeJob8 *>(ws + W.jobs8);
+    uint32_t *counters = reinterpret_cast<uint32_t *>(ws + W.cnt);
+    float *gu = reinterpret_cast<float *>(ws + W.gu);
+    float *h = reinterpret_cast<float *>(ws + W.h);
+    float *o = reinterpret_cast<float *>(ws + W.o);
 
     const uint32_t fast = pairs <= 4096 ? 1u : 0u; // per-pair placement: quadratic in the pairs, but without serial LDS walks
     {
         MoePlanParams P{ route_expert, route_len, pair_src, pair_pos, jobs, jobs8, counters, static_cast<uint32_t>(tokens),
                          static_cast<uint32_t>(top_k), static_cast<uint32_t>(experts), static_cast<uint32_t>(pairs), fast };
         const uint32_t lds = static_cast<uint32_t>((pairs + 4 * experts + 4 + (fast ? 2 * pairs : 0)) * 4);
-        int rc = launch(ctx, ctx->moe_plan, 1, 256, lds, stream, &P, sizeof P);
+        rc = launch(ctx, ctx->moe_plan, 1, 256, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }
     // Waves per job: the device takes about 8 waves per CU of these kernels; the jobs that
     // exist (at most `pairs`, typically one per routed expert) share them.
-    uint32_t job_waves = std::max<uint32_t>(16u, 4u * ctx->gemv_waves / static_cast<uint32_t>(pairs));
-    if (ctx->tune_moe_job_waves) job_waves = std::max(4u, ctx->tune_moe_job_waves);
-    auto grouped = [&](const Format &f, const void *w, size_t rb, uint32_t n, uint32_t k, const float *xin,
-                       bool x_by_token, float *yout) -> int {
+    const uint32_t job_waves = std::max<uint32_t>(16u, 4u * ctx->gemv_waves / static_cast<uint32_t>(pairs));
+    // n rows of k elements per expert, experts `stride` bytes apart; the results of a pair go to
+    // yout + its sorted position * y_stride.
+    auto grouped = [&](const Format &f, const void *w, size_t stride, size_t rb, uint32_t n, uint32_t k, const float *xin,
+                       bool x_by_token, float *yout, uint32_t y_stride) -> int {
         GemvPlan L = plan_gemv(ctx, 2, n, k, rb, job_waves);
         MoeGemvParams Q{};
         Q.g = L.P;
@@ -1065,23 +1275,25 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         Q.g.accumulate = 0;
         Q.jobs = jobs;
         Q.counters = counters;
-        Q.expert_stride = static_cast<uint64_t>(n) * rb;
+        Q.expert_stride = stride;
         Q.wgs_per_job = L.grid;
         Q.x_by_token = x_by_token ? 1u : 0u;
         Q.x_stride = k;
-        Q.y_stride = n;
+        Q.y_stride = y_stride;
         const uint64_t grid = static_cast<uint64_t>(L.grid) * pairs;
         if (grid > 0x7FFFFFFFull) return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "moe_matvec: launch grid too large");
         return launch(ctx, ctx->moe_gemv[format_index(f.dtype)], static_cast<uint32_t>(grid), L.threads, L.lds, stream,
                       &Q, sizeof Q);
     };
-    // Q4_K and Q6_K with rows of at most 16 blocks go to the int8 matrix cores, every token of
-    // an expert (up to eight per job) in one pass over its weights.  `by_token`: the activation
+    // Q4_K, Q5_K and Q6_K with rows of at most 16 blocks go to the int8 matrix cores, every token
+    // of an expert (up to eight per job) in one pass over its weights.  `by_token`: the activation
     // rows are x[token] (gate/up), else rows by sorted position (down).
-    // `glu`: n counts the gate rows of an expert, its n up rows follow them, and yout receives
-    // act(gate . x) * (up . x)
-    auto grouped_mm8 = [&](const Format &f, const void *wbase, size_t rb, uint32_t n, uint32_t k, const float *xin,
-                           bool by_token, float *yout, bool glu = false) -> int {
+    // `up_w` != null: the gated form, n gate rows per expert at `wbase` and n up rows at `up_w`,
+    // and yout receives act(gate . x) * (up . x)
+    auto grouped_mm8 = [&](const Format &f, const void *wbase, size_t stride, size_t rb, uint32_t n, uint32_t k,
+                           const float *xin, bool by_token, float *yout, uint32_t y_stride, const void *up_w = nullptr,
+                           size_t up_stride = 0) -> int {
+        const bool glu = up_w != nullptr;
         const int kind = mm8_kind(f.dtype);
         const bool q6k = kind == MM8_Q6K;
         const uint32_t groups = (k + 255u) / 256u;
@@ -1097,14 +1309,15 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         Q.g.tiles = (n + 31u) / 32u;
         Q.jobs = jobs8;
         Q.counters = counters;
-        Q.expert_stride = static_cast<uint64_t>(n) * rb * (glu ? 2u : 1u);
-        Q.y_stride = n;
+        Q.expert_stride = stride;
+        Q.up = static_cast<const uint8_t *>(up_w);
+        Q.up_stride = up_stride;
+        Q.y_stride = y_stride;
         Q.g.glu_relu = relu_gate ? 1u : 0u;
         Q.rows = by_token ? nullptr : ctx->identity_rows;
         // upper bound of the jobs: one per expert hit, plus one per eight further pairs
         const uint64_t max_jobs = std::min<uint64_t>(pairs, experts + pairs / 8);
         uint32_t slices = std::max<uint32_t>(1u, (3u * static_cast<uint32_t>(ctx->num_cus)) / (2u * static_cast<uint32_t>(std::min<uint64_t>(pairs, experts))));
-        if (ctx->tune_moe_slices) slices = ctx->tune_moe_slices;
         const uint32_t ppt = (groups + 7u) / 8u;
         hipFunction_t fn = glu ? ctx->moe_mm8_glu_fn[kind][ppt - 1] : ctx->moe_mm8_fn[kind][ppt - 1];
         uint32_t units = Q.g.tiles; // what the slices of a job share: tiles, or groups of eight tiles
@@ -1125,65 +1338,178 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up, uint32_t dtype_gu, con
         if (kind == MM8_Q6K && !ctx->moe_mm8_q6k) return false;
         return mm8_lds_bytes(groups, 8, 4, kind) <= 160u * 1024u;
     };
-    int rc = GLLMQ_OK;
+    const uint32_t F = static_cast<uint32_t>(ffn), H = static_cast<uint32_t>(hidden);
     const bool gated = fits_mm8(*fg, hidden, true); // gate, up and the activation in one launch
-    if (gated)
-        rc = grouped_mm8(*fg, gate_up, rb_gu, static_cast<uint32_t>(ffn), static_cast<uint32_t>(hidden), x, true, h, true);
-    else if (fits_mm8(*fg, hidden))
-        rc = grouped_mm8(*fg, gate_up, rb_gu, static_cast<uint32_t>(2 * ffn), static_cast<uint32_t>(hidden), x, true, gu);
-    else
-        rc = grouped(*fg, gate_up, rb_gu, static_cast<uint32_t>(2 * ffn), static_cast<uint32_t>(hidden), x, true, gu);
+    if (gated) {
+        rc = grouped_mm8(*fg, gate, gate_expert_stride, rb_gu, F, H, x, true, h, F, up, up_expert_stride);
+    } else {
+        // an expert's up rows right behind its gate rows, both under one stride: one matrix of
+        // 2 * ffn rows; otherwise the two halves of gu[pair][2 ffn] come from a launch each
+        const bool stacked = static_cast<const uint8_t *>(up) == static_cast<const uint8_t *>(gate) + gu_each &&
+                             up_expert_stride == gate_expert_stride;
+        const bool mm8 = fits_mm8(*fg, hidden);
+        for (int half = 0; half < (stacked ? 1 : 2) && rc == GLLMQ_OK; ++half) {
+            const void *wb = half ? up : gate;
+            const size_t st = half ? up_expert_stride : gate_expert_stride;
+            const uint32_t rows = stacked ? 2u * F : F;
+            if (mm8) rc = grouped_mm8(*fg, wb, st, rb_gu, rows, H, x, true, gu + half * ffn, 2u * F);
+            else rc = grouped(*fg, wb, st, rb_gu, rows, H, x, true, gu + half * ffn, 2u * F);
+        }
+    }
     if (rc != GLLMQ_OK) return rc;
     if (!gated) {
-        MoeActParams P{ gu, h, counters, static_cast<uint32_t>(ffn), relu_gate ? 1u : 0u };
-        rc = launch2d(ctx, ctx->moe_act, static_cast<uint32_t>((ffn + 255) / 256), static_cast<uint32_t>(pairs), 256, 0,
-                      stream, &P, sizeof P);
+        MoeActParams P{ gu, h, counters, F, relu_gate ? 1u : 0u };
+        rc = launch2d(ctx, ctx->moe_act, (F + 255u) / 256u, static_cast<uint32_t>(pairs), 256, 0, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
     }
-    if (fits_mm8(*fd, ffn))
-        rc = grouped_mm8(*fd, down, rb_dn, static_cast<uint32_t>(hidden), static_cast<uint32_t>(ffn), h, false, o);
-    else
-        rc = grouped(*fd, down, rb_dn, static_cast<uint32_t>(hidden), static_cast<uint32_t>(ffn), h, false, o);
+    if (fits_mm8(*fd, ffn)) rc = grouped_mm8(*fd, down, down_expert_stride, rb_dn, H, F, h, false, o, H);
+    else rc = grouped(*fd, down, down_expert_stride, rb_dn, H, F, h, false, o, H);
     if (rc != GLLMQ_OK) return rc;
     MoeCombineParams C{ o, route_weight, route_len, pair_pos, out, static_cast<uint32_t>(tokens),
-                        static_cast<uint32_t>(top_k), static_cast<uint32_t>(hidden) };
-    return launch2d(ctx, ctx->moe_combine, static_cast<uint32_t>((hidden + 255) / 256), static_cast<uint32_t>(tokens),
-                    256, 0, stream, &C, sizeof C);
+                        static_cast<uint32_t>(top_k), H };
+    return launch2d(ctx, ctx->moe_combine, (H + 255u) / 256u, static_cast<uint32_t>(tokens), 256, 0, stream, &C, sizeof C);
 }
 
-int gllmq_stream_read(gllmq_ctx *ctx, const void *buf, size_t n_bytes, void *sink, void *stream)
+int gq_quantized_matmul_on_block(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y, uint32_t dtype,
+                                 size_t m, size_t n, size_t k, void *block, size_t block_bytes, void *stream)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
-    if (!buf || !sink) return fail(ctx, GLLMQ_ERR_INVALID, "stream_read: NULL device pointer");
-    if (!aligned(buf, 16) || n_bytes % 16 != 0)
-        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "stream_read: buffer must be 16-byte aligned and sized");
-    struct { const void *b; uint64_t n; void *s; } args = { buf, n_bytes / 16, sink };
-    return launch(ctx, ctx->stream_read, static_cast<uint32_t>(ctx->num_cus) * 8u, 256, 0, stream, &args, sizeof args);
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    if (!block || block_bytes < kScratchFixedBytes || !aligned(block, 256))
+        return fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul: scratch block missing, misaligned or under %zu bytes", kScratchFixedBytes);
+    static_assert(kScratchArriveBytes == GQ_BLOCK_ZEROED_BYTES, "the arrival counters are the zeroed head of the block");
+    Scratch S;
+    S.stream = static_cast<hipStream_t>(stream);
+    S.fixed = true;
+    carve_fixed(S, block);
+    S.mmf = static_cast<uint8_t *>(block) + kScratchFixedBytes;
+    S.mmf_bytes = block_bytes - kScratchFixedBytes;
+    return matmul_on_scratch(ctx, S, w, w_bytes, x, y, dtype, m, n, k, GLLMQ_ACT_F32_SPLIT, stream);
+}
+
+namespace {
+
+// Device copy of a host weight slice, uploaded on first sight and kept (call_mutex held).  The key is
+// the slice itself (address and length): the reference treats weights as immutable once loaded
+// and keeps its uploaded blob by length alone (src/compat/hip_backend.rs:141-156).
+int cached_weights(gllmq_ctx *ctx, const void *host, size_t bytes, void **dev)
+{
+    ++ctx->use_counter;
+    for (CachedWeights &W : ctx->weights)
+        if (W.host == host && W.bytes == bytes) {
+            W.last_use = ctx->use_counter;
+            *dev = W.dev;
+            return GLLMQ_OK;
+        }
+    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
+    // make room: least recently used first
+    size_t held = 0;
+    for (const CachedWeights &W : ctx->weights) held += W.bytes;
+    while (!ctx->weights.empty() && held + bytes > ctx->weights_cache_limit) {
+        size_t lru = 0;
+        for (size_t i = 1; i < ctx->weights.size(); ++i)
+            if (ctx->weights[i].last_use < ctx->weights[lru].last_use) lru = i;
+        GLLMQ_HIP(ctx, hipDeviceSynchronize());
+        (void)hipFree(ctx->weights[lru].dev);
+        held -= ctx->weights[lru].bytes;
+        ctx->weights.erase(ctx->weights.begin() + static_cast<long>(lru));
+    }
+    CachedWeights W;
+    W.host = host;
+    W.bytes = bytes;
+    W.last_use = ctx->use_counter;
+    GLLMQ_HIP(ctx, hipMalloc(&W.dev, bytes));
+    hipError_t e = hipMemcpy(W.dev, host, bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(W.dev);
+        return fail(ctx, GLLMQ_ERR_HIP, "weight upload: %s", hipGetErrorString(e));
+    }
+    ++ctx->weight_uploads;
+    ctx->weights.push_back(W);
+    *dev = W.dev;
+    return GLLMQ_OK;
+}
+
+} // namespace
+
+void gllmq_weights_forget(gllmq_ctx *ctx, const void *host)
+{
+    if (!ctx) return;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    for (size_t i = 0; i < ctx->weights.size();) {
+        if (host == nullptr || ctx->weights[i].host == host) {
+            (void)hipDeviceSynchronize();
+            (void)hipFree(ctx->weights[i].dev);
+            ctx->weights.erase(ctx->weights.begin() + static_cast<long>(i));
+        } else {
+            ++i;
+        }
+    }
+}
+
+uint64_t gllmq_weight_uploads(const gllmq_ctx *ctx) { return ctx ? ctx->weight_uploads : 0; }
+
+int gllmq_reserve_matmul(gllmq_ctx *ctx, uint32_t dtype, size_t m, size_t n, size_t k, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    if (!find_format(dtype))
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED, "reserve_matmul: ggml dtype %u is not covered", dtype);
+    Scratch *S = nullptr;
+    int rc = acquire_scratch(ctx, stream, &S);
+    if (rc != GLLMQ_OK || m == 0 || n == 0 || k == 0) return rc;
+    // the GEMM is the only matmul kernel family whose scratch depends on the shape; it may take
+    // any call of 3 rows and more
+    if (m < 3) return GLLMQ_OK;
+    const MmfPlan L = plan_mmf(ctx, m, n, k);
+    return grow_scratch(ctx, *S, &S->mmf, &S->mmf_bytes, L.need, stream, "reserve_matmul");
+}
+
+int gllmq_reserve_ffn(gllmq_ctx *ctx, uint32_t dtype_gate_up, uint32_t dtype_down, size_t m, size_t hidden, size_t ffn,
+                      void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    int rc = gllmq_reserve_matmul(ctx, dtype_gate_up, m, 2 * ffn, hidden, stream);
+    if (rc == GLLMQ_OK) rc = gllmq_reserve_matmul(ctx, dtype_down, m, hidden, ffn, stream);
+    if (rc != GLLMQ_OK || m == 0 || hidden == 0 || ffn == 0) return rc;
+    Scratch *S = nullptr;
+    rc = acquire_scratch(ctx, stream, &S);
+    if (rc != GLLMQ_OK) return rc;
+    return grow_scratch(ctx, *S, &S->ffn, &S->ffn_bytes, ffn_scratch_bytes(m, ffn), stream, "reserve_ffn");
+}
+
+int gllmq_reserve_moe(gllmq_ctx *ctx, size_t tokens, size_t top_k, size_t hidden, size_t ffn, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    Scratch *S = nullptr;
+    int rc = acquire_scratch(ctx, stream, &S);
+    if (rc != GLLMQ_OK || tokens == 0 || top_k == 0) return rc;
+    return grow_scratch(ctx, *S, &S->moe, &S->moe_bytes, moe_workspace(tokens * top_k, hidden, ffn).total, stream,
+                        "reserve_moe");
 }
 
 int gllmq_dequantize_host(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *out, size_t n_out,
                           uint32_t dtype)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     const Format *f = find_format(dtype);
     if (!f) return gllmq_dequantize(ctx, blocks, n_bytes, out, n_out, dtype, nullptr);
     const size_t nb = std::min(n_bytes / f->block_bytes, n_out / f->block_size);
     if (nb == 0) return GLLMQ_OK;
     void *d_in = nullptr, *d_out = nullptr;
-    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
-    GLLMQ_HIP(ctx, hipMalloc(&d_in, nb * f->block_bytes));
+    int rc = cached_weights(ctx, blocks, nb * f->block_bytes, &d_in);
+    if (rc != GLLMQ_OK) return rc;
     hipError_t e = hipMalloc(&d_out, nb * f->block_size * sizeof(float));
-    int rc = GLLMQ_OK;
     if (e != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "hipMalloc: %s", hipGetErrorString(e));
-    if (rc == GLLMQ_OK && (e = hipMemcpy(d_in, blocks, nb * f->block_bytes, hipMemcpyHostToDevice)) != hipSuccess)
-        rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy H2D: %s", hipGetErrorString(e));
     if (rc == GLLMQ_OK)
         rc = gllmq_dequantize(ctx, d_in, nb * f->block_bytes, static_cast<float *>(d_out), nb * f->block_size,
                               dtype, nullptr);
     if (rc == GLLMQ_OK &&
         (e = hipMemcpy(out, d_out, nb * f->block_size * sizeof(float), hipMemcpyDeviceToHost)) != hipSuccess)
         rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy D2H: %s", hipGetErrorString(e));
-    (void)hipFree(d_in);
     (void)hipFree(d_out);
     return rc;
 }
@@ -1192,6 +1518,7 @@ int gllmq_quant_gather_host(gllmq_ctx *ctx, const void *table, size_t table_byte
                             size_t hidden, const uint32_t *ids, size_t count, float scale, float *out)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     const Format *f = find_format(dtype);
     if (!f || count == 0 || hidden == 0 || !table || !ids || !out || hidden % 4 != 0 ||
         table_bytes < vocab * gllmq_row_bytes(dtype, hidden)) // the device entry point reports these
@@ -1202,19 +1529,17 @@ int gllmq_quant_gather_host(gllmq_ctx *ctx, const void *table, size_t table_byte
                         ids[i], i, vocab);
     const size_t tb = vocab * gllmq_row_bytes(dtype, hidden);
     void *d_t = nullptr, *d_i = nullptr, *d_o = nullptr;
-    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
-    hipError_t e = hipMalloc(&d_t, tb);
-    if (e == hipSuccess) e = hipMalloc(&d_i, count * sizeof(uint32_t));
+    int rc = cached_weights(ctx, table, tb, &d_t);
+    if (rc != GLLMQ_OK) return rc;
+    hipError_t e = hipMalloc(&d_i, count * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMalloc(&d_o, count * hidden * sizeof(float));
-    if (e == hipSuccess) e = hipMemcpy(d_t, table, tb, hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemcpy(d_i, ids, count * sizeof(uint32_t), hipMemcpyHostToDevice);
-    int rc = e == hipSuccess ? GLLMQ_OK : fail(ctx, GLLMQ_ERR_HIP, "quant_gather: %s", hipGetErrorString(e));
+    rc = e == hipSuccess ? GLLMQ_OK : fail(ctx, GLLMQ_ERR_HIP, "quant_gather: %s", hipGetErrorString(e));
     if (rc == GLLMQ_OK)
         rc = gllmq_quant_gather(ctx, d_t, tb, dtype, vocab, hidden, static_cast<const uint32_t *>(d_i), count, scale,
                                 static_cast<float *>(d_o), nullptr);
     if (rc == GLLMQ_OK && (e = hipMemcpy(out, d_o, count * hidden * sizeof(float), hipMemcpyDeviceToHost)) != hipSuccess)
         rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy D2H: %s", hipGetErrorString(e));
-    (void)hipFree(d_t);
     (void)hipFree(d_i);
     (void)hipFree(d_o);
     return rc;
@@ -1224,28 +1549,27 @@ int gllmq_quantized_matmul_host(gllmq_ctx *ctx, const void *w, size_t w_bytes, c
                                 uint32_t dtype, size_t m, size_t n, size_t k)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     const Format *f = find_format(dtype);
     if (!f) return gllmq_quantized_matmul(ctx, w, w_bytes, x, y, dtype, m, n, k, nullptr);
     if (m == 0 || n == 0) return GLLMQ_OK;
+    if (!w || !x || !y) return fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul: NULL pointer");
     const size_t need = n * gllmq_row_bytes(dtype, k);
     if (w_bytes < need)
         return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quantized_matmul: weight buffer has %zu bytes, need %zu", w_bytes, need);
     void *d_w = nullptr, *d_x = nullptr, *d_y = nullptr;
-    GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
-    int rc = GLLMQ_OK;
+    int rc = cached_weights(ctx, w, need, &d_w);
+    if (rc != GLLMQ_OK) return rc;
     hipError_t e;
-    if ((e = hipMalloc(&d_w, need)) != hipSuccess || (e = hipMalloc(&d_x, m * k * sizeof(float))) != hipSuccess ||
-        (e = hipMalloc(&d_y, m * n * sizeof(float))) != hipSuccess)
+    if ((e = hipMalloc(&d_x, m * k * sizeof(float))) != hipSuccess || (e = hipMalloc(&d_y, m * n * sizeof(float))) != hipSuccess)
         rc = fail(ctx, GLLMQ_ERR_HIP, "hipMalloc: %s", hipGetErrorString(e));
-    if (rc == GLLMQ_OK && ((e = hipMemcpy(d_w, w, need, hipMemcpyHostToDevice)) != hipSuccess ||
-                           (e = hipMemcpy(d_x, x, m * k * sizeof(float), hipMemcpyHostToDevice)) != hipSuccess))
+    if (rc == GLLMQ_OK && (e = hipMemcpy(d_x, x, m * k * sizeof(float), hipMemcpyHostToDevice)) != hipSuccess)
         rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy H2D: %s", hipGetErrorString(e));
     if (rc == GLLMQ_OK)
         rc = gllmq_quantized_matmul(ctx, d_w, need, static_cast<const float *>(d_x), static_cast<float *>(d_y),
                                     dtype, m, n, k, nullptr);
     if (rc == GLLMQ_OK && (e = hipMemcpy(y, d_y, m * n * sizeof(float), hipMemcpyDeviceToHost)) != hipSuccess)
         rc = fail(ctx, GLLMQ_ERR_HIP, "hipMemcpy D2H: %s", hipGetErrorString(e));
-    (void)hipFree(d_w);
     (void)hipFree(d_x);
     (void)hipFree(d_y);
     return rc;

@@ -19,4 +19,4 @@
 #include "moe.hip.inc"
 #include "argmax.hip.inc"
 #include "ffn.hip.inc"
-#include "probe.hip.inc"
+#include "route.hip.inc"

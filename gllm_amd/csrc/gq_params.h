@@ -254,11 +254,32 @@ struct MoeMm8Params {
     const MoeJob8 *jobs;
     const uint32_t *counters;
     uint64_t expert_stride;  // bytes between experts in g.w
+    const uint8_t *up;       // gated form: the up rows of expert 0 (g.w then holds the gate rows)
+    uint64_t up_stride;      // bytes between experts in `up`
     uint32_t slices;         // workgroups that share one job's tiles
     uint32_t y_stride;       // elements between output rows (by sorted position)
     const uint32_t *rows;    // null: the activation rows are the job's tokens; else this table (0, 1, ...)
                              // counts from the job's first sorted position
 };
+
+// Router (route.hip.inc): gate logits -> route table.
+struct MoeRouteParams {
+    const float *logits;     // [tokens][experts]
+    uint32_t *route_expert;  // [tokens][top_k]
+    float *route_weight;     // [tokens][top_k]
+    uint32_t *route_len;     // [tokens]
+    uint32_t *route_pos;     // [tokens][top_k] or null: the token's place in its expert's list
+    uint32_t *expert_counts; // [experts] or null
+    uint32_t *overflow;      // [1] or null: choices dropped because their expert was full
+    uint32_t tokens, experts, top_k;
+    uint32_t capacity;       // tokens an expert takes
+    uint32_t phases;         // bit 0: softmax and top-k, bit 1: capacity filter (one workgroup)
+};
+
+constexpr int ROUTE_WAVES = 8;
+constexpr int ROUTE_THREADS = 64 * ROUTE_WAVES;
+constexpr uint32_t ROUTE_MAX_EXPERTS = 4096, ROUTE_MAX_TOP_K = 64;
+constexpr uint32_t ROUTE_FUSED_MAX_TOKENS = 64; // up to here both phases are one launch
 
 struct MoeActParams {
     const float *gu; // [pairs][2 * ffn]

@@ -6,6 +6,17 @@
  * The context's device must be the calling thread's current HIP device, and `stream` a
  * stream of that device.
  *
+ * Threads and streams (Backend is Send + Sync, src/compat/mod.rs:77; the reference guards its
+ * caches with a Mutex, src/compat/hip_backend.rs:22-30).  A context may be used from several
+ * threads and on several streams at once: enqueues take turns on one lock, and device memory that
+ * kernels use beyond their inputs and outputs ("scratch": partial sums, prepared activations,
+ * intermediates) is kept per stream, so calls on different streams never share it and calls on
+ * one stream are ordered by the stream.  Scratch is allocated the first time a stream needs it and
+ * grows on demand; growing waits for that stream's earlier work.  Neither is possible while the
+ * stream is being captured into a graph: call gllmq_reserve_* (or run the shape once) on the
+ * stream before capturing, else the call returns GLLMQ_ERR_INVALID.  After that every device
+ * entry point only enqueues kernels.
+ *
  * Reference interfaces each entry point stands in for (paths inside putao520/gllm):
  *   Backend::quantized_matmul  src/compat/mod.rs:233-246, CPU impl src/compat/cpu_backend.rs:991-1049
  *   Backend::dequantize        src/compat/mod.rs:248-256, CPU impl src/compat/cpu_backend.rs:1051-1159
@@ -64,10 +75,35 @@ typedef struct gllmq_ctx gllmq_ctx;
  * (the reference reloads its module per launch, src/compat/hip_backend.rs:211-238). */
 int gllmq_init(gllmq_ctx **out_ctx, int device);
 void gllmq_destroy(gllmq_ctx *ctx);
-/* Message of the last failing call on this context ("" if none); valid until the next call. */
+/* Message of the last failing call on this context ("" if none), copied for the calling thread:
+ * valid until this thread's next gllmq_last_error. */
 const char *gllmq_last_error(const gllmq_ctx *ctx);
 const char *gllmq_status_string(int status);
 const char *gllmq_version(void);
+
+/* Kernel-family choices of a context; no counterpart in the reference.  The defaults are the
+ * measured best and nothing needs setting; the test-suite uses this to reach every kernel family
+ * through the public entry points.  Names: "gemv_f32" (1: f32 multiply-add GEMV instead of the
+ * integer-dot one), "mm8" / "mmf" (0: no int8 / f16 matrix-core kernels), "ffn_fused" (0: the
+ * feed-forward block in three steps), "mm8_q5k_min_m" / "mm8_q6k_min_m" / "mm8_q8_0_min_m"
+ * (fewest rows that take the int8 matrix-core kernel; 0 = never), "mmf_small_min_m" (fewest rows
+ * of long rows that take the GEMM; 0 = never), "mm8_ksplit" (most K slices; 0 = never split),
+ * "moe_mm8" / "moe_mm8_q6k" / "moe_mm8_rows" / "moe_glu" (0: expert rows off the matrix cores /
+ * Q6_K ones / no wave-per-tile kernel / activation as its own launch), "weights_cache_mib" (bytes
+ * of uploaded weights the host-slice calls keep, in MiB).  Unknown names return
+ * GLLMQ_ERR_INVALID.  Not to be changed while calls are in flight on other threads. */
+int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value);
+/* Name of the kernel the context launched last ("" before the first launch): lets a profile be
+ * matched to a call.  No counterpart in the reference. */
+const char *gllmq_last_kernel_name(const gllmq_ctx *ctx);
+
+/* Sizes the stream's scratch for a later call of that shape, so that the call itself allocates
+ * nothing (needed before a stream capture).  No counterpart in the reference, whose scratch is
+ * sized when the graph is compiled (src/compat/gpu_backend_macro.rs:82-87). */
+int gllmq_reserve_matmul(gllmq_ctx *ctx, uint32_t ggml_dtype, size_t m, size_t n, size_t k, void *stream);
+int gllmq_reserve_ffn(gllmq_ctx *ctx, uint32_t dtype_gate_up, uint32_t dtype_down, size_t m, size_t hidden,
+                      size_t ffn, void *stream);
+int gllmq_reserve_moe(gllmq_ctx *ctx, size_t tokens, size_t top_k, size_t hidden, size_t ffn, void *stream);
 
 /* ---- format constants (GgmlDType::block_size / block_bytes / tensor_nbytes row rule) */
 size_t gllmq_block_size(uint32_t ggml_dtype);  /* 0 if unsupported */
@@ -108,8 +144,7 @@ int gllmq_quant_gather(gllmq_ctx *ctx, const void *table_dev, size_t table_bytes
  * with the activation in its epilogue (a workgroup runs the gate tile and the up tile of a
  * row range back to back); other shapes run the two products (one matmul when the up rows
  * follow the gate rows in memory), an activation kernel and the down projection, each with
- * the kernels gllmq_quantized_matmul would pick.  Intermediates live in the context: calls on
- * one context must not overlap in time. */
+ * the kernels gllmq_quantized_matmul would pick.  Intermediates live in the stream's scratch. */
 int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_dev, const void *up_dev, size_t gate_up_bytes_each,
                      uint32_t dtype_gate_up, const void *down_dev, size_t down_bytes, uint32_t dtype_down,
                      const float *x_dev, float *out_dev, size_t m, size_t hidden, size_t ffn, int relu_gate,
@@ -121,8 +156,8 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_dev, const void *up_dev, s
  * token_dev[r] = index of the largest entry of row r that is not NaN; of equal maxima the
  * LAST one wins; GLLMQ_ARGMAX_NONE when the row is empty or all NaN (the reference's None).
  * logits_dev is [rows][ld] f32 with n <= ld entries used per row; value_dev (may be NULL)
- * receives the winning logit (NaN for no token).  Scratch between the two launches lives
- * in the context: calls on one context must not overlap in time. */
+ * receives the winning logit (NaN for no token).  The keys between the two launches live in the
+ * stream's scratch. */
 #define GLLMQ_ARGMAX_NONE 0xFFFFFFFFu
 int gllmq_argmax(gllmq_ctx *ctx, const float *logits_dev, size_t rows, size_t n, size_t ld,
                  uint32_t *token_dev, float *value_dev, void *stream);
@@ -137,9 +172,8 @@ int gllmq_argmax(gllmq_ctx *ctx, const float *logits_dev, size_t rows, size_t n,
  * per 32-element block, its f16 scale applied in f32).  More than 8 rows run a GEMM on the
  * f16 matrix cores, 64 rows per pass: weights as the exact integers sc*q in f16 (Q6_K: q-32,
  * Q8_0: q, their scales applied per 16 or 32 elements in f32), activations as two f16 terms
- * (22 significant bits) of a per-block scaled value, f32 accumulation; its scratch
- * (activation images, partial sums of the K split) lives in the context, so such calls on
- * one context must not overlap in time.  The GEMM also takes 3..8 rows when the rows are so
+ * (22 significant bits) of a per-block scaled value, f32 accumulation; its activation images
+ * and the partial sums of its K split live in the stream's scratch.  The GEMM also takes 3..8 rows when the rows are so
  * long that the prepared activations do not fit the LDS of one 8-row pass (K above about
  * 4096..12288, by format and rows).  Q5_K with one row, Q6_K and Q8_0 with one or two, and
  * Q8_0 rows shorter than 256 elements run integer-dot GEMV kernels, two activation rows per
@@ -147,8 +181,7 @@ int gllmq_argmax(gllmq_ctx *ctx, const float *logits_dev, size_t rows, size_t n,
  * matrix-core kernel.  With so few weight rows that their 32-row tiles cover at most half of
  * the CUs, the matrix-core kernels of up to 8 rows split K across the workgroups of one launch
  * (the last workgroup of a tile adds the slice sums in slice order); slice sums and arrival
- * counters live in the context too.  Which scratch a call uses depends on its shape: calls on
- * one context must not overlap in time. */
+ * counters live in the stream's scratch too. */
 int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev,
                            float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,
                            void *stream);
@@ -173,27 +206,55 @@ typedef struct gllmq_matmul_desc {
 int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs, size_t count,
                                  void *stream);
 
+/* ---- MoE router: gate logits -> route table ------------------------------------------
+ * Replaces the graph ops MoEGate + TopK (src/arch/auto_graph_fragments/build_graph.inc.rs:2064-2071)
+ * and their host mirror ExpertRouteTable::from_gate_logits (src/moe/routing.rs:100-160) over
+ * topk_with_weights / softmax (src/moe/routing.rs:263-302).  Per token: p = softmax(logits) (sum
+ * in expert order; all p = 1/experts when the sum is not positive), the min(top_k, experts)
+ * largest p in descending order with the lower index first among equals (a stable sort),
+ * weights divided by their sum.  Then, tokens in order, a choice is kept while its expert holds
+ * fewer than capacity = ceil(capacity_factor * tokens / experts) tokens (f32 arithmetic, clamped
+ * to [0, 1e9], src/moe/routing.rs:53-61; the reference's default factor is 1.25, :40-49); a
+ * token whose choices are all full goes to the least loaded expert (the first of equals) with
+ * weight 1.0.  logits_dev is [tokens x experts] f32; the outputs are the [tokens x top_k] /
+ * [tokens] arrays gllmq_moe_matvec takes (entries past route_len[t] are written as 0);
+ * route_pos_dev (the token's position in its expert's list), expert_counts_dev [experts] and
+ * overflow_dev [1] (choices dropped) may be NULL.  exp() is the device's: a weight may differ
+ * from a libm-based host by an ulp or two, and two experts whose probabilities collide within
+ * that may swap places.
+ * Limits of this build: experts <= 4096, top_k <= 64.  Up to 64 tokens this is one launch. */
+int gllmq_moe_route(gllmq_ctx *ctx, const float *logits_dev, size_t tokens, size_t experts, size_t top_k,
+                    float capacity_factor, uint32_t *route_expert_dev, float *route_weight_dev,
+                    uint32_t *route_len_dev, uint32_t *route_pos_dev, uint32_t *expert_counts_dev,
+                    uint32_t *overflow_dev, void *stream);
+
 /* ---- MoE expert matvec (ExpertRouteTable grouping, src/moe/routing.rs:163-173) -----
  * out[t] = sum_i weight[t][i] * down_e( silu(gate_e x_t) * (up_e x_t) ), e = expert[t][i],
  * summed in route order i = 0 .. route_len[t]-1 (src/moe/routing.rs:307-327); a token with
  * no route gets zeros.  Only routed (token, expert) pairs are computed (the reference graph
- * runs every expert on every token and masks, build_graph.inc.rs:2076-2123).  Q4_K gate/up
- * rows of at most 4096 elements run on the int8 matrix cores, all tokens of an expert (eight
- * per pass) against one read of its weights; other formats and the down rows run the
- * integer-dot GEMV, two tokens per pass.
- * gate_up_dev: per expert 2*ffn rows over `hidden` (gate rows, then up rows);
- * down_dev: per expert `hidden` rows over `ffn`.  route_* are [tokens x top_k] device
- * arrays, route_len[t] entries valid per token; entries past route_len[t] are ignored and
- * an expert index >= experts routes nowhere (device data is not validated on the host).
- * relu_gate != 0 applies max(g,0) before silu.
+ * runs every expert on every token and masks, build_graph.inc.rs:2076-2123).  Q4_K, Q5_K and
+ * Q6_K rows of at most 4096 elements run on the int8 matrix cores, all tokens of an expert
+ * (eight per pass) against one read of its weights, Q4_K / Q5_K gate and up with the activation
+ * in the same launch; other shapes run the integer-dot GEMV, two tokens per pass.
+ * Expert e's gate rows ([ffn x hidden] blocks of dtype_gate_up) start at gate_dev +
+ * e * gate_expert_stride, its up rows at up_dev + e * up_expert_stride, its down rows
+ * ([hidden x ffn] of dtype_down) at down_dev + e * down_expert_stride; *_bytes are the sizes of
+ * the three buffers, and every expert's matrix must lie inside its buffer.  This covers both
+ * layouts in use: the reference's, one stride over an expert's three matrices (gate, up, down
+ * back to back, build_graph.inc.rs:2080-2125: the three pointers are offsets into one buffer and
+ * the three strides are equal), and GGUF's, one stacked tensor per role (stride = one matrix).
+ * route_* are [tokens x top_k] device arrays, route_len[t] entries valid per token; entries
+ * past route_len[t] are ignored and an expert index >= experts routes nowhere (device data is
+ * not validated on the host).  relu_gate != 0 applies max(g,0) before silu.
  * Limits of this build: tokens*top_k <= 16384, experts <= 4096, hidden and ffn <= 16384
- * and multiples of 4 (else GLLMQ_ERR_UNIMPLEMENTED / BAD_SHAPE).  x_dev 16-byte aligned.
- * Intermediate buffers live in a workspace owned by the context that grows on demand:
- * calls of this function on one context must not overlap in time. */
-int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_up_dev, uint32_t dtype_gate_up,
-                     const void *down_dev, uint32_t dtype_down, const float *x_dev, float *out_dev,
-                     size_t tokens, size_t hidden, size_t ffn, size_t experts, size_t top_k,
-                     const uint32_t *route_expert_dev, const float *route_weight_dev,
+ * and multiples of 4 (else GLLMQ_ERR_UNIMPLEMENTED / BAD_SHAPE).  x_dev 16-byte aligned;
+ * weights and strides aligned as for gllmq_quantized_matmul.
+ * Intermediate buffers live in the stream's scratch. */
+int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_dev, size_t gate_bytes, size_t gate_expert_stride,
+                     const void *up_dev, size_t up_bytes, size_t up_expert_stride, uint32_t dtype_gate_up,
+                     const void *down_dev, size_t down_bytes, size_t down_expert_stride, uint32_t dtype_down,
+                     const float *x_dev, float *out_dev, size_t tokens, size_t hidden, size_t ffn, size_t experts,
+                     size_t top_k, const uint32_t *route_expert_dev, const float *route_weight_dev,
                      const uint32_t *route_len_dev, int relu_gate, void *stream);
 
 /* ---- GGUF reader and tensor upload ---------------------------------------------------
@@ -259,13 +320,15 @@ const char *gllmq_gguf_meta_array_str(const gllmq_gguf *g, const char *key, uint
 int gllmq_gguf_upload(gllmq_ctx *ctx, const gllmq_gguf *g, size_t index, void *dst_dev, size_t dst_bytes,
                       void *stream);
 
-/* ---- calibration ------------------------------------------------------------------
- * No counterpart in the reference.  Reads `n_bytes` (multiple of 16, 16-byte aligned) of
- * device memory once with a pure streaming kernel; timing it gives the read bandwidth a
- * bandwidth-bound kernel can reach on this device.  `sink_dev` points at 4 writable bytes. */
-int gllmq_stream_read(gllmq_ctx *ctx, const void *buf_dev, size_t n_bytes, void *sink_dev, void *stream);
-
-/* ---- host-pointer convenience (upload, run, download, synchronise) ---------------- */
+/* ---- host-slice forms: the literal signatures of the trait (upload, run, download, synchronise)
+ * The weight slice (blocks / table / w) is uploaded the first time it is seen and kept on the
+ * device, keyed by its address and length, as the reference keeps its uploaded weight blob
+ * (src/compat/hip_backend.rs:141-156): later calls with the same slice copy only activations and
+ * results.  Weights behind a cached slice must not change; gllmq_weights_forget(ctx, ptr) drops
+ * one slice (NULL: all) before its memory is reused.  gllmq_weight_uploads counts the
+ * host-to-device weight copies a context has made. */
+void gllmq_weights_forget(gllmq_ctx *ctx, const void *host_ptr);
+uint64_t gllmq_weight_uploads(const gllmq_ctx *ctx);
 int gllmq_dequantize_host(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *out,
                           size_t n_out, uint32_t ggml_dtype);
 int gllmq_quant_gather_host(gllmq_ctx *ctx, const void *table, size_t table_bytes, uint32_t ggml_dtype,

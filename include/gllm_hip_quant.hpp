@@ -155,15 +155,37 @@ public:
         return make(gllmq_argmax(ctx_, logits_dev, rows, n, ld, token_dev, value_dev, stream), "argmax");
     }
 
+    // ExpertRouteTable::from_gate_logits over device buffers (src/moe/routing.rs:100-160; graph ops
+    // MoEGate + TopK, build_graph.inc.rs:2064-2071); the optional outputs may be null.
+    BackendError moe_route_device(const float *logits_dev, size_t tokens, size_t experts, size_t top_k,
+                                  float capacity_factor, uint32_t *route_expert_dev, float *route_weight_dev,
+                                  uint32_t *route_len_dev, uint32_t *route_pos_dev = nullptr,
+                                  uint32_t *expert_counts_dev = nullptr, uint32_t *overflow_dev = nullptr,
+                                  void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_moe_route(ctx_, logits_dev, tokens, experts, top_k, capacity_factor, route_expert_dev,
+                                    route_weight_dev, route_len_dev, route_pos_dev, expert_counts_dev, overflow_dev, stream),
+                    "moe_route");
+    }
+
+    // One role of the expert weights: expert e's matrix starts at dev + e * expert_stride.
+    struct ExpertWeights {
+        const void *dev;
+        size_t bytes;         // size of the buffer behind dev
+        size_t expert_stride; // bytes between experts
+    };
+
     // Expert FFN over a route table (ExpertRouteTable, src/moe/routing.rs:100-173).
-    BackendError moe_matvec_device(const void *gate_up_dev, QuantType t_gate_up, const void *down_dev, QuantType t_down,
-                                   const float *x_dev, float *out_dev, size_t tokens, size_t hidden, size_t ffn,
-                                   size_t experts, size_t top_k, const uint32_t *route_expert_dev,
+    BackendError moe_matvec_device(ExpertWeights gate, ExpertWeights up, QuantType t_gate_up, ExpertWeights down,
+                                   QuantType t_down, const float *x_dev, float *out_dev, size_t tokens, size_t hidden,
+                                   size_t ffn, size_t experts, size_t top_k, const uint32_t *route_expert_dev,
                                    const float *route_weight_dev, const uint32_t *route_len_dev, bool relu_gate = false,
                                    void *stream = nullptr) const
     {
         if (!ctx_) return init_error_;
-        return make(gllmq_moe_matvec(ctx_, gate_up_dev, static_cast<uint32_t>(t_gate_up), down_dev,
+        return make(gllmq_moe_matvec(ctx_, gate.dev, gate.bytes, gate.expert_stride, up.dev, up.bytes, up.expert_stride,
+                                     static_cast<uint32_t>(t_gate_up), down.dev, down.bytes, down.expert_stride,
                                      static_cast<uint32_t>(t_down), x_dev, out_dev, tokens, hidden, ffn, experts, top_k,
                                      route_expert_dev, route_weight_dev, route_len_dev, relu_gate ? 1 : 0, stream),
                     "moe_matvec");

@@ -594,6 +594,7 @@ size_t gq_route(const float *logits, size_t tokens, size_t experts, size_t top_k
                 uint32_t *route_pos, uint32_t *route_len, uint32_t *expert_counts)
 {
     const size_t cap = gq_expert_capacity(capacity_factor, tokens, experts);
+    const size_t stride = top_k ? top_k : 1; /* row length of the route arrays: a token always gets one slot */
     size_t overflow = 0;
     uint32_t *idx = (uint32_t *)malloc((top_k ? top_k : 1) * sizeof(uint32_t));
     float *w = (float *)malloc((top_k ? top_k : 1) * sizeof(float));
@@ -604,22 +605,22 @@ size_t gq_route(const float *logits, size_t tokens, size_t experts, size_t top_k
         for (size_t i = 0; i < kk; ++i) {
             const uint32_t e = idx[i];
             if (expert_counts[e] < cap) {
-                route_expert[t * top_k + len] = e;
-                route_weight[t * top_k + len] = w[i];
-                route_pos[t * top_k + len] = expert_counts[e];
+                route_expert[t * stride + len] = e;
+                route_weight[t * stride + len] = w[i];
+                route_pos[t * stride + len] = expert_counts[e];
                 ++expert_counts[e];
                 ++len;
             } else {
                 ++overflow;
             }
         }
-        if (len == 0 && experts > 0 && top_k > 0) { /* every choice full: least-loaded expert, weight 1 */
+        if (len == 0 && experts > 0) { /* no choice kept (all full, or top_k = 0): least-loaded expert, weight 1 */
             size_t best = 0;
             for (size_t e = 1; e < experts; ++e)
                 if (expert_counts[e] < expert_counts[best]) best = e;
-            route_expert[t * top_k] = (uint32_t)best;
-            route_weight[t * top_k] = 1.0f;
-            route_pos[t * top_k] = expert_counts[best];
+            route_expert[t * stride] = (uint32_t)best;
+            route_weight[t * stride] = 1.0f;
+            route_pos[t * stride] = expert_counts[best];
             ++expert_counts[best];
             len = 1;
         }

@@ -139,7 +139,8 @@ size_t gq_topk_indices(const float *logits, size_t n, size_t k, uint32_t *idx);
 /* src/moe/routing.rs:53-61 */
 size_t gq_expert_capacity(float capacity_factor, size_t total_tokens, size_t num_experts);
 /* ExpertRouteTable::from_gate_logits, src/moe/routing.rs:100-160.
- * logits [tokens x experts]; outputs are [tokens x top_k], route_len[t] entries valid.
+ * logits [tokens x experts]; outputs are [tokens x max(top_k, 1)], route_len[t] entries valid
+ * (with top_k = 0 every token still gets the least-loaded fallback, as in the reference).
  * Returns overflow_count. expert_counts [experts]. */
 size_t gq_route(const float *logits, size_t tokens, size_t experts, size_t top_k,
                 float capacity_factor, uint32_t *route_expert, float *route_weight,

@@ -54,11 +54,27 @@ extern "C" {
                                      act_mode: c_int, stream: *mut c_void) -> c_int;
     pub fn gllmq_quantized_matmul_batch(ctx: *mut gllmq_ctx, descs: *const gllmq_matmul_desc, count: usize,
                                         stream: *mut c_void) -> c_int;
-    pub fn gllmq_moe_matvec(ctx: *mut gllmq_ctx, gate_up_dev: *const c_void, dtype_gate_up: u32,
-                            down_dev: *const c_void, dtype_down: u32, x_dev: *const f32, out_dev: *mut f32,
+    pub fn gllmq_moe_route(ctx: *mut gllmq_ctx, logits_dev: *const f32, tokens: usize, experts: usize, top_k: usize,
+                           capacity_factor: f32, route_expert_dev: *mut u32, route_weight_dev: *mut f32,
+                           route_len_dev: *mut u32, route_pos_dev: *mut u32, expert_counts_dev: *mut u32,
+                           overflow_dev: *mut u32, stream: *mut c_void) -> c_int;
+    pub fn gllmq_moe_matvec(ctx: *mut gllmq_ctx, gate_dev: *const c_void, gate_bytes: usize, gate_expert_stride: usize,
+                            up_dev: *const c_void, up_bytes: usize, up_expert_stride: usize, dtype_gate_up: u32,
+                            down_dev: *const c_void, down_bytes: usize, down_expert_stride: usize, dtype_down: u32,
+                            x_dev: *const f32, out_dev: *mut f32,
                             tokens: usize, hidden: usize, ffn: usize, experts: usize, top_k: usize,
                             route_expert_dev: *const u32, route_weight_dev: *const f32,
                             route_len_dev: *const u32, relu_gate: c_int, stream: *mut c_void) -> c_int;
+    pub fn gllmq_set_option(ctx: *mut gllmq_ctx, name: *const c_char, value: std::os::raw::c_long) -> c_int;
+    pub fn gllmq_last_kernel_name(ctx: *const gllmq_ctx) -> *const c_char;
+    pub fn gllmq_reserve_matmul(ctx: *mut gllmq_ctx, ggml_dtype: u32, m: usize, n: usize, k: usize,
+                                stream: *mut c_void) -> c_int;
+    pub fn gllmq_reserve_ffn(ctx: *mut gllmq_ctx, dtype_gate_up: u32, dtype_down: u32, m: usize, hidden: usize,
+                             ffn: usize, stream: *mut c_void) -> c_int;
+    pub fn gllmq_reserve_moe(ctx: *mut gllmq_ctx, tokens: usize, top_k: usize, hidden: usize, ffn: usize,
+                             stream: *mut c_void) -> c_int;
+    pub fn gllmq_weights_forget(ctx: *mut gllmq_ctx, host_ptr: *const c_void);
+    pub fn gllmq_weight_uploads(ctx: *const gllmq_ctx) -> u64;
     pub fn gllmq_ffn_swiglu(ctx: *mut gllmq_ctx, gate_dev: *const c_void, up_dev: *const c_void,
                             gate_up_bytes_each: usize, dtype_gate_up: u32, down_dev: *const c_void, down_bytes: usize,
                             dtype_down: u32, x_dev: *const f32, out_dev: *mut f32, m: usize, hidden: usize,
@@ -86,8 +102,10 @@ extern "C" {
 }
 
 /// Owner of one library context (one per device).  `Send + Sync` like the trait demands
-/// (src/compat/mod.rs:77): the library keeps no mutable state per call except the MoE
-/// workspace, which it guards itself.
+/// (src/compat/mod.rs:77): every entry point takes the context's lock for the time it enqueues,
+/// the device memory kernels use beyond inputs and outputs is kept per stream (calls on different
+/// streams never share it, calls on one stream are ordered by the stream), the host-slice forms
+/// synchronise before they return, and `gllmq_last_error` hands each thread its own copy.
 pub struct HipQuant {
     ctx: *mut gllmq_ctx,
 }

@@ -97,11 +97,10 @@ def test_ffn_layer_shape(hip, torch, oracle):
         check(got, want, f"layer shape m={m}")
 
 
-def test_ffn_three_step_form(torch, oracle, monkeypatch):
-    """GLLMQ_FFN_FUSED=0: the two products, the activation kernel, the down projection."""
+def test_ffn_three_step_form(torch, oracle):
+    """Option ffn_fused = 0: the two products, the activation kernel, the down projection."""
     from gllm_amd.backend import HipBackend
-    monkeypatch.setenv("GLLMQ_FFN_FUSED", "0")
-    hip2 = HipBackend(0)
+    hip2 = HipBackend(0, options={"ffn_fused": 0})
     hidden, ffn = 1024, 800
     gate, up = random_weight(Q4_K, ffn, hidden, seed=1), random_weight(Q4_K, ffn, hidden, seed=2)
     down = random_weight(Q6_K, hidden, ffn, seed=3)

@@ -1,6 +1,9 @@
-"""GPU parity of the MoE expert matvec (through the C ABI) against the oracle's
-route-by-route evaluation, which is the dense "run the expert, weight, add" rule of
-src/moe/routing.rs:307-327 restricted to the routed pairs.
+"""GPU parity of the MoE path (through the C ABI): gate logits go to the library's router
+(gllmq_moe_route), its route table goes to the expert matvec (gllmq_moe_matvec); the oracle
+routes the same logits on the CPU and evaluates route by route, which is the dense "run the
+expert, weight, add" rule of src/moe/routing.rs:307-327 restricted to the routed pairs.  The
+oracle only checks: the route tables must agree (experts and lengths exactly, weights to a few
+ulp) and the outputs must meet the bar.
 
 Bar: rel-L2 <= 1e-4 and per-element |err| <= 1e-3 * max|out| against float64 accumulation.
 """
@@ -43,7 +46,27 @@ def expert_weights(dt_gu, dt_dn, experts, hidden, ffn, seed):
     return gu, dn
 
 
-def run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, re, rw, rl, relu_gate=False):
+def route_gpu(hip, torch, oracle, logits, top_k, capacity_factor=1.25):
+    """Routes `logits` with the library's router, checks the table against the oracle's and
+    returns (device table, oracle table)."""
+    tokens, experts = logits.shape
+    lg = torch.from_numpy(np.ascontiguousarray(logits, np.float32)).cuda()
+    red = torch.full((tokens, top_k), -1, dtype=torch.int32, device="cuda")
+    rwd = torch.full((tokens, top_k), float("nan"), dtype=torch.float32, device="cuda")
+    rld = torch.full((tokens,), -1, dtype=torch.int32, device="cuda")
+    hip.moe_route(lg, top_k, red, rwd, rld, capacity_factor=capacity_factor)
+    torch.cuda.synchronize()
+    r = oracle.route(logits, top_k, capacity_factor=capacity_factor)
+    got_e, got_w, got_l = red.cpu().numpy().view(np.uint32), rwd.cpu().numpy(), rld.cpu().numpy().view(np.uint32)
+    assert np.array_equal(got_l, r["len"]), "route lengths differ from the oracle's"
+    assert np.array_equal(got_e, r["expert"]), "routed experts differ from the oracle's"
+    np.testing.assert_allclose(got_w, r["weight"], rtol=4 * top_k * 2.0 ** -24, atol=0)
+    return (red, rwd, rld), r
+
+
+def run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, re, rw, rl, relu_gate=False, split=False):
+    """re, rw, rl: the route table as numpy arrays or as device tensors.  split: gate rows and up
+    rows as a tensor each ([experts, ffn, hidden]: GGUF's layout) instead of one stacked tensor."""
     tokens = x.shape[0]
     # poison behind every input: a read past the end turns the result into NaN
     def guarded(host, fill):
@@ -54,10 +77,19 @@ def run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, re, rw, r
     gud, dnd = guarded(np.asarray(gu).view(np.uint8), 0xFF), guarded(np.asarray(dn).view(np.uint8), 0xFF)
     xd = guarded(np.ascontiguousarray(x, np.float32), float("nan")).view(tokens, -1)
     out = torch.full((tokens, hidden), float("nan"), dtype=torch.float32, device="cuda")
-    red = torch.from_numpy(np.ascontiguousarray(re, np.uint32).view(np.int32)).cuda()
-    rwd = torch.from_numpy(np.ascontiguousarray(rw, np.float32)).cuda()
-    rld = torch.from_numpy(np.ascontiguousarray(rl, np.uint32).view(np.int32)).cuda()
-    hip.moe_matvec(gud, dt_gu, dnd, dt_dn, xd, out, hidden, ffn, experts, red, rwd, rld, relu_gate=relu_gate)
+    if isinstance(re, np.ndarray):
+        red = torch.from_numpy(np.ascontiguousarray(re, np.uint32).view(np.int32)).cuda()
+        rwd = torch.from_numpy(np.ascontiguousarray(rw, np.float32)).cuda()
+        rld = torch.from_numpy(np.ascontiguousarray(rl, np.uint32).view(np.int32)).cuda()
+    else:
+        red, rwd, rld = re, rw, rl
+    if split:
+        each = ffn * row_bytes(dt_gu, hidden)
+        both = np.asarray(gu).view(np.uint8).reshape(experts, 2, each)
+        gate_d, up_d = guarded(both[:, 0], 0xFF), guarded(both[:, 1], 0xFF)
+        hip.moe_matvec(gate_d, dt_gu, dnd, dt_dn, xd, out, hidden, ffn, experts, red, rwd, rld, relu_gate=relu_gate, up=up_d)
+    else:
+        hip.moe_matvec(gud, dt_gu, dnd, dt_dn, xd, out, hidden, ffn, experts, red, rwd, rld, relu_gate=relu_gate)
     torch.cuda.synchronize()
     return out.cpu().numpy()
 
@@ -68,10 +100,12 @@ def test_moe_small_routed(hip, torch, oracle, dt_gu, dt_dn):
     experts, tokens, top_k, hidden, ffn = 8, 7, 2, 512, 256
     gu, dn = expert_weights(dt_gu, dt_dn, experts, hidden, ffn, seed=40)
     x = random_activations(tokens, hidden, seed=41)
-    r = oracle.route(random_gate_logits(tokens, experts, seed=42), top_k, capacity_factor=float(experts))
+    dev, r = route_gpu(hip, torch, oracle, random_gate_logits(tokens, experts, seed=42), top_k, float(experts))
     want = oracle.moe_ffn(gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
-    got = run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
+    got = run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, *dev)
     check_close(got, want, "moe small")
+    got = run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, *dev, split=True)
+    check_close(got, want, "moe small, gate and up as separate tensors")
 
 
 def test_moe_ragged_routes_repeats_and_empty_tokens(hip, torch, oracle):
@@ -118,7 +152,7 @@ def test_moe_matches_dense_masked_evaluation(hip, torch, oracle):
     experts, tokens, top_k, hidden, ffn = 4, 3, 2, 256, 256
     gu, dn = expert_weights(Q4_K, Q6_K, experts, hidden, ffn, seed=60)
     x = random_activations(tokens, hidden, seed=61)
-    r = oracle.route(random_gate_logits(tokens, experts, seed=62), top_k, capacity_factor=float(experts))
+    dev, r = route_gpu(hip, torch, oracle, random_gate_logits(tokens, experts, seed=62), top_k, float(experts))
     gu_f = oracle.dequantize(gu, Q4_K).reshape(experts, 2 * ffn, hidden).astype(np.float64)
     dn_f = oracle.dequantize(dn, Q6_K).reshape(experts, hidden, ffn).astype(np.float64)
     dense = np.zeros((tokens, hidden))
@@ -130,27 +164,32 @@ def test_moe_matches_dense_masked_evaluation(hip, torch, oracle):
             g = gu_f[e, :ffn] @ x[t].astype(np.float64)
             u = gu_f[e, ffn:] @ x[t].astype(np.float64)
             dense[t] += mask[e] * (dn_f[e] @ (g / (1.0 + np.exp(-g)) * u))
-    got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
+    got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, *dev)
     check_close(got, dense, "moe dense")
 
 
-def test_moe_baseline_shape_reduced_expert_count(hip, torch, oracle):
-    """The baseline MoE shape (16 tokens, top-8, gate/up Q4_K 3072x4096, down Q6_K 4096x1536)
-    over 32 experts instead of 128 so that the oracle finishes in seconds."""
-    print("moe baseline shape", flush=True)
-    experts, tokens, top_k, hidden, ffn = 32, 16, 8, 4096, 1536
+def test_moe_baseline_shape_full_size(hip, torch, oracle):
+    """The baseline MoE configuration at its full size: 128 experts, 16 tokens, top-8, gate/up
+    Q4_K 3072x4096 and down Q6_K 4096x1536 per expert (1.5 GB of expert weights, generated on the
+    host with the seeded generator), gate logits routed by the library.  The oracle evaluates the
+    128 routed pairs (about a fifth of a second per pair and thread)."""
+    print("moe baseline shape, 128 experts", flush=True)
+    experts, tokens, top_k, hidden, ffn = 128, 16, 8, 4096, 1536
     gu, dn = expert_weights(Q4_K, Q6_K, experts, hidden, ffn, seed=70)
     assert gu.size == experts * 2 * ffn * row_bytes(Q4_K, hidden)
     x = random_activations(tokens, hidden, seed=71)
-    r = oracle.route(random_gate_logits(tokens, experts, seed=72), top_k, capacity_factor=float(experts))
+    logits = random_gate_logits(tokens, experts, seed=72)
+    dev, r = route_gpu(hip, torch, oracle, logits, top_k, float(experts))
     assert int(r["len"].sum()) == tokens * top_k
-    want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
-    got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
+    want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=16)
+    got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, *dev)
     check_close(got, want, "moe baseline shape")
-    # default capacity factor 1.25: overflowing routes fall back or drop; same table on both sides
-    r2 = oracle.route(random_gate_logits(tokens, experts, seed=72), top_k)
-    want2 = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r2["expert"], r2["weight"], r2["len"], threads=8)
-    got2 = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r2["expert"], r2["weight"], r2["len"])
+    # the reference's default capacity factor 1.25: capacity 1 at 16 tokens over 128 experts, so
+    # most choices overflow and some tokens fall back to the least loaded expert
+    dev2, r2 = route_gpu(hip, torch, oracle, logits, top_k, 1.25)
+    assert r2["overflow"] > 0 and int(r2["counts"].max()) == 1
+    want2 = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r2["expert"], r2["weight"], r2["len"], threads=16)
+    got2 = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, *dev2)
     check_close(got2, want2, "moe baseline shape, default capacity")
 
 
@@ -163,15 +202,15 @@ def test_moe_more_than_eight_tokens_per_expert(hip, torch, oracle, hidden, ffn):
     experts, tokens, top_k = 4, 40, 2
     gu, dn = expert_weights(Q4_K, Q6_K, experts, hidden, ffn, seed=90)
     x = random_activations(tokens, hidden, seed=91)
-    r = oracle.route(random_gate_logits(tokens, experts, seed=92), top_k, capacity_factor=float(experts))
+    dev, r = route_gpu(hip, torch, oracle, random_gate_logits(tokens, experts, seed=92), top_k, float(experts))
     counts = np.bincount(r["expert"][:, :top_k].reshape(-1), minlength=experts)
     assert counts.max() > 8
     want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
-    got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
+    got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, *dev)
     check_close(got, want, f"moe hidden={hidden} ffn={ffn}")
 
 
-def test_moe_grouped_kernel_alternatives(torch, oracle, monkeypatch):
+def test_moe_grouped_kernel_alternatives(hip, torch, oracle):
     """The grouped kernels the default dispatch does not pick for this shape: Q6_K down rows on
     the tile-split matrix-core kernel and on the integer-dot GEMV, gate/up results through memory
     with the activation as a kernel of its own."""
@@ -179,16 +218,14 @@ def test_moe_grouped_kernel_alternatives(torch, oracle, monkeypatch):
     experts, tokens, top_k, hidden, ffn = 6, 20, 3, 512, 1024
     gu, dn = expert_weights(Q4_K, Q6_K, experts, hidden, ffn, seed=95)
     x = random_activations(tokens, hidden, seed=96)
-    r = oracle.route(random_gate_logits(tokens, experts, seed=97), top_k, capacity_factor=float(experts))
+    dev, r = route_gpu(hip, torch, oracle, random_gate_logits(tokens, experts, seed=97), top_k, float(experts))
     want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
-    for env in ({"GLLMQ_MOE_MM8_ROWS": "0"}, {"GLLMQ_MOE_MM8_Q6K": "0"}, {"GLLMQ_MOE_MM8": "0"}, {"GLLMQ_MOE_GLU": "0"}):
-        print(f"moe alternatives {env}", flush=True)
-        with monkeypatch.context() as mp:
-            for k_, v_ in env.items():
-                mp.setenv(k_, v_)
-            hip2 = HipBackend(0)
-        got = run_gpu(hip2, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
-        check_close(got, want, f"moe {env}")
+    for options in ({"moe_mm8_rows": 0}, {"moe_mm8_q6k": 0}, {"moe_mm8": 0}, {"moe_glu": 0}):
+        hip2 = HipBackend(0, options=options)
+        for split in (False, True):
+            print(f"moe alternatives {options} split={split}", flush=True)
+            got = run_gpu(hip2, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, *dev, split=split)
+            check_close(got, want, f"moe {options} split={split}")
 
 
 def test_moe_random_shapes_sweep(hip, torch, oracle):
@@ -206,9 +243,10 @@ def test_moe_random_shapes_sweep(hip, torch, oracle):
         print(f"moe sweep case {case}: gu={dt_gu} dn={dt_dn} E={experts} k={top_k} T={tokens} H={hidden} F={ffn}", flush=True)
         gu, dn = expert_weights(dt_gu, dt_dn, experts, hidden, ffn, seed=300 + case)
         x = random_activations(tokens, hidden, seed=400 + case)
-        r = oracle.route(random_gate_logits(tokens, experts, seed=500 + case), top_k, capacity_factor=float(experts))
+        factor = float(experts) if case % 3 else 1.25  # a third of the cases with the default capacity: drops and fallbacks
+        dev, r = route_gpu(hip, torch, oracle, random_gate_logits(tokens, experts, seed=500 + case), top_k, factor)
         want = oracle.moe_ffn(gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
-        got = run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
+        got = run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, *dev, split=bool(case & 1))
         check_close(got, want, f"moe sweep case {case}")
 
 
@@ -219,10 +257,10 @@ def test_moe_many_pairs(hip, torch, oracle):
     experts, tokens, top_k, hidden, ffn = 16, 640, 8, 256, 256
     gu, dn = expert_weights(Q4_K, Q6_K, experts, hidden, ffn, seed=80)
     x = random_activations(tokens, hidden, seed=81)
-    r = oracle.route(random_gate_logits(tokens, experts, seed=82), top_k, capacity_factor=float(experts))
+    dev, r = route_gpu(hip, torch, oracle, random_gate_logits(tokens, experts, seed=82), top_k, float(experts))
     assert int(r["len"].sum()) == tokens * top_k > 4096
     want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=16)
-    got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"])
+    got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, *dev)
     check_close(got, want, "moe many pairs")
 
 

@@ -264,20 +264,18 @@ def test_bf16_activation_mode(hip, torch, oracle, dtype, m):
     assert rel > 3e-4, rel
 
 
-@pytest.mark.parametrize("env", [{"GLLMQ_MM8": "0", "GLLMQ_MMF": "0"}, {"GLLMQ_MMF": "0"},
-                                 {"GLLMQ_GEMV_F32": "1", "GLLMQ_MM8": "0", "GLLMQ_MMF": "0"},
-                                 {"GLLMQ_MM8_Q6K_MIN_M": "1", "GLLMQ_MM8_Q5K_MIN_M": "1", "GLLMQ_MM8_Q8_0_MIN_M": "1"},
-                                 {"GLLMQ_MM8_Q6K_MIN_M": "0", "GLLMQ_MM8_Q5K_MIN_M": "0", "GLLMQ_MM8_Q8_0_MIN_M": "0"},
-                                 {"GLLMQ_MMF_SMALL_MIN_M": "0"}, {"GLLMQ_MM8_KSPLIT": "0"},
-                                 {"GLLMQ_MM8_KSPLIT": "2", "GLLMQ_MMF_SMALL_MIN_M": "0"}])
-def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
+@pytest.mark.parametrize("env", [{"mm8": 0, "mmf": 0}, {"mmf": 0},
+                                 {"gemv_f32": 1, "mm8": 0, "mmf": 0},
+                                 {"mm8_q6k_min_m": 1, "mm8_q5k_min_m": 1, "mm8_q8_0_min_m": 1},
+                                 {"mm8_q6k_min_m": 0, "mm8_q5k_min_m": 0, "mm8_q8_0_min_m": 0},
+                                 {"mmf_small_min_m": 0}, {"mm8_ksplit": 0},
+                                 {"mm8_ksplit": 2, "mmf_small_min_m": 0}])
+def test_alternative_kernel_paths(torch, oracle, env):
     """The kernels the default dispatch does not pick: integer-dot GEMV for Q4_K, 8-row passes
     for more than 8 rows, the f32 multiply-add flavour, Q5_K and Q6_K on the matrix cores from one
     row up and on the GEMV kernels throughout (Q8_0 too), no GEMM for few rows; selected per context at init."""
     from gllm_amd.backend import HipBackend
-    for k_, v_ in env.items():
-        monkeypatch.setenv(k_, v_)
-    hip2 = HipBackend(0)
+    hip2 = HipBackend(0, options=env)
     print(f"alternative paths {env}", flush=True)
     for dtype in ALL:
         for m in (1, 2, 5, 11):
@@ -286,7 +284,7 @@ def test_alternative_kernel_paths(torch, oracle, monkeypatch, env):
             want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=4)
             got = gpu_matmul(hip2, torch, w, x, dtype, m, n, k)
             check_close(got, want, f"env={env} dtype={dtype} m={m}")
-    if "GLLMQ_MMF_SMALL_MIN_M" in env:
+    if "mmf_small_min_m" in env:
         # long rows on the 8-row kernels: several passes over the weights, seven blocks per wave and tile
         for dtype in ALL:
             for m in (3, 8):
@@ -317,17 +315,14 @@ def test_random_shapes_sweep(hip, torch, oracle):
         check_close(got, want, f"case {case} dtype={dtype} m={m} n={n} k={k}")
 
 
-def test_k_split_of_the_8_row_kernels(torch, oracle, monkeypatch):
+def test_k_split_of_the_8_row_kernels(torch, oracle):
     """Few weight rows (tiles for at most half of the CUs) and at least two passes per tile: several
     workgroups share a tile, each takes a slice of K, the last one to finish adds the slices up.
     Every format from one row up, 2 to 8 slices, slices of unequal length, a partial last block,
     ragged n, a repeat of every call (the arrival counters must be back at zero; the sum order is
     fixed, so the repeat is bit-identical) with an unsplit call in between."""
     from gllm_amd.backend import HipBackend
-    for k_ in ("GLLMQ_MM8_Q6K_MIN_M", "GLLMQ_MM8_Q5K_MIN_M", "GLLMQ_MM8_Q8_0_MIN_M"):
-        monkeypatch.setenv(k_, "1")
-    monkeypatch.setenv("GLLMQ_MMF_SMALL_MIN_M", "0")
-    hip2 = HipBackend(0)
+    hip2 = HipBackend(0, options={"mm8_q6k_min_m": 1, "mm8_q5k_min_m": 1, "mm8_q8_0_min_m": 1, "mmf_small_min_m": 0})
     cases = [(1, 4096, 4096), (2, 1024, 4096), (1, 100, 14336), (4, 512, 8192), (8, 33, 6144), (3, 2048, 2048 + 1024),
              (5, 64, 16384), (1, 4000, 4096 + 2048), (2, 31, 4096 + 256 * 5 - 8), (8, 4096, 4096), (6, 300, 11008)]
     for dtype in ALL:

@@ -255,3 +255,12 @@ def test_avx2_matmul_matches_the_float64_yardstick(oracle, dtype):
         x[0, col] = 1.0
         y = oracle.quantized_matmul_avx2(w, x, dtype, 1, n, k)
         assert np.array_equal(y[0], deq[:, col])
+
+
+def test_route_with_top_k_zero_still_takes_the_least_loaded_fallback(oracle):
+    # src/moe/routing.rs:131-145: an empty selection (here: nothing asked for) goes to the least
+    # loaded expert with weight 1; three tokens over two experts land on 0, 1, 0
+    r = oracle.route(np.array([[1.0, 5.0]] * 3, np.float32), top_k=0, capacity_factor=2.0)
+    assert r["len"].tolist() == [1, 1, 1]
+    assert r["expert"][:, 0].tolist() == [0, 1, 0] and r["weight"][:, 0].tolist() == [1.0, 1.0, 1.0]
+    assert r["counts"].tolist() == [2, 1] and r["overflow"] == 0
