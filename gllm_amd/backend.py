@@ -89,6 +89,8 @@ def load_library() -> C.CDLL:
     L.gllmq_quantized_matmul.argtypes = [vp, vp, sz, vp, vp, u32, sz, sz, sz, vp]
     L.gllmq_quantized_matmul_ex.restype = C.c_int
     L.gllmq_quantized_matmul_ex.argtypes = [vp, vp, sz, vp, vp, u32, sz, sz, sz, C.c_int, vp]
+    L.gllmq_quantized_matmul_noalloc.restype = C.c_int
+    L.gllmq_quantized_matmul_noalloc.argtypes = [vp, vp, sz, vp, vp, u32, sz, sz, sz, vp]
     L.gllmq_quantized_matmul_batch.restype = C.c_int
     L.gllmq_quantized_matmul_batch.argtypes = [vp, C.POINTER(MatmulDesc), sz, vp]
     L.gllmq_moe_matvec.restype = C.c_int
@@ -130,6 +132,7 @@ EXPORTED_SYMBOLS = [
     "gllmq_init", "gllmq_destroy", "gllmq_last_error", "gllmq_status_string", "gllmq_version",
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
+    "gllmq_quantized_matmul_noalloc",
     "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_quant_gather", "gllmq_moe_route", "gllmq_set_option", "gllmq_last_kernel_name",
     "gllmq_reserve_matmul", "gllmq_reserve_ffn", "gllmq_reserve_moe", "gllmq_weights_forget", "gllmq_weight_uploads",
     "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
@@ -268,6 +271,21 @@ class HipBackend:
                 self._ctx, w.ctypes.data, w.size, x.ctypes.data, output.ctypes.data, dt, m, n, k)
         if rc != OK:
             self._raise(rc, "quantized_matmul")
+
+    def quantized_matmul_noalloc(self, weight_blocks, input, output, quant_type, m: int, n: int, k: int) -> None:
+        """``quantized_matmul`` on device tensors through the entry point that allocates nothing
+        (its scratch is a fixed array in device memory)."""
+        w, x, y = weight_blocks, input, output
+        if not (_is_torch(w) and w.is_cuda and x.is_cuda and y.is_cuda):
+            raise OtherError("quantized_matmul_noalloc: tensors must live on the GPU")
+        if x.dtype != self._torch.float32 or y.dtype != self._torch.float32:
+            raise Unimplemented("quantized_matmul_noalloc: activations and outputs are f32 on this backend")
+        if x.numel() < m * k or y.numel() < m * n:
+            raise OtherError("quantized_matmul_noalloc: input/output shorter than m*k / m*n")
+        rc = self._lib.gllmq_quantized_matmul_noalloc(self._ctx, w.data_ptr(), w.numel() * w.element_size(), x.data_ptr(),
+                                                      y.data_ptr(), _dtype_id(quant_type), m, n, k, self._stream())
+        if rc != OK:
+            self._raise(rc, "quantized_matmul_noalloc")
 
     def dequantize(self, block_data, output, quant_type) -> None:
         """Whole blocks of ``block_data`` -> f32 into ``output`` (chunks_exact on both sides)."""

@@ -2,10 +2,12 @@
 
     python -m gllm_amd.build
 
-Two steps, both plain compiler invocations (no cmake, no JIT cache):
+Three steps, all plain compiler invocations (no cmake, no JIT cache):
   1. hipcc --genco --offload-arch=gfx950   csrc/gllmq_kernels.hip -> csrc/build/gllmq_kernels.hsaco
-  2. hipcc (host only)                     csrc/gllmq_host.cpp, csrc/gguf_reader.cpp + the code object embedded with
-                                           .incbin                -> gllm_amd/libgllm_hip_quant.so
+  2. hipcc -c --offload-arch=gfx950        csrc/gllmq_noalloc.hip -> csrc/build/gllmq_noalloc.o (host code plus the
+                                           device array behind the entry point that allocates nothing)
+  3. hipcc (host only)                     csrc/gllmq_host.cpp, csrc/gguf_reader.cpp + the object of step 2 + the code
+                                           object of step 1 embedded with .incbin -> gllm_amd/libgllm_hip_quant.so
 """
 from __future__ import annotations
 
@@ -42,8 +44,18 @@ def build_kernels() -> str:
     return HSACO
 
 
+NOALLOC_OBJ = os.path.join(BUILD, "gllmq_noalloc.o")
+
+
+def build_noalloc() -> str:
+    os.makedirs(BUILD, exist_ok=True)
+    _run([HIPCC, "-c", "-fPIC", *DEVICE_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+          os.path.join(CSRC, "gllmq_noalloc.hip"), "-o", NOALLOC_OBJ])
+    return NOALLOC_OBJ
+
+
 def build_host() -> str:
-    _run([HIPCC, "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
+    _run([HIPCC, NOALLOC_OBJ, "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
           "-D__HIP_PLATFORM_AMD__=1", f'-DGLLMQ_HSACO_PATH="{HSACO}"',
           "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROCM, "include"),
           "-I", CSRC, os.path.join(CSRC, "gllmq_host.cpp"), os.path.join(CSRC, "gguf_reader.cpp"), "-o", LIB,
@@ -53,6 +65,7 @@ def build_host() -> str:
 
 def build() -> str:
     build_kernels()
+    build_noalloc()
     return build_host()
 
 

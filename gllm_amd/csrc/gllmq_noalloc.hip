@@ -1,0 +1,62 @@
+// gllmq_quantized_matmul_noalloc: the quantized matmul for callers that cannot allocate device
+// memory (code under stream capture, tight serving loops, harnesses that forbid hipMalloc).
+// The scratch that gllmq_quantized_matmul keeps per stream and grows on demand (arrival
+// counters and slice sums of the K split, activation images and partial sums of the GEMM) is
+// here one array in device memory that exists from the moment the library is loaded.
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+
+#include "gq_host_internal.h"
+
+namespace {
+
+constexpr size_t kNoAllocScratchBytes = GLLMQ_NOALLOC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+
+// Every GPU the library runs on holds its own copy of this array, at its own address, until the
+// process ends.  Zero at load; the arrival counters at its head are left zero by every launch
+// that uses them, and nothing else in it needs a defined value.
+static __device__ __attribute__((used)) __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+std::mutex g_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// The array's address on `device`, looked up once per device with that device current.  In host
+// code the array's name is only a handle for this lookup, never a device address.
+int scratch_address(gllmq_ctx *ctx, int device, void **out)
+{
+    if (device < 0 || device >= kMaxDevices)
+        return gq_ctx_set_error(ctx, GLLMQ_ERR_INVALID, "quantized_matmul_noalloc: device index out of range");
+    std::lock_guard<std::mutex> g(g_mutex);
+    if (!g_scratch_ptr[device]) {
+        int current = -1;
+        hipError_t e = hipGetDevice(&current);
+        if (e == hipSuccess && current != device)
+            return gq_ctx_set_error(ctx, GLLMQ_ERR_INVALID,
+                                    "quantized_matmul_noalloc: the context's device must be the calling thread's current device");
+        void *ptr = nullptr;
+        if (e == hipSuccess) e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            return gq_ctx_set_error(ctx, GLLMQ_ERR_HIP, e != hipSuccess ? hipGetErrorString(e)
+                                                                        : "hipGetSymbolAddress returned no address");
+        }
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = g_scratch_ptr[device];
+    return GLLMQ_OK;
+}
+
+} // namespace
+
+extern "C" int gllmq_quantized_matmul_noalloc(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev,
+                                              float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    void *ptr = nullptr;
+    int rc = scratch_address(ctx, gq_ctx_device(ctx), &ptr);
+    if (rc != GLLMQ_OK) return rc;
+    return gq_quantized_matmul_on_block(ctx, w_dev, w_bytes, x_dev, y_dev, ggml_dtype, m, n, k, ptr, kNoAllocScratchBytes,
+                                        stream);
+}

@@ -191,6 +191,24 @@ int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes,
                               const float *x_dev, float *y_dev, uint32_t ggml_dtype, size_t m,
                               size_t n, size_t k, int act_mode, void *stream);
 
+/* ---- the quantized matmul for callers that cannot allocate ---------------------------------
+ * No counterpart in the reference.  For callers that cannot call hipMalloc: code under stream
+ * capture, tight serving loops, harnesses that forbid allocation.  Same arguments, same kernels
+ * and bit-identical results as gllmq_quantized_matmul, but the scratch (arrival counters and slice
+ * sums of the K split, activation images and partial sums of the GEMM) is one array of
+ * GLLMQ_NOALLOC_SCRATCH_BYTES in device memory that exists from the moment the library is loaded
+ * (every GPU the library runs on holds its own copy until the process ends); the call allocates
+ * and frees nothing.  A shape whose scratch does not fit (the GEMM's: about 72 KiB per 256
+ * elements of K for up to 64 rows plus ksplit * min(m, 64) * n * 4 bytes of partial sums, in
+ * 27.9 MiB) returns GLLMQ_ERR_BAD_SHAPE with the two sizes in gllmq_last_error; every baseline
+ * shape up to 64 rows fits.  All calls on one GPU share that GPU's array, whatever their context
+ * or stream: calls that overlap in time on one GPU race, so keep them on one stream or order them
+ * yourself.  The context's device must be the calling thread's current device. */
+#define GLLMQ_NOALLOC_SCRATCH_BYTES (32u << 20)
+int gllmq_quantized_matmul_noalloc(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev,
+                                   float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,
+                                   void *stream);
+
 /* A list of independent matmuls enqueued back to back on one stream from one call
  * (one decode layer = QKV, O, gate/up, down: build_graph.inc.rs:1960-1999). */
 typedef struct gllmq_matmul_desc {

@@ -1,0 +1,76 @@
+"""The quantized matmul through the entry point that allocates nothing
+(gllmq_quantized_matmul_noalloc, scratch in a fixed device array) against
+gllmq_quantized_matmul on the same inputs, through the C ABI: same kernels and launch shapes, so
+the outputs must be equal bit for bit.  Pairs of calls in a row, the second with a smaller input,
+over the kernels that use scratch: the GEMM with its K split (activation images, partial sums)
+and the 8-row kernels' K split (slice sums, arrival counters)."""
+import numpy as np
+import pytest
+
+from gllm_amd.ggml import row_bytes
+from gllm_amd.synth import random_activations, random_weight
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from gllm_amd.backend import HipBackend
+    return HipBackend(0)
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+    return torch
+
+
+def both(hip, torch, dtype, m, n, k, seed):
+    w = torch.from_numpy(random_weight(dtype, n, k, seed=seed)).cuda()
+    x = torch.from_numpy(random_activations(m, k, seed=seed + 1)).cuda()
+    want = torch.full((m, n), float("nan"), device="cuda")
+    got = torch.full((m, n), float("nan"), device="cuda")
+    hip.quantized_matmul(w, x, want, dtype, m, n, k)
+    hip.quantized_matmul_noalloc(w, x, got, dtype, m, n, k)
+    torch.cuda.synchronize()
+    assert not bool(torch.isnan(want).any())
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32)), f"dtype={dtype} m={m} n={n} k={k}"
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q5_K, Q6_K, Q8_0])
+def test_two_calls_in_a_row_second_smaller(hip, torch, dtype):
+    # GEMM with a K split: 8 row tiles share the device, partial sums meet in the scratch
+    for m, n, k in ((32, 2048, 4096), (16, 520, 2048)):
+        print(f"noalloc GEMM dtype={dtype} m={m} n={n} k={k}", flush=True)
+        both(hip, torch, dtype, m, n, k, seed=3 * m)
+    # few weight rows of long rows on the 8-row kernels: K split with slice sums and arrival
+    # counters in the scratch; then smaller; then the same shape again (counters back at zero)
+    for m, n, k in ((4, 1024, 8192), (2, 256, 4096), (4, 1024, 8192)):
+        print(f"noalloc K split dtype={dtype} m={m} n={n} k={k}", flush=True)
+        both(hip, torch, dtype, m, n, k, seed=5 * m)
+    # shapes without scratch go through the same entry point
+    both(hip, torch, dtype, 1, 777, 1024, seed=9)
+
+
+def test_baseline_shapes_fit(hip, torch):
+    for m in (16, 64):
+        print(f"noalloc baseline GEMM m={m}", flush=True)
+        both(hip, torch, Q4_K, m, 14336, 4096, seed=m)
+    both(hip, torch, Q6_K, 32, 4096, 14336, seed=7)
+
+
+def test_too_large_a_shape_is_refused_and_nothing_runs(hip, torch):
+    from gllm_amd.backend import OtherError
+    m, n, k = 64, 16384, 65536
+    print("noalloc: refusal", flush=True)
+    w = torch.empty(n * row_bytes(Q4_K, k), dtype=torch.uint8, device="cuda")
+    x = torch.zeros(m, k, device="cuda")
+    y = torch.full((m, n), 5.0, device="cuda")
+    with pytest.raises(OtherError, match="scratch"):
+        hip.quantized_matmul_noalloc(w, x, y, Q4_K, m, n, k)
+    torch.cuda.synchronize()
+    assert bool((y == 5.0).all())
+    # and the entry point still works afterwards
+    both(hip, torch, Q4_K, 16, 520, 2048, seed=11)
