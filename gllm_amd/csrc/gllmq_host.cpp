@@ -1,5 +1,5 @@
 // Host side of libgllm_hip_quant.so: the C ABI of include/gllm_hip_quant.h over the
-// embedded gfx950 code object.  Kernels are launched with hipModuleLaunchKernel on the
+// embedded gfx950 code objects.  Kernels are launched with hipModuleLaunchKernel on the
 // caller's stream, the driver-style convention the reference's HIP backend uses
 // (src/compat/hip_backend.rs:211-238), except that the module is loaded and every
 // function resolved once per context instead of once per launch.
@@ -20,18 +20,22 @@
 #include <unordered_map>
 #include <vector>
 
-// The code object built from gllmq_kernels.hip, placed in .rodata by the assembler.
-__asm__(".section .rodata\n"
-        ".balign 4096\n"
-        ".global gllmq_code_object_begin\n"
-        "gllmq_code_object_begin:\n"
-        ".incbin \"" GLLMQ_HSACO_PATH "\"\n"
-        ".global gllmq_code_object_end\n"
-        "gllmq_code_object_end:\n"
-        ".byte 0\n"
-        ".previous\n");
-extern "C" const unsigned char gllmq_code_object_begin[];
-extern "C" const unsigned char gllmq_code_object_end[];
+// The code objects built from the kernels_*.hip translation units, placed in .rodata by the
+// assembler (GLLMQ_HSACO_DIR is the build directory).
+#define GLLMQ_EMBED(NAME)                                                              \
+    __asm__(".section .rodata\n"                                                       \
+            ".balign 4096\n"                                                           \
+            ".global gllmq_co_" #NAME "\n"                                             \
+            "gllmq_co_" #NAME ":\n"                                                    \
+            ".incbin \"" GLLMQ_HSACO_DIR "/kernels_" #NAME ".hsaco\"\n"                 \
+            ".byte 0\n"                                                                \
+            ".previous\n");                                                            \
+    extern "C" const unsigned char gllmq_co_##NAME[];
+GLLMQ_EMBED(codec)
+GLLMQ_EMBED(mm8)
+GLLMQ_EMBED(mm8_q6k_q8_0)
+GLLMQ_EMBED(mmf)
+GLLMQ_EMBED(moe)
 
 namespace {
 
@@ -151,7 +155,7 @@ struct CachedWeights {
 
 struct gllmq_ctx {
     int device = 0;
-    hipModule_t module = nullptr;
+    hipModule_t modules[5] = {}; // one per embedded code object
     hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
     hipFunction_t gather[kNumFormats][2] = {};  // quantized embedding lookup [format][0 = scalar stores, 1 = float4 stores]
     // gated form of the int8 kernels (gate and up rows in one launch, act(gate) * up out):
@@ -168,6 +172,10 @@ struct gllmq_ctx {
     // register-resident activation operands [Mm8Kind][pairs 1,2][early][passes per tile - 1]
     hipFunction_t mm8[MM8_KINDS][3][3] = {};
     hipFunction_t mm8_areg[MM8_KINDS][2][3][2] = {};
+    // streamed form (loader waves + arithmetic waves) [0 = Q4_K, 1 = Q5_K][variant]: register
+    // operands p1_e1, p1_e2, p2_e4, then LDS operands p1_e2, p2_e4, p4_e4
+    hipFunction_t mm8s[2][6] = {};
+    bool use_mm8s = true;                       // "mm8s" = 0: the fetch-and-compute kernels throughout
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
@@ -248,9 +256,15 @@ namespace {
 
 int get_function(gllmq_ctx *ctx, hipFunction_t *f, const char *name)
 {
-    hipError_t e = hipModuleGetFunction(f, ctx->module, name);
+    hipError_t e = hipErrorNotFound;
+    for (hipModule_t mod : ctx->modules) {
+        if (!mod) continue;
+        e = hipModuleGetFunction(f, mod, name);
+        if (e == hipSuccess) break;
+        (void)hipGetLastError();
+    }
     if (e != hipSuccess)
-        return fail(ctx, GLLMQ_ERR_HIP, "kernel %s missing from the code object: %s", name,
+        return fail(ctx, GLLMQ_ERR_HIP, "kernel %s missing from the code objects: %s", name,
                     hipGetErrorString(e));
     ctx->kernel_names[*f] = name;
     return GLLMQ_OK;
@@ -455,6 +469,64 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
     if (!aligned(x, 4) || !aligned(y, 4))
         return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "quantized_matmul: activations and outputs must be 4-byte aligned");
     return -1; // go on
+}
+
+// Q4_K and Q5_K with up to 8 rows in the streamed form (mm8s.hip.inc): taken when the weight rows
+// give every CU at least one 32-row tile, one pass over the weights serves all activation rows and
+// the LDS ring holds enough items.  Returns -1 when the shape is not for it.
+int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n, size_t k,
+             bool act_bf16, void *stream)
+{
+    const int kind = mm8_kind(f.dtype);
+    if (!ctx->use_mm8 || !ctx->use_mm8s || (kind != MM8_Q4K && kind != MM8_Q5K) || m == 0 || m > 8) return -1;
+    if (kind == MM8_Q5K && ctx->mm8_q5k_min_m == 0) return -1;
+    if (!aligned(x, 16) || k % 8 != 0) return -1;
+    const uint32_t cus = static_cast<uint32_t>(ctx->num_cus);
+    const uint32_t groups = static_cast<uint32_t>((k + 255) / 256), tiles = static_cast<uint32_t>((n + 31) / 32);
+    if (tiles < cus) return -1; // fewer tiles than CUs: the K split of the other form keeps more CUs busy
+    const uint32_t rows_per_wg = static_cast<uint32_t>((n + cus - 1) / cus);
+    const uint32_t grid = static_cast<uint32_t>((n + rows_per_wg - 1) / rows_per_wg);
+    const uint32_t mm = static_cast<uint32_t>(m), pi = mm <= 2 ? 0u : (mm <= 4 ? 1u : 2u), pairs = 1u << pi;
+    const uint32_t wg_tiles = (rows_per_wg + 31u) / 32u, tile_rows = (rows_per_wg + wg_tiles - 1u) / wg_tiles;
+    const uint32_t item_bytes = tile_rows * static_cast<uint32_t>(f.block_bytes);
+    const uint32_t fixed = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, 0).total;
+    if (fixed + gq::MM8S_MIN_SLOTS * item_bytes > 160u * 1024u) return -1;
+    const uint32_t items = wg_tiles * groups;
+    uint32_t slots = std::min(items, (160u * 1024u - fixed) / item_bytes);
+    if (slots < items) slots -= slots % gq::MM8S_LOADERS; // a reused ring is a whole number of rounds of the loaders
+    if (slots < items && slots < gq::MM8S_MIN_SLOTS) return -1;
+    const bool areg = groups <= 16 && pi <= 1;
+    const uint32_t steps = (((groups + 7u) / 8u + 1u) / 2u) * mm; // preparation steps per wave
+    int variant;
+    if (areg) variant = pi == 1 ? 2 : (steps <= 1 ? 0 : 1);
+    else variant = 3 + static_cast<int>(pi);
+    Mm8Params P{};
+    P.w = w;
+    P.x = x;
+    P.y = y;
+    P.n = static_cast<uint32_t>(n);
+    P.k = static_cast<uint32_t>(k);
+    P.groups = groups;
+    P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
+    P.m = mm;
+    P.ldx = static_cast<uint32_t>(k);
+    P.ldy = static_cast<uint32_t>(n);
+    P.tiles = tiles;
+    P.grid = grid;
+    P.act_bf16 = act_bf16 ? 1u : 0u;
+    P.xrows = ctx->identity_rows;
+    P.rows_per_wg = rows_per_wg;
+    P.tile_rows = tile_rows;
+    P.ring_slots = slots;
+    P.wg_tiles = wg_tiles;
+    P.last_wg_rows = P.n - (grid - 1u) * rows_per_wg;
+    P.last_wg_tiles = (P.last_wg_rows + tile_rows - 1u) / tile_rows;
+    const gq::Mm8sLds L = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, slots);
+    P.lds_ctrl = L.ctrl;
+    P.lds_ring = L.ring;
+    const uint32_t lds = L.total;
+    return launch(ctx, ctx->mm8s[kind == MM8_Q5K ? 1 : 0][variant], grid, (gq::MM8S_CWAVES + gq::MM8S_LOADERS) * 64, lds, stream,
+                  &P, sizeof P);
 }
 
 // Q4_K, Q5_K and Q6_K on the int8 matrix cores, activation rows in passes of at most 8 (a pass keeps
@@ -671,7 +743,9 @@ int dispatch_matmul(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *
 {
     int rc = run_mmf(ctx, S, f, w, x, y, m, n, k, bf16, stream);
     if (rc >= 0) return rc;
-    // up to 8 rows: the int8 kernel when one pass over the weights does it, else the GEMM
+    // up to 8 rows: the int8 kernels when one pass over the weights does it, else the GEMM
+    rc = run_mm8s(ctx, f, w, x, y, m, n, k, bf16, stream);
+    if (rc >= 0) return rc;
     rc = run_mm8(ctx, S, f, w, x, y, m, n, k, bf16, stream, true);
     if (rc >= 0) return rc;
     if (ctx->mmf_small_min_m > 0) {
@@ -761,11 +835,16 @@ int gllmq_init(gllmq_ctx **out, int device)
             return GLLMQ_ERR_UNIMPLEMENTED;
         }
     }
-    e = hipModuleLoadData(&ctx->module, gllmq_code_object_begin);
-    if (e != hipSuccess) {
-        fprintf(stderr, "gllmq_init: hipModuleLoadData: %s\n", hipGetErrorString(e));
-        delete ctx;
-        return GLLMQ_ERR_HIP;
+    const unsigned char *const images[5] = { gllmq_co_codec, gllmq_co_mm8, gllmq_co_mm8_q6k_q8_0, gllmq_co_mmf, gllmq_co_moe };
+    for (int i = 0; i < 5; ++i) {
+        e = hipModuleLoadData(&ctx->modules[i], images[i]);
+        if (e != hipSuccess) {
+            fprintf(stderr, "gllmq_init: hipModuleLoadData: %s\n", hipGetErrorString(e));
+            for (hipModule_t mod : ctx->modules)
+                if (mod) (void)hipModuleUnload(mod);
+            delete ctx;
+            return GLLMQ_ERR_HIP;
+        }
     }
     int rc = GLLMQ_OK;
     char name[64];
@@ -850,10 +929,17 @@ int gllmq_init(gllmq_ctx **out, int device)
                 }
             }
         if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->glu_act, "gq_glu_act");
+        static const char *const kMm8s[6] = { "p1_e1_a", "p1_e2_a", "p2_e4_a", "p1_e2", "p2_e4", "p4_e4" };
+        for (int q = 0; q < 2; ++q)
+            for (int v = 0; v < 6 && rc == GLLMQ_OK; ++v) {
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s", q ? "q5k" : "q4k", kMm8s[v]);
+                rc = get_function(ctx, &ctx->mm8s[q][v], name);
+            }
     }
     if (rc != GLLMQ_OK) {
         fprintf(stderr, "gllmq_init: %s\n", ctx->err.c_str());
-        (void)hipModuleUnload(ctx->module);
+        for (hipModule_t mod : ctx->modules)
+            if (mod) (void)hipModuleUnload(mod);
         delete ctx;
         return rc;
     }
@@ -869,7 +955,8 @@ void gllmq_destroy(gllmq_ctx *ctx)
     for (CachedWeights &W : ctx->weights)
         if (W.dev) (void)hipFree(W.dev);
     if (ctx->identity_rows) (void)hipFree(ctx->identity_rows);
-    if (ctx->module) (void)hipModuleUnload(ctx->module);
+    for (hipModule_t mod : ctx->modules)
+        if (mod) (void)hipModuleUnload(mod);
     delete ctx;
 }
 
@@ -895,6 +982,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     if (n == "gemv_f32") ctx->gemv_f32 = value != 0;
     else if (n == "mm8") ctx->use_mm8 = value != 0;
     else if (n == "mmf") ctx->use_mmf = value != 0;
+    else if (n == "mm8s") ctx->use_mm8s = value != 0;
     else if (n == "ffn_fused") ctx->ffn_fused = value != 0;
     else if (n == "mmf_small_min_m") ctx->mmf_small_min_m = u;
     else if (n == "mm8_ksplit") ctx->mm8_ksplit_max = u;

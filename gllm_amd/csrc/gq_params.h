@@ -57,6 +57,13 @@ struct Mm8Params {
     uint32_t ksplit, kslice_groups;
     float *part;
     uint32_t *arrive;
+    // streamed kernels (mm8s.hip.inc) only, all worked out by the host so that a loader wave's
+    // way to its first load is short: weight rows per workgroup, rows per tile (<= 32: a
+    // workgroup's rows are cut into tiles of equal height), item slots of the LDS ring (a
+    // multiple of the loader waves unless the ring holds every item), tiles of a full
+    // workgroup and of the last one, rows of the last one, and the LDS offsets of the counters
+    // and of the ring
+    uint32_t rows_per_wg, tile_rows, ring_slots, wg_tiles, last_wg_tiles, last_wg_rows, lds_ctrl, lds_ring;
 };
 
 constexpr uint32_t MM8_SPLIT_MAX_LISTS = 256;        // tile lists (workgroups per slice) of a K-split launch
@@ -103,6 +110,45 @@ GQ_HD inline Mm8Lds mm8_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, 
     L.red = (L.scales + m * groups * 4u + 15u) & ~15u;
     L.stage = L.red + 2u * MM8_WAVES * pairs * 64u * 4u;
     L.total = L.stage + MM8_WAVES * stage_bytes;
+    return L;
+}
+
+// Streamed form of the int8 matrix-core kernels (mm8s.hip.inc): loader waves and arithmetic waves.
+constexpr int MM8S_CWAVES = 8;      // arithmetic waves
+#ifndef GQ_MM8S_LOADERS
+#define GQ_MM8S_LOADERS 4
+#endif
+#ifndef GQ_MM8S_DEPTH
+#define GQ_MM8S_DEPTH 2
+#endif
+constexpr int MM8S_LOADERS = GQ_MM8S_LOADERS; // loader waves
+constexpr int MM8S_RED_BUFS = 4;    // tiles whose partial sums can be waiting in LDS
+constexpr int MM8S_DEPTH = GQ_MM8S_DEPTH; // items a loader keeps unconfirmed
+constexpr uint32_t MM8S_MIN_SLOTS = 2u * MM8S_DEPTH * MM8S_LOADERS; // fewer slots could dead-lock loaders and consumers
+
+struct Mm8sCtrl {                    // counters in LDS, all start at zero
+    uint32_t landed[8];              // per loader: items whose bytes are in LDS
+    uint32_t done[MM8S_CWAVES];      // per arithmetic wave: items consumed
+    uint32_t arrived[MM8S_RED_BUFS]; // per partial-sum buffer: waves that left their sums
+    uint32_t reduced;                // tiles summed and stored
+    uint32_t pad[3];
+};
+
+// LDS carve-up of the streamed kernels: the preparation's planes, sums and scales as in
+// mm8_lds_layout, then the counters, the partial sums and the ring of item slots.
+struct Mm8sLds {
+    Mm8Lds prep;
+    uint32_t ctrl, red, ring, total;
+};
+
+GQ_HD inline Mm8sLds mm8s_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, uint32_t item_bytes, uint32_t slots)
+{
+    Mm8sLds L;
+    L.prep = mm8_lds_layout(groups, m, pairs, 8u, 0u);
+    L.ctrl = (L.prep.red + 15u) & ~15u; // the area of mm8.hip.inc's partial sums and stages is not used here
+    L.red = L.ctrl + static_cast<uint32_t>(sizeof(Mm8sCtrl));
+    L.ring = (L.red + MM8S_RED_BUFS * MM8S_CWAVES * pairs * 64u * 4u + 1023u) & ~1023u;
+    L.total = L.ring + slots * item_bytes;
     return L;
 }
 

@@ -1,0 +1,80 @@
+"""GPU parity of the streamed form of the int8 matrix-core kernels (loader waves bring the weights
+into an LDS ring, arithmetic waves take them out; Q4_K and Q5_K, up to 8 activation rows, at least
+one 32-row tile per CU) against the oracle, through the C ABI.  Same bar as the other matmul
+tests: rel-L2 <= 1e-4 and |err| <= 1e-3 * max|y| against float64 accumulation; against the
+fetch-and-compute kernels (option "mm8s" = 0) the results are equal bit for bit whenever the two
+forms add a row's blocks in the same order, which they do (wave order, block order)."""
+import numpy as np
+import pytest
+
+from gllm_amd.synth import random_activations, random_weight
+from tests.test_gpu_parity import check_close, gpu_matmul
+
+pytestmark = pytest.mark.gpu
+
+Q4_K, Q5_K = 12, 13
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from gllm_amd.backend import HipBackend
+    return HipBackend(0)
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+    return torch
+
+
+def cus(torch):
+    return torch.cuda.get_device_properties(0).multi_processor_count
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q5_K])
+def test_streamed_shapes_against_the_oracle(hip, torch, oracle, dtype):
+    """Rows per workgroup that are and are not whole tiles, a ragged last workgroup, a partial last
+    block of K, one to eight activation rows, rows whose operands stay in registers (K <= 4096) and
+    rows that read them from LDS, and a ring that is reused many times (K = 14336)."""
+    c = cus(torch)
+    # (rows, weight rows, k, streamed?): eight rows of 4096 elements leave no room for the ring
+    # beside their digit planes (99 KB of the 160 KB of LDS) and stay on the other form
+    cases = [(1, 32 * c, 4096, True), (1, 56 * c, 4096, True), (2, 56 * c + 17, 4096, True), (1, 33 * c, 2048, True),
+             (3, 40 * c, 1024, True), (4, 56 * c, 4096 - 8, True), (5, 32 * c + 5, 1536, True), (8, 35 * c, 4096, False),
+             (1, 32 * c, 14336, True), (2, 33 * c + 1, 8192 + 256 * 3 - 64, True), (6, 32 * c, 2048, True),
+             (1, 64 * c + 3, 256, True), (7, 96 * c, 512, True), (8, 32 * c, 1024, True)]
+    for m, n, k, streamed in cases:
+        print(f"streamed dtype={dtype} m={m} n={n} k={k}", flush=True)
+        w, x = random_weight(dtype, n, k, seed=m + n), random_activations(m, k, seed=k + m)
+        want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=16)
+        got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+        check_close(got, want, f"streamed dtype={dtype} m={m} n={n} k={k}")
+        assert hip.last_kernel_name().startswith("gq_mm8s_") == streamed, hip.last_kernel_name()
+
+
+def test_streamed_equals_the_fetch_and_compute_form_bitwise(hip, torch):
+    from gllm_amd.backend import HipBackend
+    plain = HipBackend(0, options={"mm8s": 0})
+    c = cus(torch)
+    for dtype, m, n, k in ((Q4_K, 1, 56 * c, 4096), (Q4_K, 4, 40 * c + 9, 2048), (Q5_K, 2, 56 * c, 4096), (Q4_K, 8, 32 * c, 1024)):
+        print(f"streamed vs plain dtype={dtype} m={m} n={n} k={k}", flush=True)
+        w, x = random_weight(dtype, n, k, seed=3), random_activations(m, k, seed=4)
+        a = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+        assert hip.last_kernel_name().startswith("gq_mm8s_")
+        b = gpu_matmul(plain, torch, w, x, dtype, m, n, k)
+        assert not plain.last_kernel_name().startswith("gq_mm8s_")
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_streamed_large_vocabulary_and_repeats(hip, torch, oracle):
+    """A Llama-3 vocabulary of Q4_K rows (501 rows per workgroup, 16 tiles, the ring reused eight
+    times), twice in a row with different inputs: the counters in LDS start from zero every launch."""
+    n, k = 128256, 4096
+    w = random_weight(Q4_K, n, k, seed=9)
+    for seed in (1, 2):
+        print(f"streamed vocabulary seed={seed}", flush=True)
+        x = random_activations(1, k, seed=seed)
+        want = oracle.quantized_matmul(w, x, Q4_K, 1, n, k, acc=oracle.ACC_F64, threads=16)
+        got = gpu_matmul(hip, torch, w, x, Q4_K, 1, n, k)
+        check_close(got, want, f"vocabulary seed={seed}")
+    assert hip.last_kernel_name().startswith("gq_mm8s_")
