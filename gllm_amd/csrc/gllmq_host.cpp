@@ -176,6 +176,7 @@ struct gllmq_ctx {
     // operands p1_e1, p1_e2, p2_e4, then LDS operands p1_e2, p2_e4, p4_e4
     hipFunction_t mm8s[2][6] = {};
     bool use_mm8s = true;                       // "mm8s" = 0: the fetch-and-compute kernels throughout
+    uint32_t mm8s_min_rows = 8;                 // "mm8s_min_rows": fewest weight rows per CU that take the streamed form
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
@@ -483,7 +484,11 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     if (!aligned(x, 16) || k % 8 != 0) return -1;
     const uint32_t cus = static_cast<uint32_t>(ctx->num_cus);
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256), tiles = static_cast<uint32_t>((n + 31) / 32);
-    if (tiles < cus) return -1; // fewer tiles than CUs: the K split of the other form keeps more CUs busy
+    // Every CU gets its share of the rows, as tiles of equal height; with fewer than 32 rows per CU
+    // the tiles are lower than the 32 rows the matrix cores multiply, which costs nothing here (the
+    // stream bounds the kernel).  Below `mm8s_min_rows` rows per CU the K split of the other form,
+    // which keeps whole tiles and shares their blocks between CUs, is left to do it.
+    if (n < static_cast<size_t>(ctx->mm8s_min_rows) * cus) return -1;
     const uint32_t rows_per_wg = static_cast<uint32_t>((n + cus - 1) / cus);
     const uint32_t grid = static_cast<uint32_t>((n + rows_per_wg - 1) / rows_per_wg);
     const uint32_t mm = static_cast<uint32_t>(m), pi = mm <= 2 ? 0u : (mm <= 4 ? 1u : 2u), pairs = 1u << pi;
@@ -983,6 +988,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "mm8") ctx->use_mm8 = value != 0;
     else if (n == "mmf") ctx->use_mmf = value != 0;
     else if (n == "mm8s") ctx->use_mm8s = value != 0;
+    else if (n == "mm8s_min_rows") ctx->mm8s_min_rows = std::max(1u, u);
     else if (n == "ffn_fused") ctx->ffn_fused = value != 0;
     else if (n == "mmf_small_min_m") ctx->mmf_small_min_m = u;
     else if (n == "mm8_ksplit") ctx->mm8_ksplit_max = u;

@@ -85,7 +85,7 @@ const char *gllmq_version(void);
  * measured best and nothing needs setting; the test-suite uses this to reach every kernel family
  * through the public entry points.  Names: "gemv_f32" (1: f32 multiply-add GEMV instead of the
  * integer-dot one), "mm8" / "mmf" (0: no int8 / f16 matrix-core kernels), "mm8s" (0: no loader-wave form of the
- * int8 kernels), "ffn_fused" (0: the
+ * int8 kernels), "mm8s_min_rows" (fewest weight rows per CU that take it), "ffn_fused" (0: the
  * feed-forward block in three steps), "mm8_q5k_min_m" / "mm8_q6k_min_m" / "mm8_q8_0_min_m"
  * (fewest rows that take the int8 matrix-core kernel; 0 = never), "mmf_small_min_m" (fewest rows
  * of long rows that take the GEMM; 0 = never), "mm8_ksplit" (most K slices; 0 = never split),
