@@ -213,7 +213,10 @@ def run_other(args):
         # one step = one call of the batch entry point over one set; a region is one C call over
         # `steps` consecutive sets of the rotation
         per_set = len(ops)
-        batch = hip.make_batch([d for i in range(steps + copies) for d in sets[i % copies]])
+        # the matmuls of one set are independent of each other (their kernels may overlap); a set is
+        # a step of its own and starts after the one before it
+        batch = hip.make_batch([d for i in range(steps + copies) for d in sets[i % copies]],
+                               after_previous=lambda i: i % per_set == 0)
 
         def region(r):
             hip.run_batch(batch, ((r * steps) % copies) * per_set, steps * per_set)
@@ -455,8 +458,10 @@ def main():
 
     # One list of steps + COPIES descriptors; region r is one C call over `steps` consecutive
     # entries starting where region r - 1 stopped in the rotation.
-    rotating = hip.make_batch([(ws[i % COPIES], x, ys[i % COPIES], DTYPE, M, N, K_DIM) for i in range(steps + COPIES)])
-    resident = hip.make_batch([(ws[0], x, ys[0], DTYPE, M, N, K_DIM)] * steps)
+    # every entry is a call of its own: it starts after the one before it has finished
+    rotating = hip.make_batch([(ws[i % COPIES], x, ys[i % COPIES], DTYPE, M, N, K_DIM) for i in range(steps + COPIES)],
+                              after_previous=lambda i: True)
+    resident = hip.make_batch([(ws[0], x, ys[0], DTYPE, M, N, K_DIM)] * steps, after_previous=lambda i: True)
 
     if args.copy_probe:
         # A plain copy kernel of known size: 33,030,144 bytes read and as many written per launch.

@@ -25,6 +25,7 @@ LIB_PATH = os.path.join(_HERE, "libgllm_hip_quant.so")
 
 OK, ERR_UNIMPLEMENTED, ERR_BAD_SHAPE, ERR_BAD_ALIGNMENT, ERR_HIP, ERR_INVALID = range(6)
 ACT_F32_SPLIT, ACT_BF16 = 0, 1
+DESC_AFTER_PREVIOUS = 1  # gllmq_matmul_desc.flags: the entry depends on the entries before it
 
 
 ARGMAX_NONE = 0xFFFFFFFF  # gllmq_argmax: the row has no entry that is not NaN
@@ -48,7 +49,7 @@ class OtherError(BackendError):
 
 class MatmulDesc(C.Structure):
     _fields_ = [("w_dev", C.c_void_p), ("w_bytes", C.c_size_t), ("x_dev", C.c_void_p),
-                ("y_dev", C.c_void_p), ("ggml_dtype", C.c_uint32), ("reserved", C.c_uint32),
+                ("y_dev", C.c_void_p), ("ggml_dtype", C.c_uint32), ("flags", C.c_uint32),
                 ("m", C.c_size_t), ("n", C.c_size_t), ("k", C.c_size_t)]
 
 
@@ -306,14 +307,17 @@ class HipBackend:
             self._raise(rc, "dequantize")
 
     # --------------------------------------------------------------- extensions
-    def make_batch(self, descs):
+    def make_batch(self, descs, after_previous=None):
         """A descriptor array for ``run_batch``; descs: iterable of (w, x, y, quant_type, m, n, k)
-        device tensors, which must stay alive while the array is used."""
+        device tensors, which must stay alive while the array is used.  ``after_previous``: a
+        function of the entry's index that says whether the entry depends on the ones before it
+        (``GLLMQ_DESC_AFTER_PREVIOUS``); by default the entries are independent."""
         items = list(descs)
         arr = (MatmulDesc * len(items))()
         for i, (w, x, y, qt, m, n, k) in enumerate(items):
+            flags = DESC_AFTER_PREVIOUS if after_previous is not None and after_previous(i) else 0
             arr[i] = MatmulDesc(w.data_ptr(), w.numel() * w.element_size(), x.data_ptr(), y.data_ptr(),
-                                _dtype_id(qt), 0, m, n, k)
+                                _dtype_id(qt), flags, m, n, k)
         return arr
 
     def run_batch(self, arr, start: int = 0, count: int | None = None) -> None:

@@ -8,6 +8,7 @@
 #include "gq_params.h"
 
 #include <hip/hip_runtime_api.h>
+#include <hip/hip_ext.h>
 
 #include <algorithm>
 #include <cmath>
@@ -176,6 +177,7 @@ struct gllmq_ctx {
     // operands p1_e1, p1_e2, p2_e4, then LDS operands p1_e2, p2_e4, p4_e4
     hipFunction_t mm8s[2][6] = {};
     bool use_mm8s = true;                       // "mm8s" = 0: the fetch-and-compute kernels throughout
+    bool batch_overlap = true;                  // "batch_overlap" = 0: the kernels of a batch run strictly one after the other
     uint32_t mm8s_min_rows = 8;                 // "mm8s_min_rows": fewest weight rows per CU that take the streamed form
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
@@ -207,6 +209,13 @@ struct gllmq_ctx {
 
     // One lock over every enqueue on this context: calls from several threads take turns on the
     // host (the kernels they enqueue overlap as their streams allow).
+    // State of gllmq_quantized_matmul_batch while it enqueues (see launch2d).
+    struct Overlap {
+        bool on = false;                 // inside a batch
+        bool entry_first = false;        // the next launch is the first of its entry
+        bool group_open = false;         // a launch of this batch has been enqueued
+        bool group_uses_scratch = false; // a kernel that may still be running uses the scratch
+    } overlap;
     std::recursive_mutex call_mutex;
     std::vector<Scratch> scratch;               // one set per stream the context has been used on
     uint64_t use_counter = 0;
@@ -364,21 +373,39 @@ int grow_scratch(gllmq_ctx *ctx, const Scratch &S, void **buf, size_t *have, siz
     return GLLMQ_OK;
 }
 
+// `uses_scratch`: the kernel reads or writes the stream's scratch.
+// Inside a batch of independent matmuls (ctx->overlap.on) the first launch of an entry is enqueued
+// without the order that a stream otherwise imposes on its kernels, so that it may start while
+// the kernels of earlier entries are still running (the gap between two kernels and the first and
+// last microsecond of each, when few CUs stream, are what a decode layer's matmuls lose most to).
+// Everything else is an ordinary launch, which starts after all earlier work of the stream has
+// finished, unordered launches included.  Two kernels that use the scratch never overlap.
 int launch2d(gllmq_ctx *ctx, hipFunction_t f, uint32_t grid_x, uint32_t grid_y, uint32_t block, uint32_t lds,
-             void *stream, void *params, size_t params_size)
+             void *stream, void *params, size_t params_size, bool uses_scratch = false)
 {
     void *config[] = { HIP_LAUNCH_PARAM_BUFFER_POINTER, params, HIP_LAUNCH_PARAM_BUFFER_SIZE,
                        &params_size, HIP_LAUNCH_PARAM_END };
-    GLLMQ_HIP(ctx, hipModuleLaunchKernel(f, grid_x, grid_y, 1, block, 1, 1, lds, static_cast<hipStream_t>(stream),
-                                         nullptr, config));
+    gllmq_ctx::Overlap &ov = ctx->overlap;
+    const bool unordered = ov.on && ov.entry_first && ov.group_open && !(uses_scratch && ov.group_uses_scratch);
+    if (unordered) {
+        GLLMQ_HIP(ctx, hipExtModuleLaunchKernel(f, grid_x * block, grid_y, 1, block, 1, 1, lds, static_cast<hipStream_t>(stream),
+                                                nullptr, config, nullptr, nullptr, hipExtAnyOrderLaunch));
+    } else {
+        GLLMQ_HIP(ctx, hipModuleLaunchKernel(f, grid_x, grid_y, 1, block, 1, 1, lds, static_cast<hipStream_t>(stream),
+                                             nullptr, config));
+        ov.group_uses_scratch = false; // it waits for everything before it
+    }
+    ov.group_open = true;
+    ov.entry_first = false;
+    ov.group_uses_scratch = ov.group_uses_scratch || uses_scratch;
     ctx->last_kernel = f;
     return GLLMQ_OK;
 }
 
 int launch(gllmq_ctx *ctx, hipFunction_t f, uint32_t grid, uint32_t block, uint32_t lds, void *stream,
-           void *params, size_t params_size)
+           void *params, size_t params_size, bool uses_scratch = false)
 {
-    return launch2d(ctx, f, grid, 1, block, lds, stream, params, params_size);
+    return launch2d(ctx, f, grid, 1, block, lds, stream, params, params_size, uses_scratch);
 }
 
 bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
@@ -644,7 +671,7 @@ int run_mm8(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         const bool even_slices = ksplit == 1 || ppt_row % slice_passes == 0;
         if (pi <= 1 && ppt <= 2 && even_slices)
             fn = glu ? ctx->mm8_glu_areg[gi][pi][ei][ppt - 1] : ctx->mm8_areg[kind][pi][ei][ppt - 1];
-        int rc = launch(ctx, fn, grid * ksplit, 512, lds, stream, &P, sizeof P);
+        int rc = launch(ctx, fn, grid * ksplit, 512, lds, stream, &P, sizeof P, ksplit > 1);
         if (rc != GLLMQ_OK) return rc;
     }
     return GLLMQ_OK;
@@ -710,14 +737,14 @@ int run_mmf(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         P.blocks_per_split = bps;
         P.act_bf16 = act_bf16 ? 1u : 0u;
         MmfPrepParams Q{ P.x, P.ximg, mm, P.k, P.ldx, P.act_bf16 };
-        int rc = launch2d(ctx, ctx->mmf_prep[mt - 1], groups, 16, 64, 0, stream, &Q, sizeof Q);
+        int rc = launch2d(ctx, ctx->mmf_prep[mt - 1], groups, 16, 64, 0, stream, &Q, sizeof Q, true);
         if (rc != GLLMQ_OK) return rc;
         rc = launch(ctx, ctx->mmf_q4k[fmt][mt - 1][act_bf16 ? 1 : 0], row_tiles * ksplit, 512, mmf_lds_bytes(mt, fmt), stream,
-                    &P, sizeof P);
+                    &P, sizeof P, true);
         if (rc == GLLMQ_OK && ksplit > 1) {
             MmfReduceParams R{ P.partial, P.y, mm, P.n, P.ldy, ksplit };
             const uint64_t quads = (static_cast<uint64_t>(mm) * n + 3) / 4;
-            rc = launch(ctx, ctx->mmf_reduce, static_cast<uint32_t>((quads + 255) / 256), 256, 0, stream, &R, sizeof R);
+            rc = launch(ctx, ctx->mmf_reduce, static_cast<uint32_t>((quads + 255) / 256), 256, 0, stream, &R, sizeof R, true);
         }
         if (rc != GLLMQ_OK) return rc;
     }
@@ -988,6 +1015,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "mm8") ctx->use_mm8 = value != 0;
     else if (n == "mmf") ctx->use_mmf = value != 0;
     else if (n == "mm8s") ctx->use_mm8s = value != 0;
+    else if (n == "batch_overlap") ctx->batch_overlap = value != 0;
     else if (n == "mm8s_min_rows") ctx->mm8s_min_rows = std::max(1u, u);
     else if (n == "ffn_fused") ctx->ffn_fused = value != 0;
     else if (n == "mmf_small_min_m") ctx->mmf_small_min_m = u;
@@ -1199,13 +1227,22 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
     Scratch *S = nullptr;
     int rc = acquire_scratch(ctx, stream, &S);
     if (rc != GLLMQ_OK) return rc;
-    for (size_t i = 0; i < count; ++i) {
+    ctx->overlap = gllmq_ctx::Overlap{};
+    ctx->overlap.on = ctx->batch_overlap;
+    for (size_t i = 0; i < count && rc == GLLMQ_OK; ++i) {
         const gllmq_matmul_desc &d = descs[i];
+        if (d.flags & ~static_cast<uint32_t>(GLLMQ_DESC_AFTER_PREVIOUS)) {
+            rc = fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul_batch: unknown flag bits 0x%x in entry %zu", d.flags, i);
+            break;
+        }
+        // an entry that depends on the ones before it starts a new group: its first launch is an
+        // ordinary one
+        ctx->overlap.entry_first = !(d.flags & GLLMQ_DESC_AFTER_PREVIOUS);
         rc = matmul_on_scratch(ctx, *S, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k,
                                GLLMQ_ACT_F32_SPLIT, stream);
-        if (rc != GLLMQ_OK) return rc;
     }
-    return GLLMQ_OK;
+    ctx->overlap = gllmq_ctx::Overlap{};
+    return rc;
 }
 
 int gllmq_moe_route(gllmq_ctx *ctx, const float *logits, size_t tokens, size_t experts, size_t top_k,

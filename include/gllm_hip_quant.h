@@ -85,7 +85,8 @@ const char *gllmq_version(void);
  * measured best and nothing needs setting; the test-suite uses this to reach every kernel family
  * through the public entry points.  Names: "gemv_f32" (1: f32 multiply-add GEMV instead of the
  * integer-dot one), "mm8" / "mmf" (0: no int8 / f16 matrix-core kernels), "mm8s" (0: no loader-wave form of the
- * int8 kernels), "mm8s_min_rows" (fewest weight rows per CU that take it), "ffn_fused" (0: the
+ * int8 kernels), "mm8s_min_rows" (fewest weight rows per CU that take it), "batch_overlap" (0: the kernels of a
+ * batch run strictly one after the other), "ffn_fused" (0: the
  * feed-forward block in three steps), "mm8_q5k_min_m" / "mm8_q6k_min_m" / "mm8_q8_0_min_m"
  * (fewest rows that take the int8 matrix-core kernel; 0 = never), "mmf_small_min_m" (fewest rows
  * of long rows that take the GEMM; 0 = never), "mm8_ksplit" (most K slices; 0 = never split),
@@ -210,15 +211,22 @@ int gllmq_quantized_matmul_noalloc(gllmq_ctx *ctx, const void *w_dev, size_t w_b
                                    float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,
                                    void *stream);
 
-/* A list of independent matmuls enqueued back to back on one stream from one call
- * (one decode layer = QKV, O, gate/up, down: build_graph.inc.rs:1960-1999). */
+/* A list of matmuls enqueued on one stream from one call (the QuantGemm ops of one decode layer
+ * = QKV, O, gate/up, down: build_graph.inc.rs:1960-1999).  The entries are taken to be independent
+ * of each other (no entry reads what another writes): their kernels may overlap in time on the
+ * device, which saves the gap between two kernels and hides each one's first and last
+ * microsecond.  An entry that does depend on the entries before it carries
+ * GLLMQ_DESC_AFTER_PREVIOUS in `flags`: it starts after they have finished.  The batch as a whole
+ * is ordered like any other call: it starts after the stream's earlier work and later work
+ * starts after all of it. */
+#define GLLMQ_DESC_AFTER_PREVIOUS 1u
 typedef struct gllmq_matmul_desc {
     const void *w_dev;
     size_t w_bytes;
     const float *x_dev;
     float *y_dev;
     uint32_t ggml_dtype;
-    uint32_t reserved;
+    uint32_t flags; /* 0 or GLLMQ_DESC_AFTER_PREVIOUS */
     size_t m, n, k;
 } gllmq_matmul_desc;
 

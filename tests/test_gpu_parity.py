@@ -244,6 +244,70 @@ def test_decode_layer_mix_batch(hip, torch, oracle):
         check_close(yd.cpu().numpy(), want, f"layer mix dtype={dtype} n={n} k={k}")
 
 
+def test_batch_overlap_keeps_results_and_order(hip, torch, oracle):
+    """The kernels of a batch of independent matmuls may overlap on the device.  A batch with
+    several users of the stream's scratch (two K-split launches, two GEMMs, which must not overlap
+    with each other), a chain of entries that depend on each other (each reads what the one before
+    it wrote, marked GLLMQ_DESC_AFTER_PREVIOUS) and plain one-row entries, repeated several times
+    with work of the caller's own behind it on the same stream: every result equals, bit for bit,
+    what the same entries give one call at a time."""
+    from gllm_amd.backend import HipBackend
+    print("batch overlap", flush=True)
+    serial = HipBackend(0, options={"batch_overlap": 0})
+    shapes = [(Q4_K, 1, 8192, 4096), (Q6_K, 1, 2048, 11008), (Q4_K, 16, 1024, 2048), (Q5_K, 2, 1024, 12288),
+              (Q8_0, 12, 512, 1024), (Q4_K, 1, 4096, 4096), (Q6_K, 3, 4096, 4096)]
+    base = []
+    for i, (dtype, m, n, k) in enumerate(shapes):
+        w = hip.upload_weights(random_weight(dtype, n, k, seed=50 + i))
+        x = torch.from_numpy(random_activations(m, k, seed=60 + i)).cuda()
+        base.append((w, x, dtype, m, n, k))
+    # a dependent chain: 4096 -> 4096 -> 4096, each entry reading the previous entry's output
+    chain_w = [hip.upload_weights(random_weight(Q4_K, 4096, 4096, seed=70 + i)) for i in range(3)]
+    chain_x0 = torch.from_numpy(random_activations(1, 4096, seed=77)).cuda()
+
+    def build(backend):
+        outs, descs, dep = [], [], []
+        for w, x, dtype, m, n, k in base:
+            y = torch.full((m, n), float("nan"), device="cuda")
+            descs.append((w, x, y, dtype, m, n, k))
+            dep.append(False)
+            outs.append(y)
+        cur = chain_x0
+        for i, w in enumerate(chain_w):
+            y = torch.full((1, 4096), float("nan"), device="cuda")
+            descs.append((w, cur, y, Q4_K, 1, 4096, 4096))
+            dep.append(i > 0)
+            outs.append(y)
+            cur = y
+        return backend.make_batch(descs, after_previous=lambda i: dep[i]), descs, outs
+
+    batch_s, descs_s, outs_s = build(serial)
+    for w, x, y, dtype, m, n, k in descs_s:  # one call at a time
+        serial.quantized_matmul(w, x, y, dtype, m, n, k)
+    torch.cuda.synchronize()
+    want = [o.clone() for o in outs_s]
+    # the chain against the oracle, so that "equal to serial" means "right"
+    hx = chain_x0.cpu().numpy()
+    for i in range(3):
+        hw = chain_w[i].cpu().numpy()
+        hx = oracle.quantized_matmul(hw, hx.astype(np.float32), Q4_K, 1, 4096, 4096, acc=oracle.ACC_F64, threads=8)
+    check_close(want[-1].cpu().numpy(), hx, "dependent chain")
+    batch_o, descs_o, outs_o = build(hip)
+    for rep in range(5):
+        for o in outs_o:
+            o.fill_(float("nan"))
+        hip.run_batch(batch_o)
+        after = outs_o[-1] * 2.0  # the caller's own work behind the batch sees finished results
+        torch.cuda.synchronize()
+        for i, (o, wnt) in enumerate(zip(outs_o, want)):
+            assert torch.equal(o.view(torch.int32), wnt.view(torch.int32)), f"rep {rep} entry {i}"
+        assert torch.equal(after, want[-1] * 2.0)
+    with pytest.raises(Exception):
+        bad = hip.make_batch(descs_o[:1])
+        bad[0].flags = 6
+        hip.run_batch(bad)
+
+
 @pytest.mark.parametrize("dtype", ALL)
 @pytest.mark.parametrize("m", [1, 16, 40])
 def test_bf16_activation_mode(hip, torch, oracle, dtype, m):
