@@ -70,6 +70,10 @@ def percentile(sorted_vals, q):
     return sorted_vals[lo] + (sorted_vals[hi] - sorted_vals[lo]) * (pos - lo)
 
 
+def parse_options(args):
+    return {k: int(v) for k, v in (o.split("=", 1) for o in args.option)}
+
+
 def measure(torch, enqueue_region, steps: int, warmup: int):
     """Times regions of exactly `steps` steps.  `enqueue_region(r)` enqueues the steps of region
     number r on torch's current stream (the stream the library launches on, so the events below
@@ -175,7 +179,7 @@ def run_other(args):
     from gllm_amd.synth import random_activations, random_gate_logits, random_weight
     from oracle import cref  # the checker, here only as the CPU baseline leg
 
-    hip = HipBackend(0)
+    hip = HipBackend(0, options=parse_options(args))
     g = torch.Generator(device="cuda")
     g.manual_seed(0)
     threads = max(1, min(os.cpu_count() or 1, 16))
@@ -359,7 +363,7 @@ def run_other(args):
         "pct_of_hbm_peak": round(gbs / HBM_PEAK_GBS * 100, 2), "tflops": round(flops / us / 1e6, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16" if name.startswith("gemm") else ("f32" if name.startswith(("dequant", "gather")) else "i8"), "data": "synthetic",
-        "config": {"workload": desc, "bytes_per_call": byts, **extra},
+        "config": {"workload": desc, "bytes_per_call": byts, **extra, **({"options": parse_options(args)} if args.option else {})},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
     }
@@ -423,6 +427,8 @@ def main():
     ap.add_argument("--workload", default="gemv_q4k",
                     help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m4, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, lm_head_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
                          "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="kernel-family option of the library for this run (repeatable), e.g. mm8s=0")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch plain device-to-device copies of one 33 MB weight buffer (counter calibration)")
     args = ap.parse_args()
@@ -445,7 +451,7 @@ def main():
     if args.workload != "gemv_q4k":
         run_other(args)
         return
-    hip = HipBackend(0)
+    hip = HipBackend(0, options=parse_options(args))
     g = torch.Generator(device="cuda")
     g.manual_seed(0)
     ws = [device_weight_any(torch, g, DTYPE, N, K_DIM) for _ in range(COPIES)]
@@ -503,7 +509,8 @@ def main():
         "vs_baseline": None,
         "dtype": "i8",
         "data": "synthetic",
-        "config": {"workload": f"Q4_K dequant-GEMV M=1 K={K_DIM} N={N} (GGUF 144-byte super-blocks), f32 activations "
+        "config": {**({"options": parse_options(args)} if args.option else {}),
+                   "workload": f"Q4_K dequant-GEMV M=1 K={K_DIM} N={N} (GGUF 144-byte super-blocks), f32 activations "
                                f"~N(0,1) as 23-bit block fixed point, int8 MFMA with i32 accumulation, f32 scales; "
                                f"weights rotate over {COPIES} copies ({COPIES * nb >> 20} MiB) so every call reads HBM",
                    "bytes_per_call": bytes_per_call, "kernel": hip.last_kernel_name()},

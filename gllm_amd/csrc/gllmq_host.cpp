@@ -34,6 +34,7 @@
     extern "C" const unsigned char gllmq_co_##NAME[];
 GLLMQ_EMBED(codec)
 GLLMQ_EMBED(mm8)
+GLLMQ_EMBED(mm8s)
 GLLMQ_EMBED(mm8_q6k_q8_0)
 GLLMQ_EMBED(mmf)
 GLLMQ_EMBED(moe)
@@ -156,7 +157,7 @@ struct CachedWeights {
 
 struct gllmq_ctx {
     int device = 0;
-    hipModule_t modules[5] = {}; // one per embedded code object
+    hipModule_t modules[6] = {}; // one per embedded code object
     hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
     hipFunction_t gather[kNumFormats][2] = {};  // quantized embedding lookup [format][0 = scalar stores, 1 = float4 stores]
     // gated form of the int8 kernels (gate and up rows in one launch, act(gate) * up out):
@@ -173,11 +174,13 @@ struct gllmq_ctx {
     // register-resident activation operands [Mm8Kind][pairs 1,2][early][passes per tile - 1]
     hipFunction_t mm8[MM8_KINDS][3][3] = {};
     hipFunction_t mm8_areg[MM8_KINDS][2][3][2] = {};
-    // streamed form (loader waves + arithmetic waves) [0 = Q4_K, 1 = Q5_K][variant]: register
+    // streamed form (loader waves + arithmetic waves) [0 = Q4_K, 1 = Q5_K, 2 = Q6_K][variant]: register
     // operands p1_e1, p1_e2, p2_e4, then LDS operands p1_e2, p2_e4, p4_e4
-    hipFunction_t mm8s[2][6] = {};
+    hipFunction_t mm8s[3][7] = {};
     bool use_mm8s = true;                       // "mm8s" = 0: the fetch-and-compute kernels throughout
     bool batch_overlap = true;                  // "batch_overlap" = 0: the kernels of a batch run strictly one after the other
+    bool mm8s_all = false;                      // "mm8s_all" = 1: the streamed form wherever it fits, also where another was timed faster
+    uint32_t mm8s_depth = 0;                    // "mm8s_depth": items a loader keeps unconfirmed, 0 = by item size
     uint32_t mm8s_min_rows = 8;                 // "mm8s_min_rows": fewest weight rows per CU that take the streamed form
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
@@ -506,8 +509,12 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
              bool act_bf16, void *stream)
 {
     const int kind = mm8_kind(f.dtype);
-    if (!ctx->use_mm8 || !ctx->use_mm8s || (kind != MM8_Q4K && kind != MM8_Q5K) || m == 0 || m > 8) return -1;
+    if (!ctx->use_mm8 || !ctx->use_mm8s || (kind != MM8_Q4K && kind != MM8_Q5K && kind != MM8_Q6K) || m == 0 || m > 8) return -1;
     if (kind == MM8_Q5K && ctx->mm8_q5k_min_m == 0) return -1;
+    if (kind == MM8_Q6K && ctx->mm8_q6k_min_m == 0) return -1;
+    const int sfmt = kind == MM8_Q6K ? 2 : kind == MM8_Q5K ? 1 : 0;
+    const uint32_t pieces = sfmt == 2 ? gq::Mm8sFormat<2>::PIECES : sfmt == 1 ? gq::Mm8sFormat<1>::PIECES : gq::Mm8sFormat<0>::PIECES;
+    const uint32_t subs = sfmt == 2 ? 16u : 8u;
     if (!aligned(x, 16) || k % 8 != 0) return -1;
     const uint32_t cus = static_cast<uint32_t>(ctx->num_cus);
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256), tiles = static_cast<uint32_t>((n + 31) / 32);
@@ -520,18 +527,39 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     const uint32_t grid = static_cast<uint32_t>((n + rows_per_wg - 1) / rows_per_wg);
     const uint32_t mm = static_cast<uint32_t>(m), pi = mm <= 2 ? 0u : (mm <= 4 ? 1u : 2u), pairs = 1u << pi;
     const uint32_t wg_tiles = (rows_per_wg + 31u) / 32u, tile_rows = (rows_per_wg + wg_tiles - 1u) / wg_tiles;
-    const uint32_t item_bytes = tile_rows * static_cast<uint32_t>(f.block_bytes);
-    const uint32_t fixed = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, 0).total;
-    if (fixed + gq::MM8S_MIN_SLOTS * item_bytes > 160u * 1024u) return -1;
+    const uint32_t item_bytes = tile_rows * pieces * 16u; // a row of an item in LDS: its 16-byte pieces side by side
+    const uint32_t fixed = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, 0, subs).total;
     const uint32_t items = wg_tiles * groups;
-    uint32_t slots = std::min(items, (160u * 1024u - fixed) / item_bytes);
+    uint32_t slots = std::min(items, (160u * 1024u - std::min(fixed, 160u * 1024u)) / item_bytes);
     if (slots < items) slots -= slots % gq::MM8S_LOADERS; // a reused ring is a whole number of rounds of the loaders
-    if (slots < items && slots < gq::MM8S_MIN_SLOTS) return -1;
+    // items a loader keeps unconfirmed: about MM8S_DEPTH_BYTES worth of them, fewer when a reused
+    // ring is too short for that many
+    uint32_t depth = std::min(gq::MM8S_MAX_DEPTH, std::max(2u, (gq::MM8S_DEPTH_BYTES + item_bytes / 2u) / item_bytes));
+    if (ctx->mm8s_depth) depth = std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth);
+    while (depth > 2u && slots < items && slots < gq::mm8s_min_slots(depth)) --depth;
+    if (slots < items && slots < gq::mm8s_min_slots(depth)) return -1;
     const bool areg = groups <= 16 && pi <= 1;
+    // Q6_K with more than two activation rows and its operands in LDS needs more registers than
+    // a wave of a twelve-wave workgroup has: left to the fetch-and-compute form
+    if (kind == MM8_Q6K && pi > 0 && !areg) return -1;
+    // Where the other kernels were timed faster (rows of 14336 and of 4096 elements over 4096 to
+    // 128256 weight rows): several activation rows of long weight rows, whose preparation every
+    // workgroup repeats in full (Q4_K 2 x 14336 -> 4096: 13.0 against 12.2 us); Q6_K other than
+    // one long row (14336 -> 4096: 14.6 against 16.3 us, 11008 -> 4096: 11.7 against 14.4) or two
+    // short ones (4096 -> 14336: 12.9 against 16.0), the integer-dot GEMV being ahead for one short
+    // row (4096 -> 14336: 11.5 against 12.8 us) and the arithmetic of a Q6_K item costing the same
+    // for a low tile as for a full one.
+    // Five to eight activation rows, and three or four of Q5_K, need more registers here than a
+    // wave of a twelve-wave workgroup has (6 x 2048 -> 14336 Q4_K: 16.1 against 11.0 us).
+    if (!ctx->mm8s_all) {
+        if (pi == 2 || (pi == 1 && kind == MM8_Q5K)) return -1;
+        if (mm >= 2 && groups > 16) return -1;
+        if (kind == MM8_Q6K && !((mm == 1 && groups >= 40) || (mm == 2 && areg))) return -1;
+    }
     const uint32_t steps = (((groups + 7u) / 8u + 1u) / 2u) * mm; // preparation steps per wave
     int variant;
     if (areg) variant = pi == 1 ? 2 : (steps <= 1 ? 0 : 1);
-    else variant = 3 + static_cast<int>(pi);
+    else variant = (pi == 0 && steps > 2) ? 6 : 3 + static_cast<int>(pi);
     Mm8Params P{};
     P.w = w;
     P.x = x;
@@ -553,11 +581,12 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     P.wg_tiles = wg_tiles;
     P.last_wg_rows = P.n - (grid - 1u) * rows_per_wg;
     P.last_wg_tiles = (P.last_wg_rows + tile_rows - 1u) / tile_rows;
-    const gq::Mm8sLds L = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, slots);
+    const gq::Mm8sLds L = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, slots, subs);
     P.lds_ctrl = L.ctrl;
     P.lds_ring = L.ring;
+    P.depth = depth;
     const uint32_t lds = L.total;
-    return launch(ctx, ctx->mm8s[kind == MM8_Q5K ? 1 : 0][variant], grid, (gq::MM8S_CWAVES + gq::MM8S_LOADERS) * 64, lds, stream,
+    return launch(ctx, ctx->mm8s[sfmt][variant], grid, (gq::MM8S_CWAVES + gq::MM8S_LOADERS) * 64, lds, stream,
                   &P, sizeof P);
 }
 
@@ -867,8 +896,9 @@ int gllmq_init(gllmq_ctx **out, int device)
             return GLLMQ_ERR_UNIMPLEMENTED;
         }
     }
-    const unsigned char *const images[5] = { gllmq_co_codec, gllmq_co_mm8, gllmq_co_mm8_q6k_q8_0, gllmq_co_mmf, gllmq_co_moe };
-    for (int i = 0; i < 5; ++i) {
+    const unsigned char *const images[6] = { gllmq_co_codec, gllmq_co_mm8, gllmq_co_mm8s, gllmq_co_mm8_q6k_q8_0, gllmq_co_mmf,
+                                             gllmq_co_moe };
+    for (int i = 0; i < 6; ++i) {
         e = hipModuleLoadData(&ctx->modules[i], images[i]);
         if (e != hipSuccess) {
             fprintf(stderr, "gllmq_init: hipModuleLoadData: %s\n", hipGetErrorString(e));
@@ -961,10 +991,10 @@ int gllmq_init(gllmq_ctx **out, int device)
                 }
             }
         if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->glu_act, "gq_glu_act");
-        static const char *const kMm8s[6] = { "p1_e1_a", "p1_e2_a", "p2_e4_a", "p1_e2", "p2_e4", "p4_e4" };
-        for (int q = 0; q < 2; ++q)
-            for (int v = 0; v < 6 && rc == GLLMQ_OK; ++v) {
-                snprintf(name, sizeof name, "gq_mm8s_%s_%s", q ? "q5k" : "q4k", kMm8s[v]);
+        static const char *const kMm8s[7] = { "p1_e1_a", "p1_e2_a", "p2_e4_a", "p1_e2", "p2_e4", "p4_e4", "p1_e4" };
+        for (int q = 0; q < 3; ++q)
+            for (int v = 0; v < 7 && rc == GLLMQ_OK; ++v) {
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8s[v]);
                 rc = get_function(ctx, &ctx->mm8s[q][v], name);
             }
     }
@@ -1016,6 +1046,8 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "mmf") ctx->use_mmf = value != 0;
     else if (n == "mm8s") ctx->use_mm8s = value != 0;
     else if (n == "batch_overlap") ctx->batch_overlap = value != 0;
+    else if (n == "mm8s_all") ctx->mm8s_all = value != 0;
+    else if (n == "mm8s_depth") ctx->mm8s_depth = u;
     else if (n == "mm8s_min_rows") ctx->mm8s_min_rows = std::max(1u, u);
     else if (n == "ffn_fused") ctx->ffn_fused = value != 0;
     else if (n == "mmf_small_min_m") ctx->mmf_small_min_m = u;

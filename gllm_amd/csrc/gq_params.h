@@ -61,9 +61,9 @@ struct Mm8Params {
     // way to its first load is short: weight rows per workgroup, rows per tile (<= 32: a
     // workgroup's rows are cut into tiles of equal height), item slots of the LDS ring (a
     // multiple of the loader waves unless the ring holds every item), tiles of a full
-    // workgroup and of the last one, rows of the last one, and the LDS offsets of the counters
-    // and of the ring
-    uint32_t rows_per_wg, tile_rows, ring_slots, wg_tiles, last_wg_tiles, last_wg_rows, lds_ctrl, lds_ring;
+    // workgroup and of the last one, rows of the last one, the LDS offsets of the counters
+    // and of the ring, and the items a loader keeps unconfirmed (1 .. MM8S_MAX_DEPTH)
+    uint32_t rows_per_wg, tile_rows, ring_slots, wg_tiles, last_wg_tiles, last_wg_rows, lds_ctrl, lds_ring, depth;
 };
 
 constexpr uint32_t MM8_SPLIT_MAX_LISTS = 256;        // tile lists (workgroups per slice) of a K-split launch
@@ -85,6 +85,17 @@ template <> struct Mm8Format<1> { // Q5_K
     static constexpr uint32_t BLOCK = 176, CHUNKS = 11, QS = 48, STAGE = 6144; // 32 rows x 176 bytes, rounded up
     static constexpr int LOADS = 6;                                           // 5.5 used
 };
+
+// What the streamed kernels (mm8s.hip.inc) need to know of a format: bytes of a block in memory,
+// 16-byte pieces a block's row is fetched as (Q6_K blocks are 210 bytes and only 2-byte aligned:
+// 13 pieces at 16 p and a fourteenth at 194, so no load runs past a block), wave-loads of a
+// 32-row item, sub-block sums the preparation keeps per block.  In LDS a row of an item is its
+// pieces side by side, PIECES * 16 bytes.
+template <int FMT> struct Mm8sFormat;
+template <> struct Mm8sFormat<0> { static constexpr uint32_t BLOCK = 144, PIECES = 9, SUBS = 8; };   // Q4_K
+template <> struct Mm8sFormat<1> { static constexpr uint32_t BLOCK = 176, PIECES = 11, SUBS = 8; };  // Q5_K
+template <> struct Mm8sFormat<2> { static constexpr uint32_t BLOCK = 210, PIECES = 14, SUBS = 16; }; // Q6_K
+GQ_HD constexpr uint32_t mm8s_piece_offset(int fmt, uint32_t piece) { return (fmt == 2 && piece == 13u) ? 194u : 16u * piece; }
 
 // LDS carve-up (bytes) of the int8 matrix-core kernels.
 struct Mm8Lds {
@@ -118,13 +129,19 @@ constexpr int MM8S_CWAVES = 8;      // arithmetic waves
 #ifndef GQ_MM8S_LOADERS
 #define GQ_MM8S_LOADERS 4
 #endif
-#ifndef GQ_MM8S_DEPTH
-#define GQ_MM8S_DEPTH 2
-#endif
 constexpr int MM8S_LOADERS = GQ_MM8S_LOADERS; // loader waves
 constexpr int MM8S_RED_BUFS = 4;    // tiles whose partial sums can be waiting in LDS
-constexpr int MM8S_DEPTH = GQ_MM8S_DEPTH; // items a loader keeps unconfirmed
-constexpr uint32_t MM8S_MIN_SLOTS = 2u * MM8S_DEPTH * MM8S_LOADERS; // fewer slots could dead-lock loaders and consumers
+// Items a loader keeps unconfirmed (its depth D, chosen per launch: what is in flight per CU,
+// not the item count, is what keeps the memory system busy, and items of low tiles are small).
+// A loader's outstanding wave-loads are counted by a 6-bit counter: D times the wave-loads of
+// an item (at most 7) stays below 64.
+constexpr uint32_t MM8S_MAX_DEPTH = 6;
+constexpr uint32_t MM8S_DEPTH_BYTES = 8192; // a loader keeps about this much unconfirmed
+// A consumer sees item i once its loader has requested D more items of its own, that is item
+// i + D * MM8S_LOADERS, and that request waits for the slot of item i + D * MM8S_LOADERS - slots
+// to be free: with slots > D * MM8S_LOADERS every wait is for an item with a smaller number and
+// the chain ends.  Half as many again keep the stream going while items are being multiplied.
+inline GQ_HD uint32_t mm8s_min_slots(uint32_t depth) { return depth * MM8S_LOADERS + MM8S_LOADERS * ((depth + 1u) / 2u); }
 
 struct Mm8sCtrl {                    // counters in LDS, all start at zero
     uint32_t landed[8];              // per loader: items whose bytes are in LDS
@@ -141,10 +158,11 @@ struct Mm8sLds {
     uint32_t ctrl, red, ring, total;
 };
 
-GQ_HD inline Mm8sLds mm8s_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, uint32_t item_bytes, uint32_t slots)
+GQ_HD inline Mm8sLds mm8s_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, uint32_t item_bytes, uint32_t slots,
+                                     uint32_t subs = 8u)
 {
     Mm8sLds L;
-    L.prep = mm8_lds_layout(groups, m, pairs, 8u, 0u);
+    L.prep = mm8_lds_layout(groups, m, pairs, subs, 0u);
     L.ctrl = (L.prep.red + 15u) & ~15u; // the area of mm8.hip.inc's partial sums and stages is not used here
     L.red = L.ctrl + static_cast<uint32_t>(sizeof(Mm8sCtrl));
     L.ring = (L.red + MM8S_RED_BUFS * MM8S_CWAVES * pairs * 64u * 4u + 1023u) & ~1023u;

@@ -8,4 +8,3 @@
 #include "gq_params.h"
 
 #include "mm8.hip.inc"
-#include "mm8s.hip.inc"

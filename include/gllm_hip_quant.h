@@ -85,7 +85,9 @@ const char *gllmq_version(void);
  * measured best and nothing needs setting; the test-suite uses this to reach every kernel family
  * through the public entry points.  Names: "gemv_f32" (1: f32 multiply-add GEMV instead of the
  * integer-dot one), "mm8" / "mmf" (0: no int8 / f16 matrix-core kernels), "mm8s" (0: no loader-wave form of the
- * int8 kernels), "mm8s_min_rows" (fewest weight rows per CU that take it), "batch_overlap" (0: the kernels of a
+ * int8 kernels), "mm8s_min_rows" (fewest weight rows per CU that take it), "mm8s_all" (1: that form wherever the
+ * shape fits it, also where another kernel was timed faster), "mm8s_depth" (items a loader wave
+ * keeps in flight; 0: by item size), "batch_overlap" (0: the kernels of a
  * batch run strictly one after the other), "ffn_fused" (0: the
  * feed-forward block in three steps), "mm8_q5k_min_m" / "mm8_q6k_min_m" / "mm8_q8_0_min_m"
  * (fewest rows that take the int8 matrix-core kernel; 0 = never), "mmf_small_min_m" (fewest rows

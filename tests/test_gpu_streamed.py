@@ -1,6 +1,6 @@
 """GPU parity of the streamed form of the int8 matrix-core kernels (loader waves bring the weights
-into an LDS ring, arithmetic waves take them out; Q4_K and Q5_K, up to 8 activation rows, at least
-one 32-row tile per CU) against the oracle, through the C ABI.  Same bar as the other matmul
+into an LDS ring, arithmetic waves take them out; Q4_K, Q5_K and Q6_K, up to 8 activation rows, at
+least 8 weight rows per CU) against the oracle, through the C ABI.  Same bar as the other matmul
 tests: rel-L2 <= 1e-4 and |err| <= 1e-3 * max|y| against float64 accumulation; against the
 fetch-and-compute kernels (option "mm8s" = 0) the results are equal bit for bit whenever the two
 forms add a row's blocks in the same order, which they do (wave order, block order)."""
@@ -12,13 +12,14 @@ from tests.test_gpu_parity import check_close, gpu_matmul
 
 pytestmark = pytest.mark.gpu
 
-Q4_K, Q5_K = 12, 13
+Q4_K, Q5_K, Q6_K = 12, 13, 14
 
 
 @pytest.fixture(scope="module")
 def hip():
+    # "mm8s_all": the streamed form wherever the shape fits, not only where it was timed fastest
     from gllm_amd.backend import HipBackend
-    return HipBackend(0)
+    return HipBackend(0, options={"mm8s_all": 1})
 
 
 @pytest.fixture(scope="module")
@@ -31,7 +32,7 @@ def cus(torch):
     return torch.cuda.get_device_properties(0).multi_processor_count
 
 
-@pytest.mark.parametrize("dtype", [Q4_K, Q5_K])
+@pytest.mark.parametrize("dtype", [Q4_K, Q5_K, Q6_K])
 def test_streamed_shapes_against_the_oracle(hip, torch, oracle, dtype):
     """Rows per workgroup that are and are not whole tiles, a ragged last workgroup, a partial last
     block of K, one to eight activation rows, rows whose operands stay in registers (K <= 4096) and
@@ -49,21 +50,29 @@ def test_streamed_shapes_against_the_oracle(hip, torch, oracle, dtype):
         want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=16)
         got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
         check_close(got, want, f"streamed dtype={dtype} m={m} n={n} k={k}")
-        assert hip.last_kernel_name().startswith("gq_mm8s_") == streamed, hip.last_kernel_name()
+        # (a Q6_K item is half as large again as a Q4_K one, so fewer of the shapes with many
+        # activation rows leave room for its ring, and three and more rows of long Q6_K rows never
+        # take this form: only the shapes of up to 2 rows are checked there)
+        if dtype != Q6_K or (m <= 2 and k <= 8192):
+            assert hip.last_kernel_name().startswith("gq_mm8s_") == streamed, hip.last_kernel_name()
 
 
 def test_streamed_equals_the_fetch_and_compute_form_bitwise(hip, torch):
     from gllm_amd.backend import HipBackend
-    plain = HipBackend(0, options={"mm8s": 0})
+    plain = HipBackend(0, options={"mm8s": 0, "mm8_q6k_min_m": 1, "mm8_ksplit": 0})  # no K split there: the same order of sums
     c = cus(torch)
-    for dtype, m, n, k in ((Q4_K, 1, 56 * c, 4096), (Q4_K, 4, 40 * c + 9, 2048), (Q5_K, 2, 56 * c, 4096), (Q4_K, 8, 32 * c, 1024)):
+    for dtype, m, n, k in ((Q4_K, 1, 56 * c, 4096), (Q4_K, 4, 40 * c + 9, 2048), (Q5_K, 2, 56 * c, 4096), (Q4_K, 8, 32 * c, 1024),
+                           (Q6_K, 1, 56 * c, 4096), (Q6_K, 2, 16 * c, 14336), (Q6_K, 1, 8 * c + 3, 512)):
         print(f"streamed vs plain dtype={dtype} m={m} n={n} k={k}", flush=True)
         w, x = random_weight(dtype, n, k, seed=3), random_activations(m, k, seed=4)
         a = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
         assert hip.last_kernel_name().startswith("gq_mm8s_")
         b = gpu_matmul(plain, torch, w, x, dtype, m, n, k)
         assert not plain.last_kernel_name().startswith("gq_mm8s_")
-        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        if plain.last_kernel_name().startswith("gq_mm8_"):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        else:  # one or two rows of Q6_K take the integer-dot GEMV there: another order of sums
+            check_close(a, b, f"streamed vs GEMV dtype={dtype} m={m}")
 
 
 def test_streamed_large_vocabulary_and_repeats(hip, torch, oracle):
@@ -78,3 +87,19 @@ def test_streamed_large_vocabulary_and_repeats(hip, torch, oracle):
         got = gpu_matmul(hip, torch, w, x, Q4_K, 1, n, k)
         check_close(got, want, f"vocabulary seed={seed}")
     assert hip.last_kernel_name().startswith("gq_mm8s_")
+
+
+def test_default_choice_of_form(torch):
+    """Without "mm8s_all" the streamed form runs where it was timed fastest: Q4_K single rows
+    everywhere, Q6_K for one long row or two short ones; the results stay those of the oracle's
+    bar either way (checked against the other form here)."""
+    from gllm_amd.backend import HipBackend
+    default, plain = HipBackend(0), HipBackend(0, options={"mm8s": 0})
+    c = cus(torch)
+    for dtype, m, n, k, streamed in ((Q4_K, 1, 56 * c, 4096, True), (Q4_K, 2, 16 * c, 14336, False), (Q6_K, 1, 16 * c, 14336, True),
+                                     (Q6_K, 1, 56 * c, 4096, False), (Q6_K, 2, 56 * c, 4096, True), (Q6_K, 2, 16 * c, 14336, False)):
+        print(f"default form dtype={dtype} m={m} n={n} k={k}", flush=True)
+        w, x = random_weight(dtype, n, k, seed=5), random_activations(m, k, seed=6)
+        a = gpu_matmul(default, torch, w, x, dtype, m, n, k)
+        assert default.last_kernel_name().startswith("gq_mm8s_") == streamed, default.last_kernel_name()
+        check_close(a, gpu_matmul(plain, torch, w, x, dtype, m, n, k), f"default form dtype={dtype} m={m} n={n} k={k}")
