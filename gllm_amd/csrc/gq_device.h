@@ -30,6 +30,29 @@ __device__ __forceinline__ float round_to_bf16(float v)
     return __builtin_bit_cast(float, b & 0xFFFF0000u);
 }
 
+// Block fixed point: the powers of two that turn a group of activations whose largest magnitude
+// has the biased exponent `e_raw` (0 .. 254) into integers below 2^BITS and back.
+//   |x| < 2^(e-126)   ->   |x * pre * up| < 2^BITS,   down = 1 / (pre * up) = 2^(e - 126 - BITS)
+// With e >= BITS one multiplier does (pre = 1).  Smaller groups (down to subnormal ones, e = 1
+// covers them) need more than 2^127: pre lifts the values first, exactly, and `down` is then a
+// subnormal power of two, so such a group keeps its values to 2^(e-126-BITS) >= 2^-148 like any
+// other instead of being rounded to multiples of 2^-126.
+struct BlockScale {
+    float pre, up, down;
+};
+template <int BITS>
+__device__ __forceinline__ BlockScale block_scale(uint32_t e_raw)
+{
+    const uint32_t e = min(max(e_raw, 1u), 254u);
+    const bool tiny = e < static_cast<uint32_t>(BITS);
+    BlockScale s;
+    s.pre = tiny ? __builtin_bit_cast(float, (static_cast<uint32_t>(BITS) + 126u - e) << 23) : 1.0f;
+    s.up = tiny ? __builtin_bit_cast(float, 254u << 23) : __builtin_bit_cast(float, (static_cast<uint32_t>(BITS) + 253u - e) << 23);
+    s.down = tiny ? __builtin_bit_cast(float, 1u << (e + 23u - static_cast<uint32_t>(BITS)))
+                  : __builtin_bit_cast(float, (e + 1u - static_cast<uint32_t>(BITS)) << 23);
+    return s;
+}
+
 // Loads of 2-byte aligned data as wider words.  gfx950 under the HSA ABI runs global
 // memory in unaligned-access mode, so one load instruction serves any byte address.
 template <typename T>

@@ -50,7 +50,8 @@ def _blocks(raw, dtype: int) -> np.ndarray:
     return raw[: nb * bb].reshape(nb, bb)
 
 
-def dequant_q4_k(raw) -> np.ndarray:
+def _parts_q4_k(raw):
+    """(d sc q, dmin m) per element: the two terms whose difference is the weight."""
     b = _blocks(raw, Q4_K)
     d, dmin = _f16(b[:, 0:2]), _f16(b[:, 2:4])
     sc, mn = scale_min_k4(b[:, 4:16])
@@ -60,10 +61,15 @@ def dequant_q4_k(raw) -> np.ndarray:
     q = (qs[:, 32 * (sub // 2) + l] >> (4 * (sub % 2)).astype(np.uint8)) & 0x0F
     ds = d[:, None] * sc[:, sub].astype(np.float32)
     ms = dmin[:, None] * mn[:, sub].astype(np.float32)
-    return (ds * q.astype(np.float32) - ms).astype(np.float32)
+    return ds * q.astype(np.float32), ms
 
 
-def dequant_q5_k(raw) -> np.ndarray:
+def dequant_q4_k(raw) -> np.ndarray:
+    a, ms = _parts_q4_k(raw)
+    return (a - ms).astype(np.float32)
+
+
+def _parts_q5_k(raw):
     b = _blocks(raw, Q5_K)
     d, dmin = _f16(b[:, 0:2]), _f16(b[:, 2:4])
     sc, mn = scale_min_k4(b[:, 4:16])
@@ -75,10 +81,16 @@ def dequant_q5_k(raw) -> np.ndarray:
     q = lo4.astype(np.int32) + 16 * hi1.astype(np.int32)
     ds = d[:, None] * sc[:, sub].astype(np.float32)
     ms = dmin[:, None] * mn[:, sub].astype(np.float32)
-    return (ds * q.astype(np.float32) - ms).astype(np.float32)
+    return ds * q.astype(np.float32), ms
 
 
-def dequant_q6_k(raw) -> np.ndarray:
+def dequant_q5_k(raw) -> np.ndarray:
+    a, ms = _parts_q5_k(raw)
+    return (a - ms).astype(np.float32)
+
+
+def _parts_q6_k(raw):
+    """(d s, q - 32) per element: the weight is their product."""
     b = _blocks(raw, Q6_K)
     ql, qh = b[:, 0:128], b[:, 128:192]
     sc = b[:, 192:208].view(np.int8)
@@ -89,7 +101,12 @@ def dequant_q6_k(raw) -> np.ndarray:
     hi2 = (qh[:, 32 * n + l] >> (2 * quarter).astype(np.uint8)) & 3
     q = lo4.astype(np.int32) + 16 * hi2.astype(np.int32) - 32
     s = sc[:, 8 * n + l // 16 + 2 * quarter].astype(np.float32)
-    return ((d[:, None] * s) * q.astype(np.float32)).astype(np.float32)
+    return d[:, None] * s, q.astype(np.float32)
+
+
+def dequant_q6_k(raw) -> np.ndarray:
+    ds, q = _parts_q6_k(raw)
+    return (ds * q).astype(np.float32)
 
 
 def dequant_q8_0(raw) -> np.ndarray:
@@ -104,6 +121,22 @@ _DEQ = {Q4_K: dequant_q4_k, Q5_K: dequant_q5_k, Q6_K: dequant_q6_k, Q8_0: dequan
 def dequantize(raw, dtype: int) -> np.ndarray:
     """Flat float32 array of all whole blocks in ``raw``."""
     return _DEQ[dtype](raw).reshape(-1)
+
+
+def term_magnitudes(raw, dtype: int) -> np.ndarray:
+    """Per element, the sum of the magnitudes of the terms a fused kernel may form separately
+    before they cancel into the weight: |d sc q| + |dmin m| for Q4_K and Q5_K (the weight is
+    their difference), |d s| (q + 32) + 32 |d s| with the unsigned 6-bit q for Q6_K (the weight is
+    d s (q - 32)), |d q| for Q8_0.  Never below |weight|; the rounding errors of a kernel that
+    multiplies the quants and the offsets apart are bounded in terms of this, not of |weight|.
+    Flat float64 array over all whole blocks of ``raw``."""
+    if dtype == Q4_K or dtype == Q5_K:
+        a, ms = (_parts_q4_k if dtype == Q4_K else _parts_q5_k)(raw)
+        return (np.abs(a.astype(np.float64)) + np.abs(ms.astype(np.float64))).reshape(-1)
+    if dtype == Q6_K:
+        ds, q = _parts_q6_k(raw)
+        return (np.abs(ds.astype(np.float64)) * (q.astype(np.float64) + 64.0)).reshape(-1)
+    return np.abs(dequant_q8_0(raw).astype(np.float64)).reshape(-1)
 
 
 def quantized_matmul(w, x: np.ndarray, dtype: int, m: int, n: int, k: int) -> np.ndarray:
