@@ -142,6 +142,7 @@ EXPORTED_SYMBOLS = [
     "gllmq_gguf_find_tensor", "gllmq_gguf_tensor_data", "gllmq_gguf_meta_type", "gllmq_gguf_meta_u64",
     "gllmq_gguf_meta_i64", "gllmq_gguf_meta_f64", "gllmq_gguf_meta_bool", "gllmq_gguf_meta_str", "gllmq_gguf_meta_array",
     "gllmq_gguf_meta_array_str", "gllmq_gguf_upload",
+    "gllmq_gguf_layer_count", "gllmq_gguf_layer_tensors", "gllmq_gguf_layer_tensor", "gllmq_gguf_mixed_quant_groups",
 ]
 
 

@@ -339,6 +339,37 @@ int finish_open(gllmq_gguf *g, gllmq_gguf **out, char *err_buf, size_t err_len)
     return e.code;
 }
 
+// "blk.{layer}.{projection}.weight" -> (layer, projection); false for any other name
+bool layer_weight_name(const std::string &name, size_t *layer, std::string *projection)
+{
+    if (name.compare(0, 4, "blk.") != 0) return false;
+    const size_t dot1 = name.find('.', 4);
+    if (dot1 == std::string::npos || dot1 == 4) return false;
+    size_t l = 0;
+    for (size_t i = 4; i < dot1; ++i) {
+        if (name[i] < '0' || name[i] > '9' || l > (static_cast<size_t>(-1) >> 8)) return false;
+        l = l * 10 + static_cast<size_t>(name[i] - '0');
+    }
+    const size_t dot2 = name.find('.', dot1 + 1);
+    if (dot2 == std::string::npos || dot2 == dot1 + 1) return false;
+    if (name.compare(dot2, std::string::npos, ".weight") != 0) return false;
+    *layer = l;
+    *projection = name.substr(dot1 + 1, dot2 - dot1 - 1);
+    return true;
+}
+
+// layer -> (projection -> tensor index), over the per-layer weights of the file
+std::map<size_t, std::map<std::string, size_t>> layer_table(const gllmq_gguf *g)
+{
+    std::map<size_t, std::map<std::string, size_t>> table;
+    for (size_t i = 0; i < g->tensors.size(); ++i) {
+        size_t layer;
+        std::string proj;
+        if (layer_weight_name(g->tensors[i].name, &layer, &proj)) table[layer][proj] = i;
+    }
+    return table;
+}
+
 const Value *find_meta(const gllmq_gguf *g, const char *key)
 {
     if (!g || !key) return nullptr;
@@ -428,6 +459,57 @@ const void *gllmq_gguf_tensor_data(const gllmq_gguf *g, size_t index)
 {
     if (!g || index >= g->tensors.size()) return nullptr;
     return g->bytes + g->tensors[index].offset;
+}
+
+size_t gllmq_gguf_layer_count(const gllmq_gguf *g)
+{
+    if (!g) return 0;
+    const auto table = layer_table(g);
+    return table.empty() ? 0 : table.rbegin()->first + 1;
+}
+
+size_t gllmq_gguf_layer_tensors(const gllmq_gguf *g, size_t layer, size_t *indices, size_t capacity)
+{
+    if (!g) return 0;
+    const auto table = layer_table(g);
+    const auto it = table.find(layer);
+    if (it == table.end()) return 0;
+    size_t n = 0;
+    for (const auto &pt : it->second) { // projection-name order
+        if (indices && n < capacity) indices[n] = pt.second;
+        ++n;
+    }
+    return n;
+}
+
+long gllmq_gguf_layer_tensor(const gllmq_gguf *g, size_t layer, const char *projection)
+{
+    if (!g || !projection) return -1;
+    return gllmq_gguf_find_tensor(g, ("blk." + std::to_string(layer) + "." + projection + ".weight").c_str());
+}
+
+size_t gllmq_gguf_mixed_quant_groups(const gllmq_gguf *g, uint32_t *group_of, size_t capacity)
+{
+    if (!g) return 0;
+    const auto table = layer_table(g);
+    // a layer's signature: its (projection, dtype) pairs in projection order
+    typedef std::vector<std::pair<std::string, uint32_t>> Signature;
+    std::map<Signature, std::vector<size_t>> by_signature;
+    for (const auto &lt : table) {
+        Signature sig;
+        for (const auto &pt : lt.second) sig.emplace_back(pt.first, g->tensors[pt.second].dtype);
+        by_signature[sig].push_back(lt.first); // layers arrive in ascending order
+    }
+    for (size_t i = 0; group_of && i < capacity; ++i) group_of[i] = UINT32_MAX;
+    if (by_signature.size() <= 1) return 0;
+    // groups are numbered in signature order (pairs compared in turn, a prefix before its extensions)
+    uint32_t gi = 0;
+    for (const auto &sg : by_signature) {
+        for (size_t layer : sg.second)
+            if (group_of && layer < capacity) group_of[layer] = gi;
+        ++gi;
+    }
+    return by_signature.size();
 }
 
 int gllmq_gguf_meta_type(const gllmq_gguf *g, const char *key)

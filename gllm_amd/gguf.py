@@ -72,6 +72,14 @@ def _declare(L):
     L.gllmq_gguf_meta_array.argtypes = [vp, C.c_char_p, C.POINTER(C.c_uint32), C.POINTER(C.c_uint64)]
     L.gllmq_gguf_meta_array_str.restype = vp
     L.gllmq_gguf_meta_array_str.argtypes = [vp, C.c_char_p, C.c_uint64, C.POINTER(sz)]
+    L.gllmq_gguf_layer_count.restype = sz
+    L.gllmq_gguf_layer_count.argtypes = [vp]
+    L.gllmq_gguf_layer_tensors.restype = sz
+    L.gllmq_gguf_layer_tensors.argtypes = [vp, sz, C.POINTER(sz), sz]
+    L.gllmq_gguf_layer_tensor.restype = C.c_long
+    L.gllmq_gguf_layer_tensor.argtypes = [vp, sz, C.c_char_p]
+    L.gllmq_gguf_mixed_quant_groups.restype = sz
+    L.gllmq_gguf_mixed_quant_groups.argtypes = [vp, C.POINTER(C.c_uint32), sz]
     L.gllmq_gguf_upload.restype = C.c_int
     L.gllmq_gguf_upload.argtypes = [vp, vp, sz, vp, sz, vp]
     return L
@@ -176,27 +184,41 @@ class GgufFile:
         """``{layer: {projection: TensorInfo}}`` over the per-layer weights ``blk.{layer}.{projection}.weight``
         (attn_q, attn_k, attn_v, attn_output, ffn_gate, ffn_up, ffn_down, ...): the (layer, projection) ->
         dtype table a host walks to call the kernels with each matrix's own format, as `*_K_M` files
-        mix Q4_K / Q5_K with Q6_K from layer to layer."""
+        mix Q4_K / Q5_K with Q6_K from layer to layer (gllmq_gguf_layer_count / gllmq_gguf_layer_tensors)."""
         table: dict = {}
-        for t in self.tensors():
-            parts = t.name.split(".")
-            if len(parts) == 4 and parts[0] == "blk" and parts[1].isdigit() and parts[3] == "weight":
-                table.setdefault(int(parts[1]), {})[parts[2]] = t
-        return dict(sorted(table.items()))
+        for layer in range(self._lib.gllmq_gguf_layer_count(self._h)):
+            n = self._lib.gllmq_gguf_layer_tensors(self._h, layer, None, 0)
+            if n == 0:
+                continue
+            idx = (C.c_size_t * n)()
+            self._lib.gllmq_gguf_layer_tensors(self._h, layer, idx, n)
+            table[layer] = {}
+            for i in idx:
+                t = self.tensor(int(i))
+                table[layer][t.name.split(".")[2]] = t
+        return table
+
+    def layer_tensor(self, layer: int, projection: str):
+        """The weight ``blk.{layer}.{projection}.weight`` or None (gllmq_gguf_layer_tensor)."""
+        i = self._lib.gllmq_gguf_layer_tensor(self._h, layer, projection.encode())
+        return None if i < 0 else self.tensor(int(i))
 
     def mixed_quant_groups(self):
         """Layers grouped by their dtype signature (sorted ``(projection, dtype)`` pairs), or None when
         every layer has the same one: what the reference's graph builder detects before it emits
         per-group matmul ops (src/arch/auto_graph_fragments/build_graph.inc.rs:388-470).  Groups come
-        in a fixed order: by signature, then by first layer."""
-        sigs = {layer: tuple(sorted((proj, t.ggml_dtype) for proj, t in projs.items()))
-                for layer, projs in self.layer_table().items()}
-        if len(set(sigs.values())) <= 1:
+        in a fixed order, by signature (gllmq_gguf_mixed_quant_groups)."""
+        layers = self._lib.gllmq_gguf_layer_count(self._h)
+        group_of = (C.c_uint32 * max(layers, 1))()
+        count = self._lib.gllmq_gguf_mixed_quant_groups(self._h, group_of, layers)
+        if count == 0:
             return None
-        groups: dict = {}
-        for layer, sig in sigs.items():
-            groups.setdefault(sig, []).append(layer)
-        return sorted(groups.items(), key=lambda kv: (kv[0], kv[1][0]))
+        table = self.layer_table()
+        groups = [[] for _ in range(count)]
+        for layer in range(layers):
+            if group_of[layer] != 0xFFFFFFFF:
+                groups[group_of[layer]].append(layer)
+        return [(tuple(sorted((proj, t.ggml_dtype) for proj, t in table[g[0]].items())), g) for g in groups]
 
     def upload(self, hip: "backend.HipBackend", key, dst) -> TensorInfo:
         """Copies the tensor's bytes, as stored, into the device uint8 tensor ``dst``."""

@@ -333,6 +333,21 @@ size_t gllmq_gguf_data_offset(const gllmq_gguf *g);
 int gllmq_gguf_tensor_at(const gllmq_gguf *g, size_t index, gllmq_gguf_tensor *out);
 long gllmq_gguf_find_tensor(const gllmq_gguf *g, const char *name); /* -1: no such tensor */
 const void *gllmq_gguf_tensor_data(const gllmq_gguf *g, size_t index);
+/* The per-layer weights `blk.{layer}.{projection}.weight` (attn_q, attn_k, attn_v, attn_output,
+ * ffn_gate, ffn_up, ffn_down, ...) as a table: what a host walks to call the kernels with each
+ * matrix's own format, `*_K_M` files mixing Q4_K / Q5_K with Q6_K from layer to layer.
+ * gllmq_gguf_layer_count: highest layer index + 1 (0: no such tensors);
+ * gllmq_gguf_layer_tensors: number of weights of `layer`, their tensor indices in projection-name
+ * order into indices[0 .. capacity); gllmq_gguf_layer_tensor: index of one of them or -1.
+ * gllmq_gguf_mixed_quant_groups: the reference's grouping of layers by dtype signature (the sorted
+ * (projection, dtype) pairs of a layer; src/arch/auto_graph_fragments/build_graph.inc.rs:388-470):
+ * returns 0 when every layer has the same signature (the reference's plan is None then), else the
+ * number of groups, numbered in signature order; group_of[layer] (layer < capacity) receives the
+ * layer's group, UINT32_MAX for a layer index without weights. */
+size_t gllmq_gguf_layer_count(const gllmq_gguf *g);
+size_t gllmq_gguf_layer_tensors(const gllmq_gguf *g, size_t layer, size_t *indices, size_t capacity);
+long gllmq_gguf_layer_tensor(const gllmq_gguf *g, size_t layer, const char *projection);
+size_t gllmq_gguf_mixed_quant_groups(const gllmq_gguf *g, uint32_t *group_of, size_t capacity);
 /* metadata: the GgufValueType id (0..12) of a key or -1; the getters return 1 when the key
  * exists and converts (gllmq_gguf_meta_u64 like GgufValue::as_u64: unsigned kinds, and signed
  * kinds that are not negative), else 0 */

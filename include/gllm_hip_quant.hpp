@@ -18,6 +18,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <string>
+#include <vector>
 
 #include "gllm_hip_quant.h"
 
@@ -209,6 +210,32 @@ private:
     gllmq_ctx *ctx_ = nullptr;
     BackendError init_error_;
 };
+
+// The layers of an open GGUF file grouped by their per-layer quant-type signature, as the
+// reference's graph builder groups them before it emits per-group matmul ops
+// (MixedQuantPlan, src/arch/auto_graph_fragments/build_graph.inc.rs:388-470): `groups[i]` lists
+// the layers of group i in ascending order, `group_of[layer]` is the layer's group (UINT32_MAX
+// for a layer index without weights).  `mixed()` is false when every layer has the same signature
+// (the reference's plan is None then) and both lists are empty.
+struct MixedQuantPlan {
+    std::vector<std::vector<size_t>> groups;
+    std::vector<uint32_t> group_of;
+    bool mixed() const { return !groups.empty(); }
+};
+
+inline MixedQuantPlan mixed_quant_plan(const gllmq_gguf *file)
+{
+    MixedQuantPlan plan;
+    const size_t layers = gllmq_gguf_layer_count(file);
+    std::vector<uint32_t> group_of(layers, UINT32_MAX);
+    const size_t count = gllmq_gguf_mixed_quant_groups(file, group_of.data(), layers);
+    if (count == 0) return plan;
+    plan.groups.resize(count);
+    for (size_t layer = 0; layer < layers; ++layer)
+        if (group_of[layer] != UINT32_MAX) plan.groups[group_of[layer]].push_back(layer);
+    plan.group_of = std::move(group_of);
+    return plan;
+}
 
 } // namespace gllm
 

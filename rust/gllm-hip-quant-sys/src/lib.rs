@@ -95,6 +95,12 @@ extern "C" {
     pub fn gllmq_gguf_tensor_data(g: *const c_void, index: usize) -> *const c_void;
     pub fn gllmq_gguf_upload(ctx: *mut gllmq_ctx, g: *const c_void, index: usize, dst_dev: *mut c_void,
                              dst_bytes: usize, stream: *mut c_void) -> c_int;
+    // per-layer weight table and the grouping of layers by dtype signature
+    // (src/arch/auto_graph_fragments/build_graph.inc.rs:388-470)
+    pub fn gllmq_gguf_layer_count(g: *const c_void) -> usize;
+    pub fn gllmq_gguf_layer_tensors(g: *const c_void, layer: usize, indices: *mut usize, capacity: usize) -> usize;
+    pub fn gllmq_gguf_layer_tensor(g: *const c_void, layer: usize, projection: *const c_char) -> std::os::raw::c_long;
+    pub fn gllmq_gguf_mixed_quant_groups(g: *const c_void, group_of: *mut u32, capacity: usize) -> usize;
     pub fn gllmq_dequantize_host(ctx: *mut gllmq_ctx, blocks: *const c_void, n_bytes: usize, out: *mut f32,
                                  n_out: usize, ggml_dtype: u32) -> c_int;
     pub fn gllmq_quantized_matmul_host(ctx: *mut gllmq_ctx, w: *const c_void, w_bytes: usize, x: *const f32,
@@ -111,6 +117,22 @@ pub struct HipQuant {
 }
 unsafe impl Send for HipQuant {}
 unsafe impl Sync for HipQuant {}
+
+/// `(group of layer i or None, number of groups)` of an open GGUF file: the layers grouped by
+/// their per-layer quant-type signature as `MixedQuantPlan::group_of` holds them
+/// (build_graph.inc.rs:388-470); `None` for the whole plan when every layer has the same signature.
+///
+/// # Safety
+/// `g` must be a live handle from `gllmq_gguf_open`.
+pub unsafe fn mixed_quant_group_of(g: *const c_void) -> Option<(Vec<Option<u32>>, usize)> {
+    let layers = gllmq_gguf_layer_count(g);
+    let mut group_of = vec![u32::MAX; layers];
+    let groups = gllmq_gguf_mixed_quant_groups(g, group_of.as_mut_ptr(), layers);
+    if groups == 0 {
+        return None;
+    }
+    Some((group_of.into_iter().map(|v| if v == u32::MAX { None } else { Some(v) }).collect(), groups))
+}
 
 /// Mirrors gllm's `BackendError` variants used on this path
 /// (src/engine/executor_types.rs:322-329).

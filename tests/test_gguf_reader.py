@@ -200,3 +200,22 @@ def test_layer_table_and_mixed_quant_groups():
     assert dict(groups[1][0])["ffn_down"] == Q6_K
     uniform, _ = k_m_style_file(down_q6k=())
     assert GgufFile(image=uniform).mixed_quant_groups() is None          # the reference's plan is None for uniform models
+    # look-ups through the C ABI: a weight by (layer, projection), absent ones, names that are not per-layer weights
+    assert g.layer_tensor(3, "ffn_down").name == "blk.3.ffn_down.weight" and g.layer_tensor(3, "ffn_down").ggml_dtype == Q6_K
+    assert g.layer_tensor(4, "ffn_down") is None and g.layer_tensor(0, "attn_q") is None
+    assert all("output_norm" not in projs for projs in table.values())
+
+
+def test_layer_table_with_gaps_and_other_names():
+    """Layer indices without weights get no group; names with another shape than
+    blk.{layer}.{projection}.weight (biases, nested names, non-numeric layers) stay out of the table."""
+    w = lambda name, dt: (name, [256, 4], dt, np.asarray(random_weight(dt, 4, 256, seed=1)).tobytes())
+    tensors = [w("blk.0.ffn_down.weight", Q4_K), w("blk.2.ffn_down.weight", Q6_K), w("blk.5.ffn_down.weight", Q4_K),
+               w("blk.5.ffn_up.weight", Q4_K), w("blk.1.ffn_down.bias", Q4_K), w("blk.x.ffn_down.weight", Q4_K),
+               w("blk.3.attn.q.weight", Q4_K), w("enc.blk.0.ffn_down.weight", Q4_K)]
+    g = GgufFile(image=W.build([("general.architecture", W.STR, "llama")], tensors))
+    table = g.layer_table()
+    assert list(table) == [0, 2, 5] and sorted(table[5]) == ["ffn_down", "ffn_up"]
+    groups = g.mixed_quant_groups()
+    # signatures in order: (ffn_down Q4_K), (ffn_down Q4_K, ffn_up Q4_K), (ffn_down Q6_K)
+    assert [layers for _, layers in groups] == [[0], [5], [2]]
