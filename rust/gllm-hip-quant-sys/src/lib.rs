@@ -226,6 +226,40 @@ impl HipQuant {
                                     x, out, m, hidden, ffn, 0, stream), "ffn_swiglu")
     }
 
+    /// `ExpertRouteTable::from_gate_logits` on the device (src/moe/routing.rs:100-160): gate logits
+    /// `[tokens][experts]` in, the route table `gllmq_moe_matvec` takes out (`route_expert` and
+    /// `route_weight` are `[tokens][top_k]`, `route_len` is `[tokens]`).
+    ///
+    /// # Safety
+    /// All pointers are device pointers on this context's device with the sizes above.
+    pub unsafe fn moe_route_device(&self, logits: *const f32, tokens: usize, experts: usize, top_k: usize,
+                                   capacity_factor: f32, route_expert: *mut u32, route_weight: *mut f32,
+                                   route_len: *mut u32, stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_moe_route(self.ctx, logits, tokens, experts, top_k, capacity_factor, route_expert, route_weight,
+                                   route_len, std::ptr::null_mut(), std::ptr::null_mut(), std::ptr::null_mut(), stream),
+                   "moe_route")
+    }
+
+    /// The routed experts' feed-forward blocks, summed per token with the router weights.  Gate, up
+    /// and down are the expert tensors as the file stores them, `*_stride` the bytes from one
+    /// expert's rows to the next.
+    ///
+    /// # Safety
+    /// All pointers are device pointers on this context's device; the route table is the one
+    /// `moe_route_device` writes.
+    #[allow(clippy::too_many_arguments)]
+    pub unsafe fn moe_matvec_device(&self, gate: *const c_void, gate_bytes: usize, gate_stride: usize,
+                                    up: *const c_void, up_bytes: usize, up_stride: usize, dtype_gate_up: u32,
+                                    down: *const c_void, down_bytes: usize, down_stride: usize, dtype_down: u32,
+                                    x: *const f32, out: *mut f32, tokens: usize, hidden: usize, ffn: usize,
+                                    experts: usize, top_k: usize, route_expert: *const u32, route_weight: *const f32,
+                                    route_len: *const u32, relu_gate: bool, stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_moe_matvec(self.ctx, gate, gate_bytes, gate_stride, up, up_bytes, up_stride, dtype_gate_up,
+                                    down, down_bytes, down_stride, dtype_down, x, out, tokens, hidden, ffn, experts,
+                                    top_k, route_expert, route_weight, route_len, relu_gate as c_int, stream),
+                   "moe_matvec")
+    }
+
     /// `Op::Argmax` over device logits `[rows][ld]` (argmax_token, src/engine/executor_step.rs:48-55):
     /// `token[r]` is `u32::MAX` where the reference returns `None`.
     ///
