@@ -37,6 +37,7 @@ GLLMQ_EMBED(mm8)
 GLLMQ_EMBED(mm8s)
 GLLMQ_EMBED(mm8_q6k_q8_0)
 GLLMQ_EMBED(mmf)
+GLLMQ_EMBED(mmfs)
 GLLMQ_EMBED(moe)
 
 namespace {
@@ -157,7 +158,7 @@ struct CachedWeights {
 
 struct gllmq_ctx {
     int device = 0;
-    hipModule_t modules[6] = {}; // one per embedded code object
+    hipModule_t modules[7] = {}; // one per embedded code object
     hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
     hipFunction_t gather[kNumFormats][2] = {};  // quantized embedding lookup [format][0 = scalar stores, 1 = float4 stores]
     // gated form of the int8 kernels (gate and up rows in one launch, act(gate) * up out):
@@ -184,6 +185,11 @@ struct gllmq_ctx {
     uint32_t mm8s_min_rows = 8;                 // "mm8s_min_rows": fewest weight rows per CU that take the streamed form
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
+    hipFunction_t mmfs[2][2] = {};              // its streamed form [0 = Q4_K, 1 = Q5_K][bf16 mode]
+    bool mmfs_all = false;                      // "mmfs_all" = 1: the streamed GEMM wherever it fits, also where the other form was timed faster
+    bool use_mmfs = true;                       // "mmfs" = 0: the three-launch GEMM throughout
+    uint32_t mmfs_min_rows = 8;                 // "mmfs_min_rows": fewest weight rows per CU that take the streamed GEMM
+    hipFunction_t mmf_prep_lanes = nullptr;     // the images of the streamed form
     hipFunction_t mmf_prep[2] = {};             // its activation preparation [32-row activation tiles - 1]
     hipFunction_t mmf_reduce = nullptr;         // and the in-order sum of its K-split partial results
     hipFunction_t moe_plan = nullptr, moe_act = nullptr, moe_combine = nullptr, moe_route = nullptr;
@@ -780,6 +786,109 @@ int run_mmf(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
     return GLLMQ_OK;
 }
 
+// Launch geometry of the streamed GEMM (mmfs.hip.inc) for one matmul; ok = false when the shape is
+// left to the three-launch form.
+struct MmfsPlan {
+    bool ok = false;
+    uint32_t groups = 0, ksplit = 1, rows_per_wg = 0, grid = 0, wg_tiles = 0, tile_rows = 0, slots = 0, depth = 2,
+             lds_ctrl = 0, lds_ring = 0, lds = 0;
+    size_t img_bytes = 0, need = 0; // scratch: one image per block of K (32 activation rows per launch), then the slice sums
+};
+
+MmfsPlan plan_mmfs(const gllmq_ctx *ctx, const Format &f, size_t m, size_t n, size_t k)
+{
+    MmfsPlan L;
+    const int fmt = f.dtype == T_Q5_K ? 1 : f.dtype == T_Q4_K ? 0 : -1;
+    if (!ctx->use_mmf || !ctx->use_mmfs || fmt < 0 || m == 0 || n == 0) return L;
+    const uint32_t cus = static_cast<uint32_t>(ctx->num_cus);
+    if (n < static_cast<size_t>(ctx->mmfs_min_rows) * cus) return L;
+    // Timed against the three-launch form at 16 and 32 rows: ahead on matrices of up to 6144 x 4096
+    // (32 rows: 13.2 against 22.0 us at 4096 x 4096, 15.5 against 19.2 at 6144 x 4096: two launches
+    // instead of three, no pass over partial sums in a launch of its own), behind from 14336 x 4096
+    // on (24.6 against 23.9 us; 38.1 against 34.0 at 28672 x 4096; 31.8 against 26.7 at 4096 x 14336):
+    // one arithmetic wave per SIMD does not hide its own dependent instructions once the stream
+    // is long enough to matter.
+    if (!ctx->mmfs_all && n * k > (40ull << 20)) return L;
+    L.groups = static_cast<uint32_t>((k + 255) / 256);
+    // a workgroup multiplies four blocks of K (one per arithmetic wave); the row ranges are as many
+    // as give every CU a workgroup
+    L.ksplit = (L.groups + gq::MMFS_CWAVES - 1u) / gq::MMFS_CWAVES;
+    const uint32_t ranges = std::max(1u, cus / L.ksplit);
+    L.rows_per_wg = static_cast<uint32_t>((n + ranges - 1) / ranges);
+    L.grid = static_cast<uint32_t>((n + L.rows_per_wg - 1) / L.rows_per_wg);
+    // the loader's 32-bit offsets stay inside a workgroup's rows
+    if (static_cast<size_t>(L.rows_per_wg) * gllmq_row_bytes(f.dtype, k) > 0xFFFFFFFFull) return L;
+    L.wg_tiles = (L.rows_per_wg + 31u) / 32u;
+    L.tile_rows = (L.rows_per_wg + L.wg_tiles - 1u) / L.wg_tiles; // equal heights, <= 32
+    if (L.ksplit > 1 && L.grid > kScratchArriveBytes / 4u) return L; // one arrival counter per row range
+    const uint32_t pieces = fmt == 1 ? gq::Mm8sFormat<1>::PIECES : gq::Mm8sFormat<0>::PIECES;
+    const uint32_t item_bytes = L.tile_rows * pieces * 16u;
+    L.lds_ctrl = 0;
+    L.lds_ring = (static_cast<uint32_t>(sizeof(gq::Mm8sCtrl)) + gq::MMFS_RED_BUFS * gq::MMFS_CWAVES * 4096u + 1023u) & ~1023u;
+    const uint32_t items = L.wg_tiles * gq::MMFS_CWAVES;
+    L.slots = std::min(items, (160u * 1024u - L.lds_ring) / item_bytes);
+    if (L.slots < items) L.slots -= L.slots % gq::MMFS_LOADERS; // a reused ring is a whole number of rounds of the loaders
+    L.depth = std::min(gq::MM8S_MAX_DEPTH, std::max(2u, (gq::MM8S_DEPTH_BYTES + item_bytes / 2u) / item_bytes));
+    while (L.depth > 2u && L.slots < items && L.slots < gq::mm8s_min_slots(L.depth)) --L.depth;
+    if (L.slots < items && L.slots < gq::mm8s_min_slots(L.depth)) return L;
+    L.lds = L.lds_ring + L.slots * item_bytes;
+    L.img_bytes = static_cast<size_t>(L.groups) * gq::MmfLanes::image;
+    L.need = L.img_bytes + (L.ksplit > 1 ? static_cast<size_t>(L.ksplit) * L.grid * L.wg_tiles * 4096u : 0u);
+    L.ok = true;
+    return L;
+}
+
+// Q4_K and Q5_K, more than 8 activation rows, from `mmfs_min_rows` weight rows per CU up: the
+// streamed GEMM, 32 activation rows per launch (a preparation launch for their images, then the
+// GEMM, which leaves y complete).  Returns -1 when the shape is left to run_mmf.
+int run_mmfs(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
+             size_t k, bool act_bf16, void *stream, size_t min_m = 9)
+{
+    if (m < min_m) return -1;
+    if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
+    const MmfsPlan L = plan_mmfs(ctx, f, m, n, k);
+    if (!L.ok) return -1;
+    int grc = grow_scratch(ctx, S, &S.mmf, &S.mmf_bytes, L.need, stream, "quantized_matmul (GEMM)");
+    if (grc != GLLMQ_OK) return grc;
+    const int fmt = f.dtype == T_Q5_K ? 1 : 0;
+    for (size_t m0 = 0; m0 < m; m0 += 32) {
+        const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(32, m - m0));
+        MmfPrepParams Q{ x + m0 * k, static_cast<uint8_t *>(S.mmf), mm, static_cast<uint32_t>(k), static_cast<uint32_t>(k),
+                         act_bf16 ? 1u : 0u };
+        int rc = launch2d(ctx, ctx->mmf_prep_lanes, L.groups, 16, 64, 0, stream, &Q, sizeof Q, true);
+        if (rc != GLLMQ_OK) return rc;
+        Mm8Params P{};
+        P.w = w;
+        P.x = static_cast<const float *>(S.mmf); // the images
+        P.y = y + m0 * n;
+        P.n = static_cast<uint32_t>(n);
+        P.k = static_cast<uint32_t>(k);
+        P.groups = L.groups;
+        P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
+        P.m = mm;
+        P.ldx = static_cast<uint32_t>(k);
+        P.ldy = static_cast<uint32_t>(n);
+        P.grid = L.grid;
+        P.ksplit = L.ksplit;
+        P.kslice_groups = gq::MMFS_CWAVES;
+        P.part = reinterpret_cast<float *>(static_cast<uint8_t *>(S.mmf) + L.img_bytes);
+        P.arrive = S.mm8_arrive;
+        P.rows_per_wg = L.rows_per_wg;
+        P.tile_rows = L.tile_rows;
+        P.ring_slots = L.slots;
+        P.wg_tiles = L.wg_tiles;
+        P.last_wg_rows = P.n - (L.grid - 1u) * L.rows_per_wg;
+        P.last_wg_tiles = (P.last_wg_rows + L.tile_rows - 1u) / L.tile_rows;
+        P.lds_ctrl = L.lds_ctrl;
+        P.lds_ring = L.lds_ring;
+        P.depth = L.depth;
+        rc = launch(ctx, ctx->mmfs[fmt][act_bf16 ? 1 : 0], L.grid * L.ksplit, (gq::MMFS_CWAVES + gq::MMFS_LOADERS) * 64, L.lds,
+                    stream, &P, sizeof P, true);
+        if (rc != GLLMQ_OK) return rc;
+    }
+    return GLLMQ_OK;
+}
+
 int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
              size_t k, bool act_bf16, void *stream)
 {
@@ -802,7 +911,9 @@ int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
 int dispatch_matmul(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m,
                     size_t n, size_t k, bool bf16, void *stream)
 {
-    int rc = run_mmf(ctx, S, f, w, x, y, m, n, k, bf16, stream);
+    int rc = run_mmfs(ctx, S, f, w, x, y, m, n, k, bf16, stream);
+    if (rc >= 0) return rc;
+    rc = run_mmf(ctx, S, f, w, x, y, m, n, k, bf16, stream);
     if (rc >= 0) return rc;
     // up to 8 rows: the int8 kernels when one pass over the weights does it, else the GEMM
     rc = run_mm8s(ctx, f, w, x, y, m, n, k, bf16, stream);
@@ -896,9 +1007,9 @@ int gllmq_init(gllmq_ctx **out, int device)
             return GLLMQ_ERR_UNIMPLEMENTED;
         }
     }
-    const unsigned char *const images[6] = { gllmq_co_codec, gllmq_co_mm8, gllmq_co_mm8s, gllmq_co_mm8_q6k_q8_0, gllmq_co_mmf,
-                                             gllmq_co_moe };
-    for (int i = 0; i < 6; ++i) {
+    const unsigned char *const images[7] = { gllmq_co_codec, gllmq_co_mm8, gllmq_co_mm8s, gllmq_co_mm8_q6k_q8_0, gllmq_co_mmf,
+                                             gllmq_co_mmfs, gllmq_co_moe };
+    for (int i = 0; i < 7; ++i) {
         e = hipModuleLoadData(&ctx->modules[i], images[i]);
         if (e != hipSuccess) {
             fprintf(stderr, "gllmq_init: hipModuleLoadData: %s\n", hipGetErrorString(e));
@@ -933,6 +1044,7 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_route, "gq_moe_route");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[0], "gq_mmf_prep_t1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[1], "gq_mmf_prep_t2");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep_lanes, "gq_mmf_prep_lanes");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_reduce, "gq_mmf_reduce");
     for (int q = 0; q < 4 && rc == GLLMQ_OK; ++q)
         for (int t = 0; t < 2 && rc == GLLMQ_OK; ++t)
@@ -940,6 +1052,11 @@ int gllmq_init(gllmq_ctx **out, int device)
                 snprintf(name, sizeof name, "gq_mmf_%s_t%d%s", q == 3 ? "q8_0" : q == 2 ? "q6k" : q == 1 ? "q5k" : "q4k", t + 1, b ? "_bf16" : "");
                 rc = get_function(ctx, &ctx->mmf_q4k[q][t][b], name);
             }
+    for (int q = 0; q < 2 && rc == GLLMQ_OK; ++q)
+        for (int b = 0; b < 2 && rc == GLLMQ_OK; ++b) {
+            snprintf(name, sizeof name, "gq_mmfs_%s%s", q ? "q5k" : "q4k", b ? "_bf16" : "");
+            rc = get_function(ctx, &ctx->mmfs[q][b], name);
+        }
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_plan, "gq_moe_plan");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_act, "gq_moe_act");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_combine, "gq_moe_combine");
@@ -1045,6 +1162,9 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "mm8") ctx->use_mm8 = value != 0;
     else if (n == "mmf") ctx->use_mmf = value != 0;
     else if (n == "mm8s") ctx->use_mm8s = value != 0;
+    else if (n == "mmfs") ctx->use_mmfs = value != 0;
+    else if (n == "mmfs_all") ctx->mmfs_all = value != 0;
+    else if (n == "mmfs_min_rows") ctx->mmfs_min_rows = std::max(1u, u);
     else if (n == "batch_overlap") ctx->batch_overlap = value != 0;
     else if (n == "mm8s_all") ctx->mm8s_all = value != 0;
     else if (n == "mm8s_depth") ctx->mm8s_depth = u;
@@ -1624,8 +1744,11 @@ int gllmq_reserve_matmul(gllmq_ctx *ctx, uint32_t dtype, size_t m, size_t n, siz
     // the GEMM is the only matmul kernel family whose scratch depends on the shape; it may take
     // any call of 3 rows and more
     if (m < 3) return GLLMQ_OK;
-    const MmfPlan L = plan_mmf(ctx, m, n, k);
-    return grow_scratch(ctx, *S, &S->mmf, &S->mmf_bytes, L.need, stream, "reserve_matmul");
+    // (either form of it: which one runs also depends on the activation pointer's alignment)
+    size_t need = plan_mmf(ctx, m, n, k).need;
+    const MmfsPlan Ls = plan_mmfs(ctx, *find_format(dtype), m, n, k);
+    if (Ls.ok) need = std::max(need, Ls.need);
+    return grow_scratch(ctx, *S, &S->mmf, &S->mmf_bytes, need, stream, "reserve_matmul");
 }
 
 int gllmq_reserve_ffn(gllmq_ctx *ctx, uint32_t dtype_gate_up, uint32_t dtype_down, size_t m, size_t hidden, size_t ffn,

@@ -30,6 +30,8 @@ __device__ __forceinline__ float round_to_bf16(float v)
     return __builtin_bit_cast(float, b & 0xFFFF0000u);
 }
 
+typedef uint32_t u4v __attribute__((ext_vector_type(4))); // plain 16-byte register quad
+
 // Block fixed point: the powers of two that turn a group of activations whose largest magnitude
 // has the biased exponent `e_raw` (0 .. 254) into integers below 2^BITS and back.
 //   |x| < 2^(e-126)   ->   |x * pre * up| < 2^BITS,   down = 1 / (pre * up) = 2^(e - 126 - BITS)

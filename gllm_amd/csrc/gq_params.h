@@ -230,6 +230,22 @@ struct MmfLds {
     static constexpr uint32_t total = stage + (twice ? 2u : 1u) * stages;
 };
 
+// Streamed form of the Q4_K / Q5_K GEMM (mmfs.hip.inc): takes Mm8Params like the streamed int8
+// kernels, whose loader it shares (x holds the activation images, groups all blocks of K,
+// kslice_groups the blocks of a workgroup's slice of K, grid the row ranges).
+// Its activation image of one block of K and 32 rows, in the order the lanes hold it: for each of
+// the 16 K steps of the block the 64 lanes' 16-byte operands (lane = row + 32 * half of the step)
+// one after the other, hi plane then lo plane; the sub-block sums as the operand of the min term
+// (hi sums for the lanes of half 0, lo sums for half 1); the rows' inverse scales.  Every register
+// of a wave is then one contiguous 1 KiB load.
+struct MmfLanes {
+    static constexpr uint32_t hi = 0, lo = 16u * 1024u, sums = 32u * 1024u, inv = 33u * 1024u, image = 34u * 1024u;
+};
+constexpr int MMFS_CWAVES = 4;  // arithmetic waves = blocks of K per workgroup
+constexpr int MMFS_LOADERS = 4; // loader waves (MM8S_LOADERS: the loader is the same code)
+constexpr int MMFS_RED_BUFS = 3; // tiles whose block sums can be waiting in LDS
+static_assert(MMFS_LOADERS == MM8S_LOADERS, "mm8s_min_slots() is worked out for that many loaders");
+
 struct MmfPrepParams {
     const float *x;
     uint8_t *ximg;

@@ -87,7 +87,8 @@ const char *gllmq_version(void);
  * integer-dot one), "mm8" / "mmf" (0: no int8 / f16 matrix-core kernels), "mm8s" (0: no loader-wave form of the
  * int8 kernels), "mm8s_min_rows" (fewest weight rows per CU that take it), "mm8s_all" (1: that form wherever the
  * shape fits it, also where another kernel was timed faster), "mm8s_depth" (items a loader wave
- * keeps in flight; 0: by item size), "batch_overlap" (0: the kernels of a
+ * keeps in flight; 0: by item size), "mmfs" / "mmfs_all" / "mmfs_min_rows" (the same three for the loader-wave
+ * form of the f16 GEMM), "batch_overlap" (0: the kernels of a
  * batch run strictly one after the other), "ffn_fused" (0: the
  * feed-forward block in three steps), "mm8_q5k_min_m" / "mm8_q6k_min_m" / "mm8_q8_0_min_m"
  * (fewest rows that take the int8 matrix-core kernel; 0 = never), "mmf_small_min_m" (fewest rows
