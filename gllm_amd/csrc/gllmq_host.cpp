@@ -35,6 +35,7 @@
 GLLMQ_EMBED(codec)
 GLLMQ_EMBED(mm8)
 GLLMQ_EMBED(mm8s)
+GLLMQ_EMBED(mm8c)
 GLLMQ_EMBED(mm8_q6k_q8_0)
 GLLMQ_EMBED(mmf)
 GLLMQ_EMBED(mmfs)
@@ -82,6 +83,8 @@ using gq::Mm8Params;
 using gq::MmfParams;
 using gq::MmfPrepParams;
 using gq::MmfReduceParams;
+using gq::Mm8ChainEntry;
+using gq::Mm8ChainParams;
 using gq::MoeActParams;
 using gq::MoeCombineParams;
 using gq::MoeGemvParams;
@@ -141,7 +144,8 @@ struct Scratch {
     size_t moe_bytes = 0;
 };
 
-constexpr size_t kScratchArriveBytes = 4096; // MM8_SPLIT_MAX_LISTS words, padded
+constexpr size_t kScratchArriveBytes = 4096; // MM8_SPLIT_MAX_LISTS words, padded; the chain kernel's counters behind them
+constexpr size_t kChainCountersAt = 512;     // first of its MM8C_MAX_ENTRIES + 1 words in that area
 constexpr size_t kScratchKeysBytes = sizeof(uint64_t) * gq::ARGMAX_MAX_ROWS * gq::ARGMAX_MAX_PARTS;
 constexpr size_t kScratchPartBytes = sizeof(float) * gq::MM8_SPLIT_PART_FLOATS;
 constexpr size_t kScratchFixedBytes = kScratchArriveBytes + kScratchKeysBytes + kScratchPartBytes;
@@ -158,7 +162,7 @@ struct CachedWeights {
 
 struct gllmq_ctx {
     int device = 0;
-    hipModule_t modules[7] = {}; // one per embedded code object
+    hipModule_t modules[8] = {}; // one per embedded code object
     hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
     hipFunction_t gather[kNumFormats][2] = {};  // quantized embedding lookup [format][0 = scalar stores, 1 = float4 stores]
     // gated form of the int8 kernels (gate and up rows in one launch, act(gate) * up out):
@@ -186,6 +190,11 @@ struct gllmq_ctx {
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmfs[2][2] = {};              // its streamed form [0 = Q4_K, 1 = Q5_K][bf16 mode]
+    hipFunction_t mm8c[2] = {};                 // chains of streamed matmuls in one launch [0 = Q4_K, 1 = Q5_K]
+    bool chain_dependent = false;               // "chain_dependent" = 1: entries that depend on the one before stay in the chain
+    bool use_chain = true;                      // "chain" = 0: every entry of a batch is a launch of its own
+    uint32_t chain_spin_limit = 1u << 20;       // "chain_spin_limit": polls of a dependency counter before a workgroup gives up
+    uint32_t *chain_error = nullptr;            // host memory the device can write: set when such a wait ran out
     bool mmfs_all = false;                      // "mmfs_all" = 1: the streamed GEMM wherever it fits, also where the other form was timed faster
     bool use_mmfs = true;                       // "mmfs" = 0: the three-launch GEMM throughout
     uint32_t mmfs_min_rows = 8;                 // "mmfs_min_rows": fewest weight rows per CU that take the streamed GEMM
@@ -889,6 +898,90 @@ int run_mmfs(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, cons
     return GLLMQ_OK;
 }
 
+// A chain of batch entries for one launch of mm8c.hip.inc: consecutive matmuls of one format
+// (Q4_K or Q5_K), one K <= 4096 and one activation row count <= 2 that the streamed kernels
+// would take one by one.  chain_length() says how many entries from `descs` on form one (0 or 1:
+// none); run_chain() launches it.
+bool chain_entry_ok(const gllmq_ctx *ctx, const gllmq_matmul_desc &d, const gllmq_matmul_desc &first)
+{
+    const Format *f = find_format(d.ggml_dtype);
+    if (!f || (f->dtype != T_Q4_K && f->dtype != T_Q5_K)) return false;
+    if (f->dtype == T_Q5_K && ctx->mm8_q5k_min_m == 0) return false;
+    if (d.ggml_dtype != first.ggml_dtype || d.m != first.m || d.k != first.k) return false;
+    if (d.m == 0 || d.m > 2 || d.k == 0 || d.k % 8 != 0 || (d.k + 255) / 256 > 16 || d.n > 0x7FFFFFFFu) return false;
+    if (!d.w_dev || !d.x_dev || !d.y_dev || !aligned(d.x_dev, 16) || !aligned(d.y_dev, 4) || !aligned(d.w_dev, f->w_align)) return false;
+    const size_t rb = gllmq_row_bytes(d.ggml_dtype, d.k);
+    if (rb % f->w_align != 0 || d.w_bytes < d.n * rb) return false;
+    return d.n >= static_cast<size_t>(ctx->mm8s_min_rows) * static_cast<size_t>(ctx->num_cus);
+}
+
+size_t chain_length(const gllmq_ctx *ctx, const gllmq_matmul_desc *descs, size_t count)
+{
+    if (!ctx->use_chain || !ctx->use_mm8 || !ctx->use_mm8s || count < 2) return 0;
+    size_t len = 0;
+    while (len < count && len < gq::MM8C_MAX_ENTRIES && !(descs[len].flags & ~1u) && chain_entry_ok(ctx, descs[len], descs[0])) {
+        // an entry that depends on the one before it starts a launch of its own unless told otherwise:
+        // waiting inside a launch costs more than the launch boundary
+        if (len > 0 && (descs[len].flags & 1u) && !ctx->chain_dependent) break;
+        ++len;
+    }
+    return len;
+}
+
+int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t len, void *stream)
+{
+    const Format &f = *find_format(descs[0].ggml_dtype);
+    const int fmt = f.dtype == T_Q5_K ? 1 : 0;
+    const uint32_t cus = static_cast<uint32_t>(ctx->num_cus);
+    const size_t k = descs[0].k;
+    Mm8ChainParams P{};
+    P.count = static_cast<uint32_t>(len);
+    P.k = static_cast<uint32_t>(k);
+    P.groups = static_cast<uint32_t>((k + 255) / 256);
+    P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
+    P.m = static_cast<uint32_t>(descs[0].m);
+    P.ldx = P.k;
+    P.act_bf16 = 0;
+    const uint32_t pieces = fmt == 1 ? gq::Mm8sFormat<1>::PIECES : gq::Mm8sFormat<0>::PIECES;
+    P.slot_bytes = 32u * pieces * 16u; // a slot holds an item of any entry: 32 rows of one block
+    // LDS: the preparation's planes, sums and scales; the counters; the partial sums; the ring
+    const gq::Mm8Lds prep = gq::mm8_lds_layout(P.groups, P.m, 1u, 8u, 0u);
+    P.lds_ctrl = (prep.red + 15u) & ~15u;
+    const uint32_t red = P.lds_ctrl + static_cast<uint32_t>(sizeof(gq::Mm8sCtrl)) + gq::MM8C_MAX_SLOTS * 4u;
+    P.lds_ring = (red + gq::MM8C_RED_BUFS * gq::MM8C_CWAVES * 64u * 4u + 1023u) & ~1023u;
+    P.depth = 2;
+    if (P.lds_ring >= 160u * 1024u) return -1;
+    uint32_t slots = std::min(gq::MM8C_MAX_SLOTS, (160u * 1024u - P.lds_ring) / P.slot_bytes);
+    slots -= slots % gq::MM8C_LOADERS;
+    if (slots < gq::mm8s_min_slots(P.depth)) return -1;
+    P.ring_slots = slots;
+    P.spin_limit = ctx->chain_spin_limit;
+    P.done = S.mm8_arrive + kChainCountersAt;
+    P.error = ctx->chain_error;
+    uint32_t launched = 0;
+    for (size_t i = 0; i < len; ++i) {
+        const gllmq_matmul_desc &d = descs[i];
+        Mm8ChainEntry &E = P.e[i];
+        E.w = static_cast<const uint8_t *>(d.w_dev);
+        E.x = static_cast<const float *>(d.x_dev);
+        E.y = static_cast<float *>(d.y_dev);
+        E.n = static_cast<uint32_t>(d.n);
+        E.ldy = E.n;
+        E.rows_per_wg = (E.n + cus - 1u) / cus;
+        E.grid = (E.n + E.rows_per_wg - 1u) / E.rows_per_wg;
+        E.wg_tiles = (E.rows_per_wg + 31u) / 32u;
+        E.tile_rows = (E.rows_per_wg + E.wg_tiles - 1u) / E.wg_tiles;
+        E.last_wg_rows = E.n - (E.grid - 1u) * E.rows_per_wg;
+        E.last_wg_tiles = (E.last_wg_rows + E.tile_rows - 1u) / E.tile_rows;
+        E.flags = i > 0 ? (d.flags & 1u) : 0u; // the chain's first entry is ordered by the stream
+        if (i > 0 && E.flags) P.e[i - 1].flags |= 2u;
+        launched = std::max(launched, E.grid);
+    }
+    P.launched = launched;
+    return launch(ctx, ctx->mm8c[fmt], launched, (gq::MM8C_CWAVES + gq::MM8C_LOADERS) * 64, P.lds_ring + slots * P.slot_bytes,
+                  stream, &P, sizeof P, true);
+}
+
 int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
              size_t k, bool act_bf16, void *stream)
 {
@@ -1007,9 +1100,9 @@ int gllmq_init(gllmq_ctx **out, int device)
             return GLLMQ_ERR_UNIMPLEMENTED;
         }
     }
-    const unsigned char *const images[7] = { gllmq_co_codec, gllmq_co_mm8, gllmq_co_mm8s, gllmq_co_mm8_q6k_q8_0, gllmq_co_mmf,
-                                             gllmq_co_mmfs, gllmq_co_moe };
-    for (int i = 0; i < 7; ++i) {
+    const unsigned char *const images[8] = { gllmq_co_codec, gllmq_co_mm8, gllmq_co_mm8s, gllmq_co_mm8c, gllmq_co_mm8_q6k_q8_0,
+                                             gllmq_co_mmf, gllmq_co_mmfs, gllmq_co_moe };
+    for (int i = 0; i < 8; ++i) {
         e = hipModuleLoadData(&ctx->modules[i], images[i]);
         if (e != hipSuccess) {
             fprintf(stderr, "gllmq_init: hipModuleLoadData: %s\n", hipGetErrorString(e));
@@ -1052,6 +1145,8 @@ int gllmq_init(gllmq_ctx **out, int device)
                 snprintf(name, sizeof name, "gq_mmf_%s_t%d%s", q == 3 ? "q8_0" : q == 2 ? "q6k" : q == 1 ? "q5k" : "q4k", t + 1, b ? "_bf16" : "");
                 rc = get_function(ctx, &ctx->mmf_q4k[q][t][b], name);
             }
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8c[0], "gq_mm8c_q4k");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8c[1], "gq_mm8c_q5k");
     for (int q = 0; q < 2 && rc == GLLMQ_OK; ++q)
         for (int b = 0; b < 2 && rc == GLLMQ_OK; ++b) {
             snprintf(name, sizeof name, "gq_mmfs_%s%s", q ? "q5k" : "q4k", b ? "_bf16" : "");
@@ -1084,6 +1179,11 @@ int gllmq_init(gllmq_ctx **out, int device)
         hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->identity_rows), sizeof kRows);
         if (he == hipSuccess) he = hipMemcpy(ctx->identity_rows, kRows, sizeof kRows, hipMemcpyHostToDevice);
         if (he != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "row table: %s", hipGetErrorString(he));
+    }
+    if (rc == GLLMQ_OK) {
+        hipError_t he = hipHostMalloc(reinterpret_cast<void **>(&ctx->chain_error), sizeof(uint32_t), hipHostMallocDefault);
+        if (he == hipSuccess) *ctx->chain_error = 0u;
+        else rc = fail(ctx, GLLMQ_ERR_HIP, "error word: %s", hipGetErrorString(he));
     }
     {
         static const struct { int pi, ei; const char *tag; } kMm8[] = {
@@ -1134,6 +1234,7 @@ void gllmq_destroy(gllmq_ctx *ctx)
     for (CachedWeights &W : ctx->weights)
         if (W.dev) (void)hipFree(W.dev);
     if (ctx->identity_rows) (void)hipFree(ctx->identity_rows);
+    if (ctx->chain_error) (void)hipHostFree(ctx->chain_error);
     for (hipModule_t mod : ctx->modules)
         if (mod) (void)hipModuleUnload(mod);
     delete ctx;
@@ -1163,6 +1264,9 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "mmf") ctx->use_mmf = value != 0;
     else if (n == "mm8s") ctx->use_mm8s = value != 0;
     else if (n == "mmfs") ctx->use_mmfs = value != 0;
+    else if (n == "chain") ctx->use_chain = value != 0;
+    else if (n == "chain_dependent") ctx->chain_dependent = value != 0;
+    else if (n == "chain_spin_limit") ctx->chain_spin_limit = u;
     else if (n == "mmfs_all") ctx->mmfs_all = value != 0;
     else if (n == "mmfs_min_rows") ctx->mmfs_min_rows = std::max(1u, u);
     else if (n == "batch_overlap") ctx->batch_overlap = value != 0;
@@ -1381,8 +1485,25 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
     if (rc != GLLMQ_OK) return rc;
     ctx->overlap = gllmq_ctx::Overlap{};
     ctx->overlap.on = ctx->batch_overlap;
+    if (*ctx->chain_error) { // a chain launched earlier gave up waiting for a counter: its results are not to be trusted
+        *ctx->chain_error = 0u;
+        return fail(ctx, GLLMQ_ERR_HIP, "quantized_matmul_batch: an earlier chained launch timed out waiting for the entry before "
+                                        "(option chain_spin_limit; is the device shared?): its outputs are invalid");
+    }
     for (size_t i = 0; i < count && rc == GLLMQ_OK; ++i) {
         const gllmq_matmul_desc &d = descs[i];
+        // consecutive one-row matmuls of one kind run as one launch whose weight stream never stops
+        const size_t chain = chain_length(ctx, descs + i, count - i);
+        if (chain >= 2) {
+            const int crc = run_chain(ctx, *S, descs + i, chain, stream);
+            if (crc >= 0) {
+                rc = crc;
+                ctx->overlap = gllmq_ctx::Overlap{};
+                ctx->overlap.on = ctx->batch_overlap;
+                i += chain - 1;
+                continue;
+            }
+        }
         if (d.flags & ~static_cast<uint32_t>(GLLMQ_DESC_AFTER_PREVIOUS)) {
             rc = fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul_batch: unknown flag bits 0x%x in entry %zu", d.flags, i);
             break;

@@ -230,6 +230,32 @@ struct MmfLds {
     static constexpr uint32_t total = stage + (twice ? 2u : 1u) * stages;
 };
 
+// A chain of streamed one- or two-row matmuls in one launch (mm8c.hip.inc).
+constexpr int MM8C_CWAVES = 8;             // arithmetic waves (MM8_WAVES: the preparation is the same code)
+constexpr int MM8C_LOADERS = 4;            // loader waves
+constexpr int MM8C_RED_BUFS = 4;           // tiles whose partial sums can be waiting in LDS
+constexpr uint32_t MM8C_MAX_SLOTS = 32;    // ring slots (a counter each)
+constexpr uint32_t MM8C_MAX_ENTRIES = 32;  // matmuls per launch
+struct Mm8ChainEntry {
+    const uint8_t *w;
+    const float *x;
+    float *y;
+    uint32_t n, ldy;
+    // the entry's geometry, worked out by the host as for the streamed kernels: weight rows per
+    // workgroup, workgroups that take part, tile height, tiles of a full and of the last
+    // workgroup, rows of the last workgroup; flags: bit 0 = starts after the entry before it, bit 1 =
+    // the entry behind it does (so this one says when its y is stored)
+    uint32_t rows_per_wg, grid, tile_rows, wg_tiles, last_wg_tiles, last_wg_rows, flags, pad;
+};
+struct Mm8ChainParams {
+    uint32_t count, launched;     // entries, workgroups of the launch (the largest `grid`)
+    uint32_t k, groups, row_bytes, m, ldx, act_bf16;
+    uint32_t ring_slots, slot_bytes, depth, lds_ctrl, lds_ring, spin_limit;
+    uint32_t *done;               // [MM8C_MAX_ENTRIES + 1] workgroups through with each entry, and with the launch; zero at rest
+    uint32_t *error;              // host-visible word, set to 1 when a wait for `done` ran out
+    Mm8ChainEntry e[MM8C_MAX_ENTRIES];
+};
+
 // Streamed form of the Q4_K / Q5_K GEMM (mmfs.hip.inc): takes Mm8Params like the streamed int8
 // kernels, whose loader it shares (x holds the activation images, groups all blocks of K,
 // kslice_groups the blocks of a workgroup's slice of K, grid the row ranges).

@@ -1,0 +1,146 @@
+"""GPU parity of chained matmuls (consecutive one- or two-row Q4_K / Q5_K entries of
+gllmq_quantized_matmul_batch run as one launch whose loader waves go straight on from one matrix's
+weights to the next one's; entries flagged GLLMQ_DESC_AFTER_PREVIOUS wait inside the launch for the
+entry before them) against the oracle, through the C ABI.  The reference launches a decode step
+once (src/compat/hip_backend.rs:224-236) and its ops read each other's outputs
+(build_graph.inc.rs:1960-1999): the dependent case here feeds every matmul the output of the one
+before.  Same bar as the other matmul tests; against the one-launch-per-entry form (option
+"chain" = 0) the results are equal bit for bit."""
+import numpy as np
+import pytest
+
+from gllm_amd.synth import random_activations, random_weight
+from tests.test_gpu_parity import check_close
+
+pytestmark = pytest.mark.gpu
+
+Q4_K, Q5_K = 12, 13
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+    return torch
+
+
+def cus(torch):
+    return torch.cuda.get_device_properties(0).multi_processor_count
+
+
+def dev_weight(torch, w):
+    return torch.from_numpy(np.asarray(w).view(np.uint8).reshape(-1)).cuda()
+
+
+def run_batch(hip, torch, entries, after_previous):
+    """entries: [(w_dev, x_dev, y_dev, dtype, m, n, k)]"""
+    batch = hip.make_batch(entries, after_previous=after_previous)
+    hip.run_batch(batch, 0, len(entries))
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype,m", [(Q4_K, 1), (Q5_K, 1), (Q4_K, 2), (Q5_K, 2)])
+def test_independent_entries_of_different_heights(torch, oracle, dtype, m):
+    """The matmuls of a decoder layer that share K: different numbers of weight rows, so different
+    tile heights and numbers of workgroups per entry, one launch."""
+    from gllm_amd.backend import HipBackend
+    hip, plain = HipBackend(0), HipBackend(0, options={"chain": 0})
+    c, k = cus(torch), 4096
+    ns = [24 * c, 16 * c, 112 * c + 5, 8 * c, 56 * c + 31]
+    host = [(random_weight(dtype, n, k, seed=i), random_activations(m, k, seed=10 + i)) for i, n in enumerate(ns)]
+    outs = []
+    for backend in (hip, plain):
+        entries = [(dev_weight(torch, w), torch.from_numpy(x).cuda(), torch.full((m, n), float("nan"), device="cuda"), dtype, m, n, k)
+                   for (w, x), n in zip(host, ns)]
+        print(f"chain: independent dtype={dtype} m={m} chain={backend is hip}", flush=True)
+        run_batch(backend, torch, entries, after_previous=None)
+        assert backend.last_kernel_name().startswith("gq_mm8c_") == (backend is hip), backend.last_kernel_name()
+        outs.append([e[2].cpu().numpy() for e in entries])
+    for i, ((w, x), n) in enumerate(zip(host, ns)):
+        want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=16)
+        check_close(outs[0][i], want, f"entry {i}")
+        assert np.array_equal(outs[0][i].view(np.uint32), outs[1][i].view(np.uint32)), f"entry {i}: chained and single launches differ"
+
+
+def test_every_entry_reads_the_output_of_the_one_before(torch, oracle):
+    """y0 = W0 x, y1 = W1 y0, ...: every entry waits inside the launch for the workgroups of the one
+    before it and reads what they stored.  Each step is checked against the oracle on the input
+    the GPU actually had; twice, so the counters are seen to be back at zero."""
+    from gllm_amd.backend import HipBackend
+    hip = HipBackend(0, options={"chain_dependent": 1})  # by default a dependent entry starts a launch of its own
+    k = 4096
+    steps = 7
+    ws = [random_weight(Q4_K, k, k, seed=20 + i) for i in range(steps)]
+    wd = [dev_weight(torch, w) for w in ws]
+    for attempt in range(2):
+        x0 = (random_activations(1, k, seed=attempt) * 0.5).astype(np.float32)
+        bufs = [torch.from_numpy(x0).cuda()] + [torch.full((1, k), float("nan"), device="cuda") for _ in range(steps)]
+        entries = [(wd[i], bufs[i], bufs[i + 1], Q4_K, 1, k, k) for i in range(steps)]
+        print(f"chain: dependent entries, attempt {attempt}", flush=True)
+        run_batch(hip, torch, entries, after_previous=lambda i: i > 0)
+        assert hip.last_kernel_name() == "gq_mm8c_q4k"
+        got = [b.cpu().numpy() for b in bufs]
+        for i in range(steps):
+            assert np.isfinite(got[i + 1]).all(), f"step {i}: an entry started before its input was complete"
+            # the outputs grow by about sqrt(k) * |w| per step: scale the next input down on the host side of the check only
+            want = oracle.quantized_matmul(ws[i], got[i], Q4_K, 1, k, k, acc=oracle.ACC_F64, threads=16)
+            check_close(got[i + 1], want, f"attempt {attempt} step {i}")
+
+
+def test_long_batch_splits_into_chains_and_mixes_with_other_kernels(torch, oracle):
+    """Seventy entries (more than one launch holds), every third one dependent, with a Q6_K matmul
+    and a 16-row GEMM in between that are not for the chain kernel; with dependent entries kept in
+    the chains and (the default) starting launches of their own."""
+    from gllm_amd.backend import HipBackend
+    for options in ({"chain_dependent": 1}, {}):
+        many_entries(HipBackend(0, options=options), torch, oracle)
+
+
+def many_entries(hip, torch, oracle):
+    c, k = cus(torch), 2048
+    n = 9 * c + 3
+    w = random_weight(Q4_K, n, k, seed=1)
+    w6 = random_weight(14, 300, k, seed=2)
+    wd, w6d = dev_weight(torch, w), dev_weight(torch, w6)
+    xs = [random_activations(1, k, seed=100 + i) for i in range(70)]
+    x16 = random_activations(16, k, seed=3)
+    entries, kinds = [], []
+    for i, x in enumerate(xs):
+        entries.append((wd, torch.from_numpy(x).cuda(), torch.full((1, n), float("nan"), device="cuda"), Q4_K, 1, n, k))
+        kinds.append(("q4", i))
+        if i == 40:
+            entries.append((w6d, torch.from_numpy(xs[0]).cuda(), torch.full((1, 300), float("nan"), device="cuda"), 14, 1, 300, k))
+            kinds.append(("q6", 0))
+            entries.append((wd, torch.from_numpy(x16).cuda(), torch.full((16, n), float("nan"), device="cuda"), Q4_K, 16, n, k))
+            kinds.append(("gemm", 0))
+    print("chain: seventy entries", flush=True)
+    run_batch(hip, torch, entries, after_previous=lambda i: i % 3 == 1)
+    want1 = {i: oracle.quantized_matmul(w, xs[i], Q4_K, 1, n, k, acc=oracle.ACC_F64, threads=16) for i in (0, 31, 32, 40, 41, 69)}
+    for e, (kind, i) in zip(entries, kinds):
+        got = e[2].cpu().numpy()
+        assert np.isfinite(got).all()
+        if kind == "q4" and i in want1:
+            check_close(got, want1[i], f"entry {i}")
+        elif kind == "q6":
+            check_close(got, oracle.quantized_matmul(w6, xs[0], 14, 1, 300, k, acc=oracle.ACC_F64, threads=4), "the Q6_K entry")
+        elif kind == "gemm":
+            check_close(got, oracle.quantized_matmul(w, x16, Q4_K, 16, n, k, acc=oracle.ACC_F64, threads=16), "the 16-row entry")
+
+
+def test_a_wait_that_runs_out_is_reported_and_the_launch_still_ends(torch):
+    """With no polls allowed a workgroup that finds the entry before it unfinished gives up at once:
+    the launch ends (nothing hangs), the next batch call reports the failure once, and the call
+    after that works again."""
+    from gllm_amd.backend import BackendError, HipBackend
+    hip = HipBackend(0, options={"chain_spin_limit": 0, "chain_dependent": 1})
+    c, k = cus(torch), 4096
+    n = 56 * c
+    wd = dev_weight(torch, random_weight(Q4_K, n, k, seed=1))
+    x = torch.from_numpy(random_activations(1, k, seed=2)).cuda()
+    entries = [(wd, x, torch.empty(1, n, device="cuda"), Q4_K, 1, n, k) for _ in range(6)]
+    print("chain: waits that run out", flush=True)
+    run_batch(hip, torch, entries, after_previous=lambda i: i > 0)
+    with pytest.raises(BackendError, match="timed out"):
+        run_batch(hip, torch, entries, after_previous=lambda i: i > 0)
+    hip.set_option("chain_spin_limit", 1 << 20)
+    run_batch(hip, torch, entries, after_previous=lambda i: i > 0)  # the error was reported once; this one runs
+    run_batch(hip, torch, entries, after_previous=lambda i: i > 0)
