@@ -88,7 +88,9 @@ const char *gllmq_version(void);
  * int8 kernels), "mm8s_min_rows" (fewest weight rows per CU that take it), "mm8s_all" (1: that form wherever the
  * shape fits it, also where another kernel was timed faster), "mm8s_depth" (items a loader wave
  * keeps in flight; 0: by item size), "mmfs" / "mmfs_all" / "mmfs_min_rows" (the same three for the loader-wave
- * form of the f16 GEMM), "batch_overlap" (0: the kernels of a
+ * form of the f16 GEMM), "chain" (0: every entry of a batch is a launch of its own), "chain_dependent" (1: entries
+ * that wait for the one before them stay inside a chained launch and wait there), "chain_spin_limit" (polls of such
+ * a wait before a workgroup gives up and the next batch call reports it), "batch_overlap" (0: the kernels of a
  * batch run strictly one after the other), "ffn_fused" (0: the
  * feed-forward block in three steps), "mm8_q5k_min_m" / "mm8_q6k_min_m" / "mm8_q8_0_min_m"
  * (fewest rows that take the int8 matrix-core kernel; 0 = never), "mmf_small_min_m" (fewest rows
@@ -217,8 +219,9 @@ int gllmq_quantized_matmul_noalloc(gllmq_ctx *ctx, const void *w_dev, size_t w_b
 /* A list of matmuls enqueued on one stream from one call (the QuantGemm ops of one decode layer
  * = QKV, O, gate/up, down: build_graph.inc.rs:1960-1999).  The entries are taken to be independent
  * of each other (no entry reads what another writes): their kernels may overlap in time on the
- * device, which saves the gap between two kernels and hides each one's first and last
- * microsecond.  An entry that does depend on the entries before it carries
+ * device, and consecutive one- or two-row Q4_K / Q5_K entries of one K <= 4096 run as ONE launch
+ * whose loaders go straight on from one matrix to the next (up to 32 entries per launch), which
+ * saves the gaps between kernels and keeps the weight stream going.  An entry that does depend on the entries before it carries
  * GLLMQ_DESC_AFTER_PREVIOUS in `flags`: it starts after they have finished.  The batch as a whole
  * is ordered like any other call: it starts after the stream's earlier work and later work
  * starts after all of it. */
