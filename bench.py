@@ -277,6 +277,34 @@ def run_other(args):
             sec *= 128.0 / pairs_c  # the oracle works pair by pair: scale to the 128 pairs of the workload
             sample = (f"{creps} passes over {pairs_c} (token, expert) pairs of the same expert shapes in {cdt:.1f} s, "
                       f"scaled to 128 pairs")
+    elif name in ("lm_head_argmax_q6k", "lm_head_then_argmax_q6k"):
+        # the tail of a decode step: Q6_K lm_head over a 128256-token vocabulary and the greedy token;
+        # as one call that never writes the logits, or as the matmul and Op::Argmax one after the other
+        dtype, n, k = 14, 128256, 4096
+        copies = 3
+        fused = name == "lm_head_argmax_q6k"
+        ws = [device_weight_any(torch, g, dtype, n, k) for _ in range(copies)]
+        xs = [torch.randn(1, k, device="cuda", generator=g) for _ in range(copies)]
+        logits = torch.empty(1, n, device="cuda")
+        tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+        def run_one(i):
+            if fused:
+                hip.lm_head_argmax(ws[i], xs[i], dtype, n, k, tok)
+            else:
+                hip.quantized_matmul(ws[i], xs[i], logits, dtype, 1, n, k)
+                hip.argmax(logits, tok)
+        t = measure(torch, rotating(run_one, copies), steps, args.warmup)
+        byts = n * row_bytes(dtype, k) + k * 4 + 4
+        flops = 2 * n * k
+        desc = (f"lm_head {TAGS[dtype]} 1x{k}->{n} + greedy token, " +
+                ("one call, logits not written" if fused else "matmul then argmax") + f", rotating over {copies} matrices")
+        if not args.no_cpu:
+            host_w, host_x = random_weight(dtype, n // 8, k, seed=0), random_activations(1, k, seed=0)
+            sec, creps, cdt = cpu_time(lambda: cref.argmax_token(
+                cref.quantized_matmul(host_w, host_x, dtype, 1, n // 8, k, acc=cref.ACC_F32, threads=threads)[0]))
+            sec *= 8.0
+            sample = f"{creps} passes over an eighth of the vocabulary ({n // 8} rows) in {cdt:.1f} s, scaled by 8"
     elif name.startswith("dequant_"):
         # Backend::dequantize of one 14336 x 4096 weight matrix: block bytes in, 4 bytes per element out
         dtype = {"dequant_q4k": 12, "dequant_q5k": 13, "dequant_q6k": 14, "dequant_q8_0": 8}.get(name)
@@ -425,7 +453,7 @@ def main():
     ap.add_argument("--no-context", action="store_true",
                     help="skip the cache-resident and copy-rate context runs (profiling: only the timed kernel launches)")
     ap.add_argument("--workload", default="gemv_q4k",
-                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m4, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, lm_head_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
+                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m4, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, lm_head_q6k, lm_head_argmax_q6k, lm_head_then_argmax_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
                          "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="kernel-family option of the library for this run (repeatable), e.g. mm8s=0")

@@ -119,6 +119,8 @@ def load_library() -> C.CDLL:
     L.gllmq_ffn_swiglu.argtypes = [vp, vp, vp, sz, u32, vp, sz, u32, vp, vp, sz, sz, sz, C.c_int, vp]
     L.gllmq_argmax.restype = C.c_int
     L.gllmq_argmax.argtypes = [vp, vp, sz, sz, sz, vp, vp, vp]
+    L.gllmq_lm_head_argmax.restype = C.c_int
+    L.gllmq_lm_head_argmax.argtypes = [vp, vp, sz, vp, C.c_uint32, sz, sz, vp, vp, vp, vp]
     L.gllmq_dequantize_host.restype = C.c_int
     L.gllmq_dequantize_host.argtypes = [vp, vp, sz, vp, sz, u32]
     L.gllmq_quant_gather_host.restype = C.c_int
@@ -134,7 +136,7 @@ EXPORTED_SYMBOLS = [
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
     "gllmq_quantized_matmul_noalloc",
-    "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_quant_gather", "gllmq_moe_route", "gllmq_set_option", "gllmq_last_kernel_name",
+    "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_lm_head_argmax", "gllmq_quant_gather", "gllmq_moe_route", "gllmq_set_option", "gllmq_last_kernel_name",
     "gllmq_reserve_matmul", "gllmq_reserve_ffn", "gllmq_reserve_moe", "gllmq_weights_forget", "gllmq_weight_uploads",
     "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
     "gllmq_gguf_open", "gllmq_gguf_parse", "gllmq_gguf_close", "gllmq_gguf_version", "gllmq_gguf_tensor_count",
@@ -393,6 +395,28 @@ class HipBackend:
                                     value.data_ptr() if value is not None else None, self._stream())
         if rc != OK:
             self._raise(rc, "argmax")
+
+    def lm_head_argmax(self, weight_blocks, input, quant_type, n: int, k: int, token, logits=None, value=None) -> None:
+        """The lm_head matvec of one activation row and the greedy token choice behind it as one
+        call: ``token[0]`` as ``argmax`` gives it on ``quantized_matmul``'s logits.  ``logits`` (device
+        f32, ``n`` entries) receives them; without it Q6_K / Q8_0 matrices never write them."""
+        w, x = weight_blocks, input
+        if not (_is_torch(w) and w.is_cuda and x.is_cuda and token.is_cuda and x.dtype == self._torch.float32
+                and token.element_size() == 4):
+            raise OtherError("lm_head_argmax: device tensors, f32 activations and a 32-bit integer token")
+        if not (w.is_contiguous() and x.is_contiguous()) or x.numel() < k or token.numel() < 1:
+            raise OtherError("lm_head_argmax: contiguous tensors of at least k activations and one token")
+        if logits is not None and not (logits.is_cuda and logits.dtype == self._torch.float32 and logits.is_contiguous()
+                                       and logits.numel() >= n):
+            raise OtherError("lm_head_argmax: logits must be a contiguous device f32 tensor of n entries")
+        if value is not None and not (value.is_cuda and value.dtype == self._torch.float32 and value.numel() >= 1):
+            raise OtherError("lm_head_argmax: value must be a device f32 tensor")
+        rc = self._lib.gllmq_lm_head_argmax(self._ctx, w.data_ptr(), w.numel() * w.element_size(), x.data_ptr(),
+                                            _dtype_id(quant_type), n, k, logits.data_ptr() if logits is not None else None,
+                                            token.data_ptr(), value.data_ptr() if value is not None else None,
+                                            self._stream())
+        if rc != OK:
+            self._raise(rc, "lm_head_argmax")
 
     def moe_route(self, logits, top_k: int, route_expert, route_weight, route_len, capacity_factor: float = 1.25,
                   route_pos=None, expert_counts=None, overflow=None) -> None:

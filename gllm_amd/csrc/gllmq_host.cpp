@@ -175,6 +175,7 @@ struct gllmq_ctx {
     hipFunction_t dequant_wave_q5k = nullptr;   // the same for Q5_K
     hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1], f32 multiply-add flavour
     hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
+    hipFunction_t gemv_i8_argmax[kNumFormats] = {}; // one row, ending in the candidates of the greedy token choice
     // int8 matrix-core kernels [Mm8Kind][pairs 1,2,4][early steps 1,2,4], and the same with
     // register-resident activation operands [Mm8Kind][pairs 1,2][early][passes per tile - 1]
     hipFunction_t mm8[MM8_KINDS][3][3] = {};
@@ -244,6 +245,7 @@ struct gllmq_ctx {
     hipFunction_t last_kernel = nullptr;
     int num_cus = 256;
     uint32_t gemv_waves = 2048; // waves a GEMV launch aims to put on the device
+    bool lm_head_fused = true;  // lm_head_argmax: candidates from the GEMV's own workgroups
     std::mutex err_mutex;
     std::string err;
 };
@@ -1133,6 +1135,9 @@ int gllmq_init(gllmq_ctx **out, int device)
             snprintf(name, sizeof name, "gq_gemv_i8_%s_m%d", kFormats[i].tag, m);
             rc = get_function(ctx, &ctx->gemv_i8[i][m - 1], name);
         }
+        if (rc != GLLMQ_OK) break;
+        snprintf(name, sizeof name, "gq_gemv_i8_%s_m1_argmax", kFormats[i].tag);
+        rc = get_function(ctx, &ctx->gemv_i8_argmax[i], name);
     }
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_route, "gq_moe_route");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[0], "gq_mmf_prep_t1");
@@ -1267,6 +1272,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "chain") ctx->use_chain = value != 0;
     else if (n == "chain_dependent") ctx->chain_dependent = value != 0;
     else if (n == "chain_spin_limit") ctx->chain_spin_limit = u;
+    else if (n == "lm_head_fused") ctx->lm_head_fused = value != 0;
     else if (n == "mmfs_all") ctx->mmfs_all = value != 0;
     else if (n == "mmfs_min_rows") ctx->mmfs_min_rows = std::max(1u, u);
     else if (n == "batch_overlap") ctx->batch_overlap = value != 0;
@@ -1385,6 +1391,57 @@ int gllmq_argmax(gllmq_ctx *ctx, const float *logits, size_t rows, size_t n, siz
         if (rc != GLLMQ_OK) return rc;
     }
     return GLLMQ_OK;
+}
+
+int gllmq_lm_head_argmax(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, uint32_t dtype, size_t n, size_t k,
+                         float *logits, uint32_t *token, float *value, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    if (!token) return fail(ctx, GLLMQ_ERR_INVALID, "lm_head_argmax: NULL token pointer");
+    if (!aligned(token, 4) || (value && !aligned(value, 4)))
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "lm_head_argmax: buffers must be 4-byte aligned");
+    if (n == 0) return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "lm_head_argmax: n = 0");
+    const Format *f = find_format(dtype);
+    // checked as the one-row matmul it is; without a logits buffer the activations stand in for it
+    int rc = check_matmul_args(ctx, f, w, w_bytes, x, logits ? logits : const_cast<float *>(x), dtype, 1, n, k);
+    if (rc >= 0) return rc;
+    Scratch *S = nullptr;
+    rc = acquire_scratch(ctx, stream, &S);
+    if (rc != GLLMQ_OK) return rc;
+    // The matvec whose workgroups leave their best candidate behind, where the one-row GEMV is the
+    // kernel such a matrix gets anyway (Q6_K and Q8_0, the types of GGUF output matrices) and one
+    // launch covers K; then the candidates, one per workgroup, to the token.
+    const size_t rb = gllmq_row_bytes(dtype, k);
+    const bool gemv_type = dtype == 14u || dtype == 8u;
+    if (ctx->lm_head_fused && gemv_type && !ctx->gemv_f32 && k <= 16384) {
+        GemvPlan L = plan_gemv(ctx, 1, static_cast<uint32_t>(n), static_cast<uint32_t>(k), rb, ctx->gemv_waves);
+        if (L.grid <= gq::ARGMAX_MAX_PARTS * gq::ARGMAX_MAX_ROWS) {
+            GemvParams &P = L.P;
+            P.w = static_cast<const uint8_t *>(w);
+            P.x = x;
+            P.y = logits;
+            P.ldx = static_cast<uint32_t>(k);
+            P.ldy = static_cast<uint32_t>(n);
+            P.x_vec = aligned(x, 16);
+            P.keys = S->argmax_keys;
+            rc = launch(ctx, ctx->gemv_i8_argmax[format_index(dtype)], L.grid, L.threads, L.lds, stream, &P, sizeof P);
+            if (rc != GLLMQ_OK) return rc;
+            ArgmaxParams A{};
+            A.keys = S->argmax_keys;
+            A.parts = L.grid;
+            A.token = token;
+            A.value = value;
+            return launch(ctx, ctx->argmax_final, 1, 256, 0, stream, &A, sizeof A);
+        }
+    }
+    if (!logits)
+        return fail(ctx, GLLMQ_ERR_UNIMPLEMENTED,
+                    "lm_head_argmax: this matrix (ggml dtype %u, k = %zu) goes through the matmul and the token choice one "
+                    "after the other, which needs a logits buffer of n floats", dtype, k);
+    rc = dispatch_matmul(ctx, *S, *f, static_cast<const uint8_t *>(w), x, logits, 1, n, k, false, stream);
+    if (rc != GLLMQ_OK) return rc;
+    return gllmq_argmax(ctx, logits, 1, n, n, token, value, stream);
 }
 
 int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y,

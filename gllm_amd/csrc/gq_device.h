@@ -32,6 +32,24 @@ __device__ __forceinline__ float round_to_bf16(float v)
 
 typedef uint32_t u4v __attribute__((ext_vector_type(4))); // plain 16-byte register quad
 
+// Candidates of the greedy token choice (argmax.hip.inc, and the GEMV that ends in it): the value
+// mapped to an unsigned number of the same order above its index; 0 = no candidate (NaN).
+__device__ __forceinline__ uint64_t argmax_key(float v, uint32_t idx)
+{
+    if (v != v) return 0ull;
+    v += 0.0f; // -0.0 becomes +0.0: the two compare equal in the reference
+    const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+    const uint32_t ord = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+    return (static_cast<uint64_t>(ord) << 32) | idx;
+}
+
+__device__ __forceinline__ float argmax_key_value(uint64_t key)
+{
+    const uint32_t ord = static_cast<uint32_t>(key >> 32);
+    const uint32_t bits = (ord & 0x80000000u) ? (ord & 0x7FFFFFFFu) : ~ord;
+    return __builtin_bit_cast(float, bits);
+}
+
 // Block fixed point: the powers of two that turn a group of activations whose largest magnitude
 // has the biased exponent `e_raw` (0 .. 254) into integers below 2^BITS and back.
 //   |x| < 2^(e-126)   ->   |x * pre * up| < 2^BITS,   down = 1 / (pre * up) = 2^(e - 126 - BITS)

@@ -31,6 +31,7 @@ struct GemvParams {
     uint32_t accumulate; // add to y instead of overwriting it (K handled in several launches)
     uint32_t prep_words; // integer-dot kernels: 32-bit words of LDS holding the prepared activations
     uint32_t act_bf16;   // integer-dot kernels: round activations to bf16 before use
+    uint64_t *keys;      // kernels that end in the greedy token choice: one candidate per workgroup (argmax_key)
 };
 
 struct Mm8Params {

@@ -169,6 +169,19 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_dev, const void *up_dev, s
 int gllmq_argmax(gllmq_ctx *ctx, const float *logits_dev, size_t rows, size_t n, size_t ld,
                  uint32_t *token_dev, float *value_dev, void *stream);
 
+/* ---- lm_head matvec and Op::Argmax as one call ---------------------------------------
+ * The tail of a decode step: the lm_head MatMul of one activation row (reached through
+ * Backend::quantized_matmul, src/compat/cpu_backend.rs:991-1049) followed by Op::Argmax
+ * (build_graph.inc.rs:2661).  w_dev is [n x k] of ggml_dtype, x_dev k f32; token_dev and
+ * value_dev as in gllmq_argmax (one row).  logits_dev (n f32) receives the logits; it may be
+ * NULL when only the token is wanted and the matrix is Q6_K or Q8_0 with k <= 16384: there
+ * every workgroup of the matvec leaves its best candidate behind and a one-workgroup launch
+ * picks among them, so the logits are neither written nor read again.  Other matrices run
+ * gllmq_quantized_matmul and gllmq_argmax one after the other and need logits_dev.  The
+ * logits and the token are those of the two calls made separately, bit for bit. */
+int gllmq_lm_head_argmax(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev, uint32_t ggml_dtype,
+                         size_t n, size_t k, float *logits_dev, uint32_t *token_dev, float *value_dev, void *stream);
+
 /* ---- Backend::quantized_matmul ----------------------------------------------------
  * y[m x n] = x[m x k] . W[n x k]^T.  w_bytes must be at least n * gllmq_row_bytes(dtype,k).
  * Alignment: w_dev 16 bytes for Q4_K/Q5_K, 2 bytes for Q6_K/Q8_0; x_dev 16, y_dev 4.

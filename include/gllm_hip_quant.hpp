@@ -156,6 +156,18 @@ public:
         return make(gllmq_argmax(ctx_, logits_dev, rows, n, ld, token_dev, value_dev, stream), "argmax");
     }
 
+    // The lm_head matvec of one row and Op::Argmax behind it as one call; logits_dev may be null
+    // for Q6_K / Q8_0 matrices with k <= 16384 (the logits then never reach memory).
+    BackendError lm_head_argmax_device(const void *w_dev, size_t w_bytes, const float *x_dev, QuantType t, size_t n, size_t k,
+                                       float *logits_dev, uint32_t *token_dev, float *value_dev = nullptr,
+                                       void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_lm_head_argmax(ctx_, w_dev, w_bytes, x_dev, static_cast<uint32_t>(t), n, k, logits_dev, token_dev,
+                                         value_dev, stream),
+                    "lm_head_argmax");
+    }
+
     // ExpertRouteTable::from_gate_logits over device buffers (src/moe/routing.rs:100-160; graph ops
     // MoEGate + TopK, build_graph.inc.rs:2064-2071); the optional outputs may be null.
     BackendError moe_route_device(const float *logits_dev, size_t tokens, size_t experts, size_t top_k,

@@ -81,6 +81,9 @@ extern "C" {
                             ffn: usize, relu_gate: c_int, stream: *mut c_void) -> c_int;
     pub fn gllmq_argmax(ctx: *mut gllmq_ctx, logits_dev: *const f32, rows: usize, n: usize, ld: usize,
                         token_dev: *mut u32, value_dev: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn gllmq_lm_head_argmax(ctx: *mut gllmq_ctx, w_dev: *const c_void, w_bytes: usize, x_dev: *const f32,
+                                ggml_dtype: u32, n: usize, k: usize, logits_dev: *mut f32, token_dev: *mut u32,
+                                value_dev: *mut f32, stream: *mut c_void) -> c_int;
     pub fn gllmq_quant_gather(ctx: *mut gllmq_ctx, table_dev: *const c_void, table_bytes: usize, ggml_dtype: u32,
                               vocab: usize, hidden: usize, ids_dev: *const u32, count: usize, scale: f32,
                               out_dev: *mut f32, stream: *mut c_void) -> c_int;
@@ -268,6 +271,19 @@ impl HipQuant {
     pub unsafe fn argmax_device(&self, logits: *const f32, rows: usize, n: usize, ld: usize, token: *mut u32,
                                 value: *mut f32, stream: *mut c_void) -> Result<(), QuantError> {
         self.check(gllmq_argmax(self.ctx, logits, rows, n, ld, token, value, stream), "argmax")
+    }
+
+    /// The lm_head matvec of one activation row and `Op::Argmax` behind it as one call.  `logits`
+    /// may be null for Q6_K / Q8_0 matrices with `k <= 16384`: the logits then never reach memory.
+    ///
+    /// # Safety
+    /// `w` must hold `w_bytes` bytes, `x` `k` f32, `logits` null or `n` f32, `token` one u32, `value`
+    /// null or one f32, all on this device.
+    pub unsafe fn lm_head_argmax_device(&self, w: *const c_void, w_bytes: usize, x: *const f32, ggml_dtype: u32, n: usize,
+                                        k: usize, logits: *mut f32, token: *mut u32, value: *mut f32,
+                                        stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_lm_head_argmax(self.ctx, w, w_bytes, x, ggml_dtype, n, k, logits, token, value, stream),
+                   "lm_head_argmax")
     }
 
     /// The same lookup with host slices (table uploaded, rows downloaded).

@@ -110,6 +110,74 @@ def test_lm_head_then_argmax(hip, torch, oracle):
         assert want[r, t] >= want[r].max() - 2e-3 * np.abs(want[r]).max()
 
 
+@pytest.mark.parametrize("dt,n,k", [(14, 32000, 2048), (14, 128256, 4096), (14, 1000, 8192), (14, 37, 256), (8, 5000, 1024),
+                                     (8, 777, 12288), (12, 32000, 2048), (13, 3000, 1024), (14, 300, 16640)])
+def test_lm_head_and_token_in_one_call(hip, torch, oracle, dt, n, k):
+    """gllmq_lm_head_argmax against the two calls it stands for: the same logits and the same token bit
+    for bit, with and without a logits buffer (Q6_K and Q8_0 within one launch of K never write
+    them; other matrices need the buffer), and the token against the oracle's choice on its own logits."""
+    from gllm_amd.backend import BackendError
+    from gllm_amd.synth import random_activations, random_weight
+    print(f"lm_head_argmax dtype={dt} n={n} k={k}", flush=True)
+    w, x = random_weight(dt, n, k, seed=n), random_activations(1, k, seed=k)
+    wd = torch.from_numpy(np.asarray(w).view(np.uint8).reshape(-1)).cuda()
+    xd = torch.from_numpy(x).cuda()
+    y = torch.empty(1, n, device="cuda")
+    tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+    val = torch.zeros(1, device="cuda")
+    hip.quantized_matmul(wd, xd, y, dt, 1, n, k)
+    hip.argmax(y, tok, val)
+    torch.cuda.synchronize()
+    y2 = torch.full((n + 64,), NAN, device="cuda")
+    tok2 = torch.full((4,), 12345, dtype=torch.int32, device="cuda")
+    val2 = torch.full((4,), 7.0, device="cuda")
+    hip.lm_head_argmax(wd, xd, dt, n, k, tok2[:1], logits=y2[:n], value=val2[:1])
+    torch.cuda.synchronize()
+    assert torch.equal(y2[:n], y[0]) and bool(torch.all(torch.isnan(y2[n:])))
+    assert int(tok2[0]) == int(tok[0]) and float(val2[0]) == float(val[0])
+    assert tok2[1:].tolist() == [12345] * 3 and val2[1:].tolist() == [7.0] * 3
+    tok3 = torch.full((1,), 777, dtype=torch.int32, device="cuda")
+    if dt in (14, 8) and k <= 16384:
+        hip.lm_head_argmax(wd, xd, dt, n, k, tok3)
+        torch.cuda.synchronize()
+        assert int(tok3[0]) == int(tok[0])
+    else:
+        with pytest.raises(BackendError):
+            hip.lm_head_argmax(wd, xd, dt, n, k, tok3)
+    yh = y.cpu().numpy()[0]
+    assert oracle.argmax_token(yh) == int(tok[0])
+    want = oracle.quantized_matmul(w, x, dt, 1, n, k, acc=oracle.ACC_F64, threads=8)[0]
+    assert want[int(tok[0])] >= want.max() - 2e-3 * np.abs(want).max()
+
+
+def test_lm_head_token_with_ties_and_nan(hip, torch, oracle):
+    """Rows of equal weights give equal logits (the LAST of them is the token), and a NaN activation
+    leaves no candidate at all."""
+    from gllm_amd.synth import random_activations, random_weight
+    print("lm_head_argmax ties and NaN", flush=True)
+    dt, n, k = 14, 4000, 1024
+    w = np.asarray(random_weight(dt, n, k, seed=1)).view(np.uint8).reshape(n, -1).copy()
+    x = random_activations(1, k, seed=2)
+    first = oracle.quantized_matmul(w.reshape(-1), x, dt, 1, n, k, acc=oracle.ACC_F64, threads=4)[0]
+    top = int(np.argmax(first))
+    for r in (5, 1999, 3998):  # copies of the winning row, in different workgroups
+        w[r] = w[top]
+    wd = torch.from_numpy(w.reshape(-1)).cuda()
+    tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+    val = torch.zeros(1, device="cuda")
+    hip.lm_head_argmax(wd, torch.from_numpy(x).cuda(), dt, n, k, tok, value=val)
+    torch.cuda.synchronize()
+    assert int(tok[0]) == max(top, 3998)
+    xn = x.copy()
+    xn[0, 100] = NAN
+    hip.lm_head_argmax(wd, torch.from_numpy(xn).cuda(), dt, n, k, tok, value=val)
+    torch.cuda.synchronize()
+    y = torch.empty(1, n, device="cuda")
+    hip.quantized_matmul(wd, torch.from_numpy(xn).cuda(), y, dt, 1, n, k)
+    want = oracle.argmax_token(y.cpu().numpy()[0])
+    assert (int(tok[0]) & 0xFFFFFFFF) == (NONE if want is None else want)
+
+
 def test_argument_errors(hip, torch):
     from gllm_amd.backend import BackendError
     print("argmax errors", flush=True)
