@@ -28,6 +28,7 @@ ACT_F32_SPLIT, ACT_BF16 = 0, 1
 DESC_AFTER_PREVIOUS = 1  # gllmq_matmul_desc.flags: the entry depends on the entries before it
 
 
+ELEM_F32, ELEM_F16, ELEM_BF16 = 0, 1, 2  # gllmq_quantized_matmul_elem: element type of activations and outputs
 ARGMAX_NONE = 0xFFFFFFFF  # gllmq_argmax: the row has no entry that is not NaN
 
 
@@ -119,6 +120,10 @@ def load_library() -> C.CDLL:
     L.gllmq_ffn_swiglu.argtypes = [vp, vp, vp, sz, u32, vp, sz, u32, vp, vp, sz, sz, sz, C.c_int, vp]
     L.gllmq_argmax.restype = C.c_int
     L.gllmq_argmax.argtypes = [vp, vp, sz, sz, sz, vp, vp, vp]
+    L.gllmq_quantized_matmul_elem.restype = C.c_int
+    L.gllmq_quantized_matmul_elem.argtypes = [vp, vp, sz, vp, vp, C.c_uint32, sz, sz, sz, C.c_int, vp]
+    L.gllmq_reserve_matmul_elem.restype = C.c_int
+    L.gllmq_reserve_matmul_elem.argtypes = [vp, C.c_uint32, sz, sz, sz, C.c_int, vp]
     L.gllmq_lm_head_argmax.restype = C.c_int
     L.gllmq_lm_head_argmax.argtypes = [vp, vp, sz, vp, C.c_uint32, sz, sz, vp, vp, vp, vp]
     L.gllmq_dequantize_host.restype = C.c_int
@@ -136,7 +141,7 @@ EXPORTED_SYMBOLS = [
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
     "gllmq_quantized_matmul_noalloc",
-    "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_lm_head_argmax", "gllmq_quant_gather", "gllmq_moe_route", "gllmq_set_option", "gllmq_last_kernel_name",
+    "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_lm_head_argmax", "gllmq_quantized_matmul_elem", "gllmq_reserve_matmul_elem", "gllmq_quant_gather", "gllmq_moe_route", "gllmq_set_option", "gllmq_last_kernel_name",
     "gllmq_reserve_matmul", "gllmq_reserve_ffn", "gllmq_reserve_moe", "gllmq_weights_forget", "gllmq_weight_uploads",
     "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
     "gllmq_gguf_open", "gllmq_gguf_parse", "gllmq_gguf_close", "gllmq_gguf_version", "gllmq_gguf_tensor_count",
@@ -201,8 +206,8 @@ class HipBackend:
         ptr = None if host_array is None else _host_bytes(host_array).ctypes.data
         self._lib.gllmq_weights_forget(self._ctx, ptr)
 
-    def reserve_matmul(self, quant_type, m: int, n: int, k: int) -> None:
-        rc = self._lib.gllmq_reserve_matmul(self._ctx, _dtype_id(quant_type), m, n, k, self._stream())
+    def reserve_matmul(self, quant_type, m: int, n: int, k: int, elem: int = ELEM_F32) -> None:
+        rc = self._lib.gllmq_reserve_matmul_elem(self._ctx, _dtype_id(quant_type), m, n, k, elem, self._stream())
         if rc != OK:
             self._raise(rc, "reserve_matmul")
 
@@ -255,15 +260,23 @@ class HipBackend:
             w, x, y = weight_blocks, input, output
             if not (w.is_cuda and x.is_cuda and y.is_cuda):
                 raise OtherError("quantized_matmul: tensors must live on the GPU")
-            if x.dtype != self._torch.float32 or y.dtype != self._torch.float32:
-                raise Unimplemented("quantized_matmul: activations and outputs are f32 on this backend")
+            elem = self._elem_of(x.dtype)
+            if elem is None or y.dtype != x.dtype:
+                raise Unimplemented("quantized_matmul: activations and outputs are f32, f16 or bf16, both of one type")
             if not (w.is_contiguous() and x.is_contiguous() and y.is_contiguous()):
                 raise OtherError("quantized_matmul: tensors must be contiguous")
             if x.numel() < m * k or y.numel() < m * n:
                 raise OtherError("quantized_matmul: input/output shorter than m*k / m*n")
-            rc = self._lib.gllmq_quantized_matmul_ex(
-                self._ctx, w.data_ptr(), w.numel() * w.element_size(), x.data_ptr(), y.data_ptr(),
-                dt, m, n, k, act_mode, self._stream())
+            if elem != ELEM_F32:
+                if act_mode != ACT_F32_SPLIT:
+                    raise Unimplemented("quantized_matmul: the bf16 activation mode is for f32 tensors")
+                rc = self._lib.gllmq_quantized_matmul_elem(
+                    self._ctx, w.data_ptr(), w.numel() * w.element_size(), x.data_ptr(), y.data_ptr(),
+                    dt, m, n, k, elem, self._stream())
+            else:
+                rc = self._lib.gllmq_quantized_matmul_ex(
+                    self._ctx, w.data_ptr(), w.numel() * w.element_size(), x.data_ptr(), y.data_ptr(),
+                    dt, m, n, k, act_mode, self._stream())
         else:
             w = _host_bytes(weight_blocks)
             x = np.ascontiguousarray(input, np.float32).reshape(-1)
@@ -275,6 +288,11 @@ class HipBackend:
                 self._ctx, w.ctypes.data, w.size, x.ctypes.data, output.ctypes.data, dt, m, n, k)
         if rc != OK:
             self._raise(rc, "quantized_matmul")
+
+    def _elem_of(self, torch_dtype):
+        """Backend<E>: the element types the reference instantiates (src/compat/mod.rs:376-378)."""
+        t = self._torch
+        return {t.float32: ELEM_F32, t.float16: ELEM_F16, t.bfloat16: ELEM_BF16}.get(torch_dtype)
 
     def quantized_matmul_noalloc(self, weight_blocks, input, output, quant_type, m: int, n: int, k: int) -> None:
         """``quantized_matmul`` on device tensors through the entry point that allocates nothing

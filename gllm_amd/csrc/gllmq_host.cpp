@@ -18,6 +18,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <type_traits>
 #include <unordered_map>
 #include <vector>
 
@@ -142,6 +143,8 @@ struct Scratch {
     size_t ffn_bytes = 0;
     void *moe = nullptr;         // gllmq_moe_matvec: pair tables, jobs, intermediate activations
     size_t moe_bytes = 0;
+    void *elem = nullptr;        // 16-bit activations and outputs as f32, for the kernels that do not convert themselves
+    size_t elem_bytes = 0;
 };
 
 constexpr size_t kScratchArriveBytes = 4096; // MM8_SPLIT_MAX_LISTS words, padded; the chain kernel's counters behind them
@@ -246,6 +249,9 @@ struct gllmq_ctx {
     int num_cus = 256;
     uint32_t gemv_waves = 2048; // waves a GEMV launch aims to put on the device
     bool lm_head_fused = true;  // lm_head_argmax: candidates from the GEMV's own workgroups
+    uint32_t call_elem = 0;     // element type of x and y of the matmul being enqueued (call_mutex held); 0 = f32
+    bool elem_fused = true;     // "elem_fused" = 0: 16-bit elements always through conversion launches
+    hipFunction_t convert_elem = nullptr;
     std::mutex err_mutex;
     std::string err;
 };
@@ -325,6 +331,7 @@ void free_scratch(Scratch &S)
     if (S.mmf) (void)hipFree(S.mmf);
     if (S.ffn) (void)hipFree(S.ffn);
     if (S.moe) (void)hipFree(S.moe);
+    if (S.elem) (void)hipFree(S.elem);
     S = Scratch{};
 }
 
@@ -430,6 +437,15 @@ int launch(gllmq_ctx *ctx, hipFunction_t f, uint32_t grid, uint32_t block, uint3
 
 bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
+// Element `index` of activations or outputs whose element type is that of the call being enqueued
+// (pointers are typed for the f32 case).
+template <class T>
+T *elem_at(const gllmq_ctx *ctx, T *base, size_t index)
+{
+    typedef typename std::conditional<std::is_const<T>::value, const uint8_t, uint8_t>::type Byte;
+    return reinterpret_cast<T *>(reinterpret_cast<Byte *>(base) + index * (ctx->call_elem ? 2u : 4u));
+}
+
 // Shape-dependent fields of a GEMV launch over at most 64 groups (16384 elements) of K and
 // m <= 2: how a row is split over lanes and waves, rows per workgroup, LDS.  `target_waves`
 // is the number of waves the launch aims to put on the device.
@@ -486,6 +502,7 @@ int launch_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, size_t row_by
     P.x_vec = aligned(x, 16) && (m == 1 || ldx % 4 == 0);
     P.accumulate = accumulate ? 1u : 0u;
     P.act_bf16 = act_bf16 ? 1u : 0u;
+    P.elem = ctx->call_elem;
     const int fi = format_index(f.dtype);
     hipFunction_t fn = ctx->gemv_f32 ? ctx->gemv[fi][m - 1] : ctx->gemv_i8[fi][m - 1];
     return launch(ctx, fn, L.grid, L.threads, L.lds, stream, &P, sizeof P);
@@ -591,6 +608,7 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     P.tiles = tiles;
     P.grid = grid;
     P.act_bf16 = act_bf16 ? 1u : 0u;
+    P.elem = ctx->call_elem;
     P.xrows = ctx->identity_rows;
     P.rows_per_wg = rows_per_wg;
     P.tile_rows = tile_rows;
@@ -690,8 +708,9 @@ int run_mm8(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         P.w2 = w2;
         P.glu_relu = glu_relu ? 1u : 0u;
         P.w = w;
-        P.x = x + m0 * k;
-        P.y = y + m0 * n;
+        P.elem = ctx->call_elem;
+        P.x = elem_at(ctx, x, m0 * k);
+        P.y = elem_at(ctx, y, m0 * n);
         P.n = static_cast<uint32_t>(n);
         P.k = static_cast<uint32_t>(k);
         P.groups = groups;
@@ -750,7 +769,7 @@ MmfPlan plan_mmf(const gllmq_ctx *ctx, size_t m, size_t n, size_t k)
 int run_mmf(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
             size_t k, bool act_bf16, void *stream, size_t min_m = 9)
 {
-    if (!ctx->use_mmf || m < min_m) return -1;
+    if (!ctx->use_mmf || m < min_m || ctx->call_elem) return -1;
     const int fmt = f.dtype == T_Q8_0 ? 3 : f.dtype == T_Q6_K ? 2 : f.dtype == T_Q5_K ? 1 : 0;
     if (fmt == 3 && k < 256) return -1; // the Q8_0 fetch window is one whole group of 8 blocks
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
@@ -855,7 +874,7 @@ MmfsPlan plan_mmfs(const gllmq_ctx *ctx, const Format &f, size_t m, size_t n, si
 int run_mmfs(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
              size_t k, bool act_bf16, void *stream, size_t min_m = 9)
 {
-    if (m < min_m) return -1;
+    if (m < min_m || ctx->call_elem) return -1;
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
     const MmfsPlan L = plan_mmfs(ctx, f, m, n, k);
     if (!L.ok) return -1;
@@ -993,7 +1012,7 @@ int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(2, m - m0));
         for (size_t k0 = 0; k0 < k; k0 += kChunk) {
             const size_t kk = std::min(kChunk, k - k0);
-            int rc = launch_gemv(ctx, f, w + (k0 / 256) * f.group_bytes, rb, x + m0 * k + k0, y + m0 * n, mm,
+            int rc = launch_gemv(ctx, f, w + (k0 / 256) * f.group_bytes, rb, elem_at(ctx, x, m0 * k + k0), elem_at(ctx, y, m0 * n), mm,
                                  static_cast<uint32_t>(n), static_cast<uint32_t>(kk), static_cast<uint32_t>(k),
                                  static_cast<uint32_t>(n), k0 != 0, act_bf16, stream);
             if (rc != GLLMQ_OK) return rc;
@@ -1140,6 +1159,7 @@ int gllmq_init(gllmq_ctx **out, int device)
         rc = get_function(ctx, &ctx->gemv_i8_argmax[i], name);
     }
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_route, "gq_moe_route");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->convert_elem, "gq_convert_elem");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[0], "gq_mmf_prep_t1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep[1], "gq_mmf_prep_t2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmf_prep_lanes, "gq_mmf_prep_lanes");
@@ -1273,6 +1293,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "chain_dependent") ctx->chain_dependent = value != 0;
     else if (n == "chain_spin_limit") ctx->chain_spin_limit = u;
     else if (n == "lm_head_fused") ctx->lm_head_fused = value != 0;
+    else if (n == "elem_fused") ctx->elem_fused = value != 0;
     else if (n == "mmfs_all") ctx->mmfs_all = value != 0;
     else if (n == "mmfs_min_rows") ctx->mmfs_min_rows = std::max(1u, u);
     else if (n == "batch_overlap") ctx->batch_overlap = value != 0;
@@ -1453,6 +1474,73 @@ int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w, size_t w_bytes, con
     int rc = acquire_scratch(ctx, stream, &S);
     if (rc != GLLMQ_OK) return rc;
     return matmul_on_scratch(ctx, *S, w, w_bytes, x, y, dtype, m, n, k, act_mode, stream);
+}
+
+namespace {
+
+int convert_elems(gllmq_ctx *ctx, const void *src, void *dst, size_t count, uint32_t elem, bool widen, void *stream)
+{
+    gq::ConvertParams C{};
+    C.src = src;
+    C.dst = dst;
+    C.count = count;
+    C.elem = elem;
+    C.widen = widen ? 1u : 0u;
+    const uint32_t grid = static_cast<uint32_t>(std::min<size_t>((count + 255) / 256, 4096));
+    return launch(ctx, ctx->convert_elem, std::max(1u, grid), 256, 0, stream, &C, sizeof C, true);
+}
+
+size_t elem_scratch_bytes(size_t m, size_t n, size_t k) { return ((m * k * 4 + 255) & ~size_t(255)) + m * n * 4; }
+
+// Whether the kernels that convert 16-bit elements in their own loads and stores take the shape:
+// the int8 and integer-dot kernels of up to 8 rows, within one launch of K.
+bool elem_in_kernel(const gllmq_ctx *ctx, size_t m, size_t k) { return ctx->elem_fused && !ctx->gemv_f32 && m <= 8 && k <= 16384; }
+
+} // namespace
+
+int gllmq_quantized_matmul_elem(gllmq_ctx *ctx, const void *w, size_t w_bytes, const void *x, void *y, uint32_t dtype,
+                                size_t m, size_t n, size_t k, int elem, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    if (elem == GLLMQ_ELEM_F32)
+        return gllmq_quantized_matmul_ex(ctx, w, w_bytes, static_cast<const float *>(x), static_cast<float *>(y), dtype, m, n,
+                                         k, GLLMQ_ACT_F32_SPLIT, stream);
+    if (elem != GLLMQ_ELEM_F16 && elem != GLLMQ_ELEM_BF16)
+        return fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul_elem: unknown element type %d", elem);
+    const Format *f = find_format(dtype);
+    int rc = check_matmul_args(ctx, f, w, w_bytes, static_cast<const float *>(x), static_cast<float *>(y), dtype, m, n, k);
+    if (rc >= 0) return rc;
+    Scratch *S = nullptr;
+    rc = acquire_scratch(ctx, stream, &S);
+    if (rc != GLLMQ_OK) return rc;
+    if (elem_in_kernel(ctx, m, k)) {
+        ctx->call_elem = static_cast<uint32_t>(elem);
+        rc = dispatch_matmul(ctx, *S, *f, static_cast<const uint8_t *>(w), static_cast<const float *>(x),
+                             static_cast<float *>(y), m, n, k, false, stream);
+        ctx->call_elem = 0;
+        return rc;
+    }
+    rc = grow_scratch(ctx, *S, &S->elem, &S->elem_bytes, elem_scratch_bytes(m, n, k), stream, "quantized_matmul_elem");
+    if (rc != GLLMQ_OK) return rc;
+    float *xf = static_cast<float *>(S->elem);
+    float *yf = reinterpret_cast<float *>(static_cast<uint8_t *>(S->elem) + ((m * k * 4 + 255) & ~size_t(255)));
+    rc = convert_elems(ctx, x, xf, m * k, static_cast<uint32_t>(elem), true, stream);
+    if (rc == GLLMQ_OK) rc = dispatch_matmul(ctx, *S, *f, static_cast<const uint8_t *>(w), xf, yf, m, n, k, false, stream);
+    if (rc == GLLMQ_OK) rc = convert_elems(ctx, yf, y, m * n, static_cast<uint32_t>(elem), false, stream);
+    return rc;
+}
+
+int gllmq_reserve_matmul_elem(gllmq_ctx *ctx, uint32_t dtype, size_t m, size_t n, size_t k, int elem, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    int rc = gllmq_reserve_matmul(ctx, dtype, m, n, k, stream);
+    if (rc != GLLMQ_OK || elem == GLLMQ_ELEM_F32 || m == 0 || n == 0 || k == 0 || elem_in_kernel(ctx, m, k)) return rc;
+    Scratch *S = nullptr;
+    rc = acquire_scratch(ctx, stream, &S);
+    if (rc != GLLMQ_OK) return rc;
+    return grow_scratch(ctx, *S, &S->elem, &S->elem_bytes, elem_scratch_bytes(m, n, k), stream, "reserve_matmul_elem");
 }
 
 int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_t gate_up_bytes_each, uint32_t dtype_gate_up,

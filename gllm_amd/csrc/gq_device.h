@@ -32,6 +32,52 @@ __device__ __forceinline__ float round_to_bf16(float v)
 
 typedef uint32_t u4v __attribute__((ext_vector_type(4))); // plain 16-byte register quad
 
+// Element types of activations and outputs at the boundary (Backend<E>, E in {f32, f16, bf16},
+// src/compat/mod.rs:376-378).  16-bit elements widen exactly on the way in; results are rounded to
+// the nearest element, ties to even, on the way out (half::f16 / half::bf16 ::from_f32, the
+// conversions of src/compat/jit_helpers.rs:35-50), NaN stays NaN.
+constexpr uint32_t ELEM_F32 = 0, ELEM_F16 = 1, ELEM_BF16 = 2;
+
+__device__ __forceinline__ float elem16_to_f32(uint32_t bits, uint32_t elem)
+{
+    return elem == ELEM_F16 ? f16_bits_to_f32(bits) : __builtin_bit_cast(float, bits << 16);
+}
+
+__device__ __forceinline__ uint16_t f32_to_elem16(float v, uint32_t elem)
+{
+    if (elem == ELEM_F16) return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
+    const uint32_t b = __builtin_bit_cast(uint32_t, v);
+    if ((b & 0x7FFFFFFFu) > 0x7F800000u) return static_cast<uint16_t>((b >> 16) | 0x0040u); // NaN, made quiet
+    return static_cast<uint16_t>((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
+}
+
+// y[idx] of an output whose elements are of type `elem` (y is typed for the f32 case)
+__device__ __forceinline__ void store_elem(float *y, size_t idx, float v, uint32_t elem)
+{
+    if (elem == ELEM_F32) y[idx] = v;
+    else reinterpret_cast<uint16_t *>(y)[idx] = f32_to_elem16(v, elem);
+}
+
+// Eight consecutive activations from element `idx` on (16-byte aligned for f32 and for 16-bit
+// elements alike: two quads or one).
+__device__ __forceinline__ void load_elem8(const float *x, size_t idx, uint32_t elem, float (&v)[8])
+{
+    if (elem == ELEM_F32) {
+        const float4 a = *reinterpret_cast<const float4 *>(x + idx);
+        const float4 c = *reinterpret_cast<const float4 *>(x + idx + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = c.x; v[5] = c.y; v[6] = c.z; v[7] = c.w;
+    } else {
+        const uint4 t = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(x) + idx);
+        const uint32_t w[4] = { t.x, t.y, t.z, t.w };
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = elem16_to_f32(w[i] & 0xFFFFu, elem);
+            v[2 * i + 1] = elem16_to_f32(w[i] >> 16, elem);
+        }
+    }
+}
+
 // Candidates of the greedy token choice (argmax.hip.inc, and the GEMV that ends in it): the value
 // mapped to an unsigned number of the same order above its index; 0 = no candidate (NaN).
 __device__ __forceinline__ uint64_t argmax_key(float v, uint32_t idx)

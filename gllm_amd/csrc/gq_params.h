@@ -31,6 +31,7 @@ struct GemvParams {
     uint32_t accumulate; // add to y instead of overwriting it (K handled in several launches)
     uint32_t prep_words; // integer-dot kernels: 32-bit words of LDS holding the prepared activations
     uint32_t act_bf16;   // integer-dot kernels: round activations to bf16 before use
+    uint32_t elem;       // integer-dot kernels: element type of x and y (ELEM_F32 / ELEM_F16 / ELEM_BF16)
     uint64_t *keys;      // kernels that end in the greedy token choice: one candidate per workgroup (argmax_key)
 };
 
@@ -56,6 +57,7 @@ struct Mm8Params {
     // row and writes its sums to part[s][m][n]; the one that finishes last adds the slices up in
     // order (arrive[tile list] counts the finished ones and is left at 0).
     uint32_t ksplit, kslice_groups;
+    uint32_t elem;      // element type of x and y (ELEM_F32 / ELEM_F16 / ELEM_BF16); the slice sums stay f32
     float *part;
     uint32_t *arrive;
     // streamed kernels (mm8s.hip.inc) only, all worked out by the host so that a loader wave's
@@ -300,6 +302,14 @@ struct GluActParams {
     const float *u; // up results, row r at u + r * ld
     float *h;       // [m][ffn]
     uint32_t m, ffn, ld, relu_gate;
+};
+
+struct ConvertParams {
+    const void *src;
+    void *dst;
+    uint64_t count;  // elements
+    uint32_t elem;   // the 16-bit type (ELEM_F16 / ELEM_BF16)
+    uint32_t widen;  // 1: 16-bit -> f32, 0: f32 -> 16-bit
 };
 
 struct ArgmaxParams {

@@ -13,3 +13,4 @@
 #include "argmax.hip.inc"
 #include "ffn.hip.inc"
 #include "route.hip.inc"
+#include "convert.hip.inc"

@@ -169,6 +169,24 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_dev, const void *up_dev, s
 int gllmq_argmax(gllmq_ctx *ctx, const float *logits_dev, size_t rows, size_t n, size_t ld,
                  uint32_t *token_dev, float *value_dev, void *stream);
 
+/* ---- Backend<E>::quantized_matmul for E = f16 and bf16 -------------------------------
+ * The reference's backend trait is generic over the element type of activations and outputs
+ * (Backend<E: Element>, f32 / half::f16 / half::bf16: src/compat/mod.rs:376-378;
+ * quantized_matmul takes input: &[E] and output: &mut [E], src/compat/mod.rs:233-246).
+ * x_dev holds m x k and y_dev m x n elements of type `elem`; 16-bit activations widen exactly,
+ * the arithmetic is that of gllmq_quantized_matmul, and a result is rounded to the nearest
+ * element, ties to even (what E::from_f32 does; NaN stays NaN, f16 overflows to infinity): y is
+ * bit for bit the rounded result of the f32 call on the widened activations.  Up to 8 rows with
+ * k <= 16384 the kernels convert in their own loads and stores; other shapes take a widening and
+ * a rounding launch around the f32 kernels, through scratch of the stream
+ * (gllmq_reserve_matmul_elem before capturing such a shape).  Both pointers 4-byte aligned. */
+#define GLLMQ_ELEM_F32 0
+#define GLLMQ_ELEM_F16 1
+#define GLLMQ_ELEM_BF16 2
+int gllmq_quantized_matmul_elem(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const void *x_dev, void *y_dev,
+                                uint32_t ggml_dtype, size_t m, size_t n, size_t k, int elem, void *stream);
+int gllmq_reserve_matmul_elem(gllmq_ctx *ctx, uint32_t ggml_dtype, size_t m, size_t n, size_t k, int elem, void *stream);
+
 /* ---- lm_head matvec and Op::Argmax as one call ---------------------------------------
  * The tail of a decode step: the lm_head MatMul of one activation row (reached through
  * Backend::quantized_matmul, src/compat/cpu_backend.rs:991-1049) followed by Op::Argmax

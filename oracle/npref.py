@@ -154,6 +154,34 @@ def bf16_rne(a: np.ndarray) -> np.ndarray:
     return r.astype(np.uint32).view(np.float32)
 
 
+ELEM_F32, ELEM_F16, ELEM_BF16 = 0, 1, 2
+
+
+def elem_bits_to_f32(bits: np.ndarray, elem: int) -> np.ndarray:
+    """Activations of a 16-bit element type (their bit patterns) as float32: exact in both types
+    (half::f16::to_f32 / half::bf16::to_f32, the Element conversions behind Backend<E>,
+    src/compat/mod.rs:376-378 and src/compat/jit_helpers.rs:35-50 of the reference)."""
+    b = np.asarray(bits, np.uint16)
+    if elem == ELEM_F16:
+        return b.view(np.float16).astype(np.float32)
+    return (b.astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_elem_bits(y: np.ndarray, elem: int) -> np.ndarray:
+    """float32 results as bit patterns of a 16-bit element type: nearest, ties to even
+    (E::from_f32); f16 through numpy's IEEE conversion, bf16 through bf16_rne above (known answers
+    1.0 -> 0x3F80, -1.0 -> 0xBF80, src/compat/weight_helpers.rs:1202-1215).  NaN patterns are
+    whatever the conversion leaves: compare them as NaN, not bit for bit."""
+    v = np.asarray(y, np.float32)
+    if elem == ELEM_F16:
+        with np.errstate(over="ignore"):
+            return v.astype(np.float16).view(np.uint16)
+    out = (bf16_rne(v).view(np.uint32) >> 16).astype(np.uint16)
+    nan = np.isnan(v)
+    out[nan] = ((v.view(np.uint32)[nan] >> 16) | 0x40).astype(np.uint16)
+    return out
+
+
 def softmax(logits: np.ndarray) -> np.ndarray:
     z = np.asarray(logits, np.float32)
     e = np.exp(z - z.max())

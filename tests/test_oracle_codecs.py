@@ -61,6 +61,30 @@ def test_bf16_rounding_known_answers_and_torch(oracle):
     assert np.array_equal(npref.bf16_rne(v).view(np.uint32) >> 16, want.astype(np.uint32))
 
 
+def test_element_type_conversions_against_torch_and_known_answers():
+    """The 16-bit element types at the boundary: widening is exact, narrowing is nearest-even,
+    checked against torch's conversions (an independent implementation), the reference's known
+    answers and hand-built ties."""
+    import torch
+    rng = np.random.default_rng(3)
+    v = np.concatenate([rng.standard_normal(4000).astype(np.float32) * np.float32(100.0),
+                        np.array([0.0, -0.0, 1.0, -1.0, 65504.0, 65519.9, 65520.0, 1e-8, 6e-8, 2.98e-8, 2.9802325e-8,
+                                  1.00048828125, 1.00146484375, 1.00390625, 1.01171875, 3.3895314e38, 3.4e38, 1e-40,
+                                  np.inf, -np.inf], np.float32)])
+    t = torch.from_numpy(v)
+    for elem, tt in ((npref.ELEM_F16, torch.float16), (npref.ELEM_BF16, torch.bfloat16)):
+        bits = npref.f32_to_elem_bits(v, elem)
+        assert np.array_equal(bits, t.to(tt).view(torch.int16).numpy().view(np.uint16)), elem
+        back = npref.elem_bits_to_f32(bits, elem)
+        assert np.array_equal(back.view(np.uint32), t.to(tt).to(torch.float32).numpy().view(np.uint32)), elem
+    bf = npref.f32_to_elem_bits(np.array([1.0, -1.0, 1.00390625, 1.01171875], np.float32), npref.ELEM_BF16)
+    assert bf.tolist() == [0x3F80, 0xBF80, 0x3F80, 0x3F82]  # the two ties go to the even neighbour
+    hf = npref.f32_to_elem_bits(np.array([1.0, 1.00048828125, 1.00146484375, 65520.0, 2.9802322e-8], np.float32), npref.ELEM_F16)
+    assert hf.tolist() == [0x3C00, 0x3C00, 0x3C02, 0x7C00, 0x0000]
+    assert np.all(np.isnan(npref.elem_bits_to_f32(npref.f32_to_elem_bits(np.array([np.nan], np.float32), npref.ELEM_BF16),
+                                                   npref.ELEM_BF16)))
+
+
 def test_scale_min_k4_inverts_the_quantizer_packing(oracle):
     rng = np.random.default_rng(7)
     for _ in range(200):
