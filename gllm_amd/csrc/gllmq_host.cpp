@@ -769,7 +769,7 @@ MmfPlan plan_mmf(const gllmq_ctx *ctx, size_t m, size_t n, size_t k)
 int run_mmf(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
             size_t k, bool act_bf16, void *stream, size_t min_m = 9)
 {
-    if (!ctx->use_mmf || m < min_m || ctx->call_elem) return -1;
+    if (!ctx->use_mmf || m < min_m) return -1;
     const int fmt = f.dtype == T_Q8_0 ? 3 : f.dtype == T_Q6_K ? 2 : f.dtype == T_Q5_K ? 1 : 0;
     if (fmt == 3 && k < 256) return -1; // the Q8_0 fetch window is one whole group of 8 blocks
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
@@ -786,8 +786,9 @@ int run_mmf(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         const uint32_t mt = mm <= 32 ? 1u : 2u;
         MmfParams P{};
         P.w = w;
-        P.x = x + m0 * k;
-        P.y = y + m0 * n;
+        P.elem = ctx->call_elem;
+        P.x = elem_at(ctx, x, m0 * k);
+        P.y = elem_at(ctx, y, m0 * n);
         P.ximg = static_cast<uint8_t *>(S.mmf);
         P.partial = reinterpret_cast<float *>(static_cast<uint8_t *>(S.mmf) + img_bytes);
         P.n = static_cast<uint32_t>(n);
@@ -801,13 +802,13 @@ int run_mmf(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         P.ksplit = ksplit;
         P.blocks_per_split = bps;
         P.act_bf16 = act_bf16 ? 1u : 0u;
-        MmfPrepParams Q{ P.x, P.ximg, mm, P.k, P.ldx, P.act_bf16 };
+        MmfPrepParams Q{ P.x, P.ximg, mm, P.k, P.ldx, P.act_bf16, P.elem };
         int rc = launch2d(ctx, ctx->mmf_prep[mt - 1], groups, 16, 64, 0, stream, &Q, sizeof Q, true);
         if (rc != GLLMQ_OK) return rc;
         rc = launch(ctx, ctx->mmf_q4k[fmt][mt - 1][act_bf16 ? 1 : 0], row_tiles * ksplit, 512, mmf_lds_bytes(mt, fmt), stream,
                     &P, sizeof P, true);
         if (rc == GLLMQ_OK && ksplit > 1) {
-            MmfReduceParams R{ P.partial, P.y, mm, P.n, P.ldy, ksplit };
+            MmfReduceParams R{ P.partial, P.y, mm, P.n, P.ldy, ksplit, P.elem };
             const uint64_t quads = (static_cast<uint64_t>(mm) * n + 3) / 4;
             rc = launch(ctx, ctx->mmf_reduce, static_cast<uint32_t>((quads + 255) / 256), 256, 0, stream, &R, sizeof R, true);
         }
@@ -874,7 +875,7 @@ MmfsPlan plan_mmfs(const gllmq_ctx *ctx, const Format &f, size_t m, size_t n, si
 int run_mmfs(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
              size_t k, bool act_bf16, void *stream, size_t min_m = 9)
 {
-    if (m < min_m || ctx->call_elem) return -1;
+    if (m < min_m) return -1;
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
     const MmfsPlan L = plan_mmfs(ctx, f, m, n, k);
     if (!L.ok) return -1;
@@ -883,14 +884,15 @@ int run_mmfs(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, cons
     const int fmt = f.dtype == T_Q5_K ? 1 : 0;
     for (size_t m0 = 0; m0 < m; m0 += 32) {
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(32, m - m0));
-        MmfPrepParams Q{ x + m0 * k, static_cast<uint8_t *>(S.mmf), mm, static_cast<uint32_t>(k), static_cast<uint32_t>(k),
-                         act_bf16 ? 1u : 0u };
+        MmfPrepParams Q{ elem_at(ctx, x, m0 * k), static_cast<uint8_t *>(S.mmf), mm, static_cast<uint32_t>(k), static_cast<uint32_t>(k),
+                         act_bf16 ? 1u : 0u, ctx->call_elem };
         int rc = launch2d(ctx, ctx->mmf_prep_lanes, L.groups, 16, 64, 0, stream, &Q, sizeof Q, true);
         if (rc != GLLMQ_OK) return rc;
         Mm8Params P{};
         P.w = w;
         P.x = static_cast<const float *>(S.mmf); // the images
-        P.y = y + m0 * n;
+        P.y = elem_at(ctx, y, m0 * n);
+        P.elem = ctx->call_elem;
         P.n = static_cast<uint32_t>(n);
         P.k = static_cast<uint32_t>(k);
         P.groups = L.groups;
@@ -1492,9 +1494,13 @@ int convert_elems(gllmq_ctx *ctx, const void *src, void *dst, size_t count, uint
 
 size_t elem_scratch_bytes(size_t m, size_t n, size_t k) { return ((m * k * 4 + 255) & ~size_t(255)) + m * n * 4; }
 
-// Whether the kernels that convert 16-bit elements in their own loads and stores take the shape:
-// the int8 and integer-dot kernels of up to 8 rows, within one launch of K.
-bool elem_in_kernel(const gllmq_ctx *ctx, size_t m, size_t k) { return ctx->elem_fused && !ctx->gemv_f32 && m <= 8 && k <= 16384; }
+// Whether the kernels convert 16-bit elements in their own loads and stores: all but the GEMV when
+// it covers K in several launches (which add up in y), and its f32 flavour.
+bool elem_in_kernel(const gllmq_ctx *ctx, size_t m, size_t k)
+{
+    (void)m;
+    return ctx->elem_fused && !ctx->gemv_f32 && k <= 16384;
+}
 
 } // namespace
 

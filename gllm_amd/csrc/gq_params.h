@@ -194,6 +194,7 @@ struct MmfParams {
     uint32_t ksplit;           // workgroups per row tile
     uint32_t blocks_per_split; // 256-element blocks of K per workgroup
     uint32_t act_bf16;
+    uint32_t elem;             // element type of y (ELEM_F32 / ELEM_F16 / ELEM_BF16); partial sums stay f32
 };
 
 constexpr int MMF_WAVES = 8;
@@ -279,12 +280,14 @@ struct MmfPrepParams {
     const float *x;
     uint8_t *ximg;
     uint32_t m, k, ldx, act_bf16;
+    uint32_t elem; // element type of x
 };
 
 struct MmfReduceParams {
     const float *partial; // [ksplit][m][n]
     float *y;             // [m][ldy]
     uint32_t m, n, ldy, ksplit;
+    uint32_t elem; // element type of y
 };
 
 struct GatherParams {

@@ -156,6 +156,17 @@ public:
         return make(gllmq_argmax(ctx_, logits_dev, rows, n, ld, token_dev, value_dev, stream), "argmax");
     }
 
+    // Backend<E>::quantized_matmul for E = f16 / bf16 (src/compat/mod.rs:376-378): x_dev and y_dev hold
+    // elements of type `elem` (GLLMQ_ELEM_*); results are the f32 call's, rounded to nearest even.
+    BackendError quantized_matmul_elem_device(const void *w_dev, size_t w_bytes, const void *x_dev, void *y_dev, QuantType t,
+                                              size_t m, size_t n, size_t k, int elem, void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_quantized_matmul_elem(ctx_, w_dev, w_bytes, x_dev, y_dev, static_cast<uint32_t>(t), m, n, k, elem,
+                                                stream),
+                    "quantized_matmul");
+    }
+
     // The lm_head matvec of one row and Op::Argmax behind it as one call; logits_dev may be null
     // for Q6_K / Q8_0 matrices with k <= 16384 (the logits then never reach memory).
     BackendError lm_head_argmax_device(const void *w_dev, size_t w_bytes, const float *x_dev, QuantType t, size_t n, size_t k,

@@ -81,6 +81,11 @@ extern "C" {
                             ffn: usize, relu_gate: c_int, stream: *mut c_void) -> c_int;
     pub fn gllmq_argmax(ctx: *mut gllmq_ctx, logits_dev: *const f32, rows: usize, n: usize, ld: usize,
                         token_dev: *mut u32, value_dev: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn gllmq_quantized_matmul_elem(ctx: *mut gllmq_ctx, w_dev: *const c_void, w_bytes: usize, x_dev: *const c_void,
+                                       y_dev: *mut c_void, ggml_dtype: u32, m: usize, n: usize, k: usize, elem: c_int,
+                                       stream: *mut c_void) -> c_int;
+    pub fn gllmq_reserve_matmul_elem(ctx: *mut gllmq_ctx, ggml_dtype: u32, m: usize, n: usize, k: usize, elem: c_int,
+                                     stream: *mut c_void) -> c_int;
     pub fn gllmq_lm_head_argmax(ctx: *mut gllmq_ctx, w_dev: *const c_void, w_bytes: usize, x_dev: *const f32,
                                 ggml_dtype: u32, n: usize, k: usize, logits_dev: *mut f32, token_dev: *mut u32,
                                 value_dev: *mut f32, stream: *mut c_void) -> c_int;
@@ -271,6 +276,19 @@ impl HipQuant {
     pub unsafe fn argmax_device(&self, logits: *const f32, rows: usize, n: usize, ld: usize, token: *mut u32,
                                 value: *mut f32, stream: *mut c_void) -> Result<(), QuantError> {
         self.check(gllmq_argmax(self.ctx, logits, rows, n, ld, token, value, stream), "argmax")
+    }
+
+    /// `Backend<E>::quantized_matmul` for `E` = `half::f16` (`elem` 1) or `half::bf16` (`elem` 2) over
+    /// device buffers of that element type (src/compat/mod.rs:376-378); 0 is f32.  Results are the
+    /// f32 call's, rounded to the nearest element, ties to even (`E::from_f32`).
+    ///
+    /// # Safety
+    /// `w` must hold `w_bytes` bytes, `x` `m * k` and `y` `m * n` elements of the type, on this device.
+    pub unsafe fn quantized_matmul_elem_device(&self, w: *const c_void, w_bytes: usize, x: *const c_void, y: *mut c_void,
+                                               ggml_dtype: u32, m: usize, n: usize, k: usize, elem: c_int,
+                                               stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_quantized_matmul_elem(self.ctx, w, w_bytes, x, y, ggml_dtype, m, n, k, elem, stream),
+                   "quantized_matmul")
     }
 
     /// The lm_head matvec of one activation row and `Op::Argmax` behind it as one call.  `logits`
