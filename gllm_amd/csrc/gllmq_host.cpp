@@ -250,6 +250,12 @@ struct gllmq_ctx {
     uint32_t gemv_waves = 2048; // waves a GEMV launch aims to put on the device
     bool lm_head_fused = true;  // lm_head_argmax: candidates from the GEMV's own workgroups
     uint32_t call_elem = 0;     // element type of x and y of the matmul being enqueued (call_mutex held); 0 = f32
+    // activations of the matmul being enqueued that are a gated product: x[r][i] = act(x[r][i]) * x[r][i + call_glu_off],
+    // rows call_ldx elements apart (the input of a feed-forward block's down projection); 0 = plain
+    uint32_t call_glu = 0, call_glu_off = 0, call_ldx = 0;
+    bool ffn_glu_load = true;   // "ffn_glu_load" = 0: the gate activation always runs as a kernel of its own
+    hipFunction_t mm8s_glu[3][3] = {};          // streamed kernels that take gated activations [format][p1_e2, p2_e4, p1_e4]
+    hipFunction_t gemv_i8_glu[kNumFormats][2] = {};
     bool elem_fused = true;     // "elem_fused" = 0: 16-bit elements always through conversion launches
     hipFunction_t convert_elem = nullptr;
     std::mutex err_mutex;
@@ -446,6 +452,16 @@ T *elem_at(const gllmq_ctx *ctx, T *base, size_t index)
     return reinterpret_cast<T *>(reinterpret_cast<Byte *>(base) + index * (ctx->call_elem ? 2u : 4u));
 }
 
+// Elements between activation rows of the matmul being enqueued: k unless the caller says otherwise.
+uint32_t row_stride_x(const gllmq_ctx *ctx, size_t k) { return ctx->call_ldx ? ctx->call_ldx : static_cast<uint32_t>(k); }
+
+// What a kernel family answers when it would take the shape but cannot read gated activations:
+// the caller then applies the gate in a launch of its own.
+constexpr int kNeedPlainActivations = -2;
+
+// Gated activations are read as aligned float4 from both factors.
+bool glu_vector_ok(const gllmq_ctx *ctx) { return ctx->call_glu_off % 4u == 0u && ctx->call_ldx % 4u == 0u; }
+
 // Shape-dependent fields of a GEMV launch over at most 64 groups (16384 elements) of K and
 // m <= 2: how a row is split over lanes and waves, rows per workgroup, LDS.  `target_waves`
 // is the number of waves the launch aims to put on the device.
@@ -499,12 +515,14 @@ int launch_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, size_t row_by
     P.y = y;
     P.ldx = ldx;
     P.ldy = ldy;
-    P.x_vec = aligned(x, 16) && (m == 1 || ldx % 4 == 0);
+    P.x_vec = aligned(x, 16) && (m == 1 || ldx % (ctx->call_elem ? 8 : 4) == 0);
     P.accumulate = accumulate ? 1u : 0u;
     P.act_bf16 = act_bf16 ? 1u : 0u;
     P.elem = ctx->call_elem;
+    P.glu = ctx->call_glu;
+    P.glu_off = ctx->call_glu_off;
     const int fi = format_index(f.dtype);
-    hipFunction_t fn = ctx->gemv_f32 ? ctx->gemv[fi][m - 1] : ctx->gemv_i8[fi][m - 1];
+    hipFunction_t fn = ctx->gemv_f32 ? ctx->gemv[fi][m - 1] : ctx->call_glu ? ctx->gemv_i8_glu[fi][m - 1] : ctx->gemv_i8[fi][m - 1];
     return launch(ctx, fn, L.grid, L.threads, L.lds, stream, &P, sizeof P);
 }
 
@@ -594,7 +612,15 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     int variant;
     if (areg) variant = pi == 1 ? 2 : (steps <= 1 ? 0 : 1);
     else variant = (pi == 0 && steps > 2) ? 6 : 3 + static_cast<int>(pi);
+    hipFunction_t fn = ctx->mm8s[sfmt][variant];
+    if (ctx->call_glu) {
+        const int gv = variant == 3 ? 0 : variant == 4 ? 1 : variant == 6 ? 2 : -1;
+        if (gv < 0 || !glu_vector_ok(ctx)) return kNeedPlainActivations;
+        fn = ctx->mm8s_glu[sfmt][gv];
+    }
     Mm8Params P{};
+    P.glu = ctx->call_glu;
+    P.glu_off = ctx->call_glu_off;
     P.w = w;
     P.x = x;
     P.y = y;
@@ -603,7 +629,7 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     P.groups = groups;
     P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
     P.m = mm;
-    P.ldx = static_cast<uint32_t>(k);
+    P.ldx = row_stride_x(ctx, k);
     P.ldy = static_cast<uint32_t>(n);
     P.tiles = tiles;
     P.grid = grid;
@@ -621,8 +647,7 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     P.lds_ring = L.ring;
     P.depth = depth;
     const uint32_t lds = L.total;
-    return launch(ctx, ctx->mm8s[sfmt][variant], grid, (gq::MM8S_CWAVES + gq::MM8S_LOADERS) * 64, lds, stream,
-                  &P, sizeof P);
+    return launch(ctx, fn, grid, (gq::MM8S_CWAVES + gq::MM8S_LOADERS) * 64, lds, stream, &P, sizeof P);
 }
 
 // Q4_K, Q5_K and Q6_K on the int8 matrix cores, activation rows in passes of at most 8 (a pass keeps
@@ -695,6 +720,7 @@ int run_mm8(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         --rows_per_pass;
     if (rows_per_pass == 0) return -1;
     if (one_pass_only && rows_per_pass < m) return -1;
+    if (ctx->call_glu) return kNeedPlainActivations;
     for (size_t m0 = 0; m0 < m; m0 += rows_per_pass) {
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(rows_per_pass, m - m0));
         const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
@@ -773,6 +799,7 @@ int run_mmf(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
     const int fmt = f.dtype == T_Q8_0 ? 3 : f.dtype == T_Q6_K ? 2 : f.dtype == T_Q5_K ? 1 : 0;
     if (fmt == 3 && k < 256) return -1; // the Q8_0 fetch window is one whole group of 8 blocks
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
+    if (ctx->call_glu && !glu_vector_ok(ctx)) return kNeedPlainActivations;
     const MmfPlan L = plan_mmf(ctx, m, n, k);
     const uint32_t groups = L.groups, row_tiles = L.row_tiles, ksplit = L.ksplit, bps = L.bps;
     if (row_tiles > kMmfMaxRowTiles) return -1;
@@ -787,7 +814,8 @@ int run_mmf(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         MmfParams P{};
         P.w = w;
         P.elem = ctx->call_elem;
-        P.x = elem_at(ctx, x, m0 * k);
+        P.ldx = row_stride_x(ctx, k);
+        P.x = elem_at(ctx, x, m0 * P.ldx);
         P.y = elem_at(ctx, y, m0 * n);
         P.ximg = static_cast<uint8_t *>(S.mmf);
         P.partial = reinterpret_cast<float *>(static_cast<uint8_t *>(S.mmf) + img_bytes);
@@ -796,13 +824,12 @@ int run_mmf(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         P.groups = groups;
         P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
         P.m = mm;
-        P.ldx = static_cast<uint32_t>(k);
         P.ldy = static_cast<uint32_t>(n);
         P.row_tiles = row_tiles;
         P.ksplit = ksplit;
         P.blocks_per_split = bps;
         P.act_bf16 = act_bf16 ? 1u : 0u;
-        MmfPrepParams Q{ P.x, P.ximg, mm, P.k, P.ldx, P.act_bf16, P.elem };
+        MmfPrepParams Q{ P.x, P.ximg, mm, P.k, P.ldx, P.act_bf16, P.elem, ctx->call_glu, ctx->call_glu_off };
         int rc = launch2d(ctx, ctx->mmf_prep[mt - 1], groups, 16, 64, 0, stream, &Q, sizeof Q, true);
         if (rc != GLLMQ_OK) return rc;
         rc = launch(ctx, ctx->mmf_q4k[fmt][mt - 1][act_bf16 ? 1 : 0], row_tiles * ksplit, 512, mmf_lds_bytes(mt, fmt), stream,
@@ -879,13 +906,14 @@ int run_mmfs(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, cons
     if (!aligned(x, 16) || k % 4 != 0) return -1; // activation rows are loaded as aligned float4
     const MmfsPlan L = plan_mmfs(ctx, f, m, n, k);
     if (!L.ok) return -1;
+    if (ctx->call_glu && !glu_vector_ok(ctx)) return kNeedPlainActivations;
     int grc = grow_scratch(ctx, S, &S.mmf, &S.mmf_bytes, L.need, stream, "quantized_matmul (GEMM)");
     if (grc != GLLMQ_OK) return grc;
     const int fmt = f.dtype == T_Q5_K ? 1 : 0;
     for (size_t m0 = 0; m0 < m; m0 += 32) {
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(32, m - m0));
-        MmfPrepParams Q{ elem_at(ctx, x, m0 * k), static_cast<uint8_t *>(S.mmf), mm, static_cast<uint32_t>(k), static_cast<uint32_t>(k),
-                         act_bf16 ? 1u : 0u, ctx->call_elem };
+        MmfPrepParams Q{ elem_at(ctx, x, m0 * row_stride_x(ctx, k)), static_cast<uint8_t *>(S.mmf), mm, static_cast<uint32_t>(k),
+                         row_stride_x(ctx, k), act_bf16 ? 1u : 0u, ctx->call_elem, ctx->call_glu, ctx->call_glu_off };
         int rc = launch2d(ctx, ctx->mmf_prep_lanes, L.groups, 16, 64, 0, stream, &Q, sizeof Q, true);
         if (rc != GLLMQ_OK) return rc;
         Mm8Params P{};
@@ -1010,12 +1038,14 @@ int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
 {
     const size_t rb = gllmq_row_bytes(f.dtype, k);
     constexpr size_t kChunk = 16384; // elements of K one launch covers (four waves of 4096)
+    if (ctx->call_glu && ctx->gemv_f32) return kNeedPlainActivations;
+    const uint32_t ldx = row_stride_x(ctx, k);
     for (size_t m0 = 0; m0 < m; m0 += 2) {
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(2, m - m0));
         for (size_t k0 = 0; k0 < k; k0 += kChunk) {
             const size_t kk = std::min(kChunk, k - k0);
-            int rc = launch_gemv(ctx, f, w + (k0 / 256) * f.group_bytes, rb, elem_at(ctx, x, m0 * k + k0), elem_at(ctx, y, m0 * n), mm,
-                                 static_cast<uint32_t>(n), static_cast<uint32_t>(kk), static_cast<uint32_t>(k),
+            int rc = launch_gemv(ctx, f, w + (k0 / 256) * f.group_bytes, rb, elem_at(ctx, x, m0 * ldx + k0), elem_at(ctx, y, m0 * n), mm,
+                                 static_cast<uint32_t>(n), static_cast<uint32_t>(kk), ldx,
                                  static_cast<uint32_t>(n), k0 != 0, act_bf16, stream);
             if (rc != GLLMQ_OK) return rc;
         }
@@ -1028,20 +1058,20 @@ int dispatch_matmul(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *
                     size_t n, size_t k, bool bf16, void *stream)
 {
     int rc = run_mmfs(ctx, S, f, w, x, y, m, n, k, bf16, stream);
-    if (rc >= 0) return rc;
+    if (rc >= 0 || rc == kNeedPlainActivations) return rc;
     rc = run_mmf(ctx, S, f, w, x, y, m, n, k, bf16, stream);
-    if (rc >= 0) return rc;
+    if (rc >= 0 || rc == kNeedPlainActivations) return rc;
     // up to 8 rows: the int8 kernels when one pass over the weights does it, else the GEMM
     rc = run_mm8s(ctx, f, w, x, y, m, n, k, bf16, stream);
-    if (rc >= 0) return rc;
+    if (rc >= 0 || rc == kNeedPlainActivations) return rc;
     rc = run_mm8(ctx, S, f, w, x, y, m, n, k, bf16, stream, true);
-    if (rc >= 0) return rc;
+    if (rc >= 0 || rc == kNeedPlainActivations) return rc;
     if (ctx->mmf_small_min_m > 0) {
         rc = run_mmf(ctx, S, f, w, x, y, m, n, k, bf16, stream, ctx->mmf_small_min_m);
-        if (rc >= 0) return rc;
+        if (rc >= 0 || rc == kNeedPlainActivations) return rc;
     }
     rc = run_mm8(ctx, S, f, w, x, y, m, n, k, bf16, stream);
-    if (rc >= 0) return rc;
+    if (rc >= 0 || rc == kNeedPlainActivations) return rc;
     return run_gemv(ctx, f, w, x, y, m, n, k, bf16, stream);
 }
 
@@ -1155,6 +1185,9 @@ int gllmq_init(gllmq_ctx **out, int device)
             if (rc != GLLMQ_OK) break;
             snprintf(name, sizeof name, "gq_gemv_i8_%s_m%d", kFormats[i].tag, m);
             rc = get_function(ctx, &ctx->gemv_i8[i][m - 1], name);
+            if (rc != GLLMQ_OK) break;
+            snprintf(name, sizeof name, "gq_gemv_i8_%s_m%d_glu", kFormats[i].tag, m);
+            rc = get_function(ctx, &ctx->gemv_i8_glu[i][m - 1], name);
         }
         if (rc != GLLMQ_OK) break;
         snprintf(name, sizeof name, "gq_gemv_i8_%s_m1_argmax", kFormats[i].tag);
@@ -1241,6 +1274,12 @@ int gllmq_init(gllmq_ctx **out, int device)
                 snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8s[v]);
                 rc = get_function(ctx, &ctx->mm8s[q][v], name);
             }
+        static const char *const kMm8sGlu[3] = { "p1_e2_g", "p2_e4_g", "p1_e4_g" };
+        for (int q = 0; q < 3; ++q)
+            for (int v = 0; v < 3 && rc == GLLMQ_OK; ++v) {
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8sGlu[v]);
+                rc = get_function(ctx, &ctx->mm8s_glu[q][v], name);
+            }
     }
     if (rc != GLLMQ_OK) {
         fprintf(stderr, "gllmq_init: %s\n", ctx->err.c_str());
@@ -1296,6 +1335,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "chain_spin_limit") ctx->chain_spin_limit = u;
     else if (n == "lm_head_fused") ctx->lm_head_fused = value != 0;
     else if (n == "elem_fused") ctx->elem_fused = value != 0;
+    else if (n == "ffn_glu_load") ctx->ffn_glu_load = value != 0;
     else if (n == "mmfs_all") ctx->mmfs_all = value != 0;
     else if (n == "mmfs_min_rows") ctx->mmfs_min_rows = std::max(1u, u);
     else if (n == "batch_overlap") ctx->batch_overlap = value != 0;
@@ -1613,6 +1653,17 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_
             A.ld = static_cast<uint32_t>(ffn);
         }
         if (rc != GLLMQ_OK) return rc;
+        // the down projection reads act(gate) * up straight from the two results where its kernel
+        // can; else the activation runs as a launch of its own and writes h
+        const size_t up_off = static_cast<size_t>(A.u - A.g);
+        if (ctx->ffn_glu_load && up_off <= 0xFFFFFFFFu) {
+            ctx->call_glu = relu_gate ? 2u : 1u;
+            ctx->call_glu_off = static_cast<uint32_t>(up_off);
+            ctx->call_ldx = A.ld;
+            rc = dispatch_matmul(ctx, S, *fd, static_cast<const uint8_t *>(down_w), gu, out, m, hidden, ffn, false, stream);
+            ctx->call_glu = ctx->call_glu_off = ctx->call_ldx = 0;
+            if (rc != kNeedPlainActivations) return rc;
+        }
         rc = launch2d(ctx, ctx->glu_act, static_cast<uint32_t>((ffn + 255) / 256),
                       static_cast<uint32_t>(std::min<size_t>(m, 65535)), 256, 0, stream, &A, sizeof A);
         if (rc != GLLMQ_OK) return rc;

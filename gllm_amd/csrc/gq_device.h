@@ -131,10 +131,13 @@ __device__ __forceinline__ T load_unaligned(const void *p)
 
 // Gate activation of the feed-forward block: SiLU, behind a ReLU when `relu`
 // (reference: Op::SwiGlu, silu(gate) * up, src/arch/auto_graph_fragments/build_graph.inc.rs:1977-1984).
+// The hardware's exponential and reciprocal (about 1 ulp each): a kernel that applies the gate to
+// the activations it loads does so in every workgroup, where a library exponential would cost
+// microseconds.
 __device__ __forceinline__ float glu_act(float g, bool relu)
 {
     if (relu) g = g > 0.0f ? g : 0.0f;
-    return g / (1.0f + expf(-g));
+    return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g));
 }
 
 // (sc, m) pair j of the 12-byte field held as three little-endian dwords s0,s1,s2

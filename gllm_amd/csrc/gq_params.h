@@ -32,6 +32,7 @@ struct GemvParams {
     uint32_t prep_words; // integer-dot kernels: 32-bit words of LDS holding the prepared activations
     uint32_t act_bf16;   // integer-dot kernels: round activations to bf16 before use
     uint32_t elem;       // integer-dot kernels: element type of x and y (ELEM_F32 / ELEM_F16 / ELEM_BF16)
+    uint32_t glu, glu_off; // integer-dot kernels: x[i] = act(x[i]) * x[i + glu_off] (0 off, 1 SiLU, 2 SiLU behind a ReLU)
     uint64_t *keys;      // kernels that end in the greedy token choice: one candidate per workgroup (argmax_key)
 };
 
@@ -67,6 +68,9 @@ struct Mm8Params {
     // workgroup and of the last one, rows of the last one, the LDS offsets of the counters
     // and of the ring, and the items a loader keeps unconfirmed (1 .. MM8S_MAX_DEPTH)
     uint32_t rows_per_wg, tile_rows, ring_slots, wg_tiles, last_wg_tiles, last_wg_rows, lds_ctrl, lds_ring, depth;
+    // activations that are the gated product of two f32 vectors (the input of a feed-forward
+    // block's down projection): x[i] = act(x[i]) * x[i + glu_off]; glu = 0 off, 1 SiLU, 2 SiLU behind a ReLU
+    uint32_t glu, glu_off;
 };
 
 constexpr uint32_t MM8_SPLIT_MAX_LISTS = 256;        // tile lists (workgroups per slice) of a K-split launch
@@ -281,6 +285,7 @@ struct MmfPrepParams {
     uint8_t *ximg;
     uint32_t m, k, ldx, act_bf16;
     uint32_t elem; // element type of x
+    uint32_t glu, glu_off; // x[i] = act(x[i]) * x[i + glu_off] (0 off, 1 SiLU, 2 SiLU behind a ReLU)
 };
 
 struct MmfReduceParams {

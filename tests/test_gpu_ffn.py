@@ -112,6 +112,34 @@ def test_ffn_three_step_form(torch, oracle):
         check(got, want, f"three steps m={m}")
 
 
+@pytest.mark.parametrize("t_gu,t_dn,hidden,ffn,ms", [
+    (Q6_K, Q6_K, 2048, 4352, (1, 2, 4, 8)),    # GEMV gate/up; streamed down projection that reads the gated product
+    (Q8_0, Q4_K, 2048, 4608, (1, 3)),          # Q8_0 gate/up, streamed Q4_K down
+    (Q6_K, Q8_0, 1024, 1536, (1, 2, 5)),       # GEMV down projection (two rows at a time)
+    (Q4_K, Q5_K, 2048, 5120, (16, 40)),        # GEMM: the preparation launch of the down projection applies the gate
+    (Q6_K, Q6_K, 512, 776, (1, 9)),            # ragged ffn
+    (Q8_0, Q8_0, 256, 200, (1, 2, 70)),        # ffn not a multiple of 64: the GEMV's scalar loads
+])
+def test_down_projection_reads_the_gated_product(torch, oracle, t_gu, t_dn, hidden, ffn, ms):
+    """Where the gate/up products are not gated in their kernel's epilogue, the down projection's
+    activation loads apply act(gate) * up themselves (no launch and no buffer for it): the same bits
+    as with the activation as a launch of its own (option ffn_glu_load = 0), for stacked and
+    separate gate/up tensors and the ReLU gate; and the oracle's bars."""
+    from gllm_amd.backend import HipBackend
+    fused, plain = HipBackend(0, options={"ffn_fused": 0}), HipBackend(0, options={"ffn_fused": 0, "ffn_glu_load": 0})
+    gate, up = random_weight(t_gu, ffn, hidden, seed=1), random_weight(t_gu, ffn, hidden, seed=2)
+    down = random_weight(t_dn, hidden, ffn, seed=3)
+    for m in ms:
+        for stacked, relu in ((True, False), (False, True)):
+            print(f"gated loads gate/up={t_gu} down={t_dn} hidden={hidden} ffn={ffn} m={m} stacked={stacked} relu={relu}", flush=True)
+            x = random_activations(m, hidden, seed=m)
+            got = run_ffn(fused, torch, gate, up, t_gu, down, t_dn, x, m, hidden, ffn, relu=relu, stacked=stacked)
+            ref = run_ffn(plain, torch, gate, up, t_gu, down, t_dn, x, m, hidden, ffn, relu=relu, stacked=stacked)
+            assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), "differs from the activation as its own launch"
+            want = oracle.ffn_swiglu(gate, up, t_gu, down, t_dn, x, m, hidden, ffn, relu_gate=relu, acc=oracle.ACC_F64, threads=8)
+            check(got, want, f"gated loads m={m}")
+
+
 def test_ffn_argument_errors(hip, torch):
     from gllm_amd.backend import BackendError, Unimplemented
     print("ffn errors", flush=True)
