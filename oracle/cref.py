@@ -67,6 +67,12 @@ def lib() -> C.CDLL:
         L.gq_have_avx2.argtypes = []
         L.gq_dequant_block_avx2.restype = C.c_int
         L.gq_dequant_block_avx2.argtypes = [C.c_uint32, u8p, f32p]
+        L.gq_quantized_matmul_avx512.restype = C.c_int
+        L.gq_quantized_matmul_avx512.argtypes = [u8p, f32p, f32p, C.c_uint32, sz, sz, sz, C.c_int]
+        L.gq_have_avx512.restype = C.c_int
+        L.gq_have_avx512.argtypes = []
+        L.gq_dequant_block_avx512.restype = C.c_int
+        L.gq_dequant_block_avx512.argtypes = [C.c_uint32, u8p, f32p]
         L.gq_softmax.restype = None
         L.gq_softmax.argtypes = [f32p, sz, f32p]
         L.gq_topk_with_weights.restype = sz
@@ -221,6 +227,34 @@ def quantized_matmul_avx2(w, x: np.ndarray, dtype: int, m: int, n: int, k: int,
     rc = lib().gq_quantized_matmul_avx2(_u8(wb), _f32(xa), _f32(y), dtype, m, n, k, threads)
     if rc != OK:
         raise NotImplementedError(f"quantized_matmul_avx2: rc={rc}")
+    return y
+
+
+def have_avx512() -> bool:
+    return bool(lib().gq_have_avx512())
+
+
+def dequant_block_avx512(block, dtype: int) -> np.ndarray:
+    """One block through the decoder of the CPU baseline's AVX-512 flavour."""
+    b = _bytes_arr(block)
+    assert b.size == block_bytes(dtype)
+    out = np.zeros(block_size(dtype), np.float32)
+    rc = lib().gq_dequant_block_avx512(dtype, _u8(b), _f32(out))
+    if rc != OK:
+        raise NotImplementedError(f"dequant_block_avx512: rc={rc}")
+    return out
+
+
+def quantized_matmul_avx512(w, x: np.ndarray, dtype: int, m: int, n: int, k: int,
+                          threads: int = 1) -> np.ndarray:
+    """The vectorised flavour of the CPU baseline (AVX-512 decode, f32 dot over sixteen-lane sums)."""
+    wb = _bytes_arr(w)
+    assert wb.size >= n * row_bytes(dtype, k), "weight buffer shorter than n rows"
+    xa = np.ascontiguousarray(x, np.float32).reshape(m, k)
+    y = np.zeros((m, n), np.float32)
+    rc = lib().gq_quantized_matmul_avx512(_u8(wb), _f32(xa), _f32(y), dtype, m, n, k, threads)
+    if rc != OK:
+        raise NotImplementedError(f"quantized_matmul_avx512: rc={rc}")
     return y
 
 

@@ -29,7 +29,7 @@
  *                                         summation order, threading and any internal
  *                                         activation handling are PARITY UNPINNED (no
  *                                         test or fixture of the reference exercises it)
- *   gq_quantized_matmul_avx2            : the vectorised baseline flavour; decoders pinned bitwise
+ *   gq_quantized_matmul_avx2 / _avx512  : the vectorised baseline flavours; decoders pinned bitwise
  *                                         against the scalar ones, the sum against the f64 yardstick;
  *                                         same status as gq_quantized_matmul otherwise
  *   gq_quant_gather                     : unscaled lookups are pinned with gq_dequantize (a row
@@ -129,6 +129,14 @@ int gq_have_avx2(void);
 int gq_dequant_block_avx2(uint32_t ggml_dtype, const uint8_t *blk, float *out);
 int gq_quantized_matmul_avx2(const uint8_t *w, const float *x, float *y, uint32_t ggml_dtype,
                              size_t m, size_t n, size_t k, int threads);
+
+/* The same sixteen elements at a time (AVX-512 F/BW/VL/DQ, compiled by function attribute and
+ * chosen at run time): decoders again equal to the scalar ones bit for bit, the dot product over
+ * sixteen-lane partial sums.  GQ_ERR_UNIMPLEMENTED where the host has no AVX-512. */
+int gq_have_avx512(void);
+int gq_dequant_block_avx512(uint32_t ggml_dtype, const uint8_t *blk, float *out);
+int gq_quantized_matmul_avx512(const uint8_t *w, const float *x, float *y, uint32_t ggml_dtype,
+                               size_t m, size_t n, size_t k, int threads);
 
 /* src/moe/routing.rs:290-302 */
 void gq_softmax(const float *logits, size_t n, float *probs);

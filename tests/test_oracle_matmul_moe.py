@@ -210,12 +210,17 @@ def test_moe_ffn_equals_dense_masked_evaluation(oracle, relu_gate):
 
 
 # ------------------------------------------- the vectorised flavour of the CPU baseline
+FLAVOURS = ["avx2", "avx512"]
+
+
+@pytest.mark.parametrize("flavour", FLAVOURS)
 @pytest.mark.parametrize("dtype", ALL)
-def test_avx2_decoders_equal_the_scalar_ones_bit_for_bit(oracle, dtype):
+def test_vector_decoders_equal_the_scalar_ones_bit_for_bit(oracle, dtype, flavour):
     """Random blocks (every byte pattern of quants and scales; f16 scales over normal, subnormal,
     zero and negative values) and blocks of all-0x00 / all-0xFF quants."""
-    if not oracle.have_avx2():
-        pytest.skip("host without AVX2+FMA")
+    if not getattr(oracle, f"have_{flavour}")():
+        pytest.skip(f"host without {flavour}")
+    decode = getattr(oracle, f"dequant_block_{flavour}")
     bb = oracle.block_bytes(dtype)
     rng = np.random.default_rng(dtype)
     blocks = rng.integers(0, 256, (400, bb), dtype=np.uint8)
@@ -229,22 +234,24 @@ def test_avx2_decoders_equal_the_scalar_ones_bit_for_bit(oracle, dtype):
     blocks[2, [j for j in range(bb) if j not in sum(([o, o + 1] for o in d_off), [])]] = 0xFF
     for blk in blocks:
         want = oracle.dequantize(blk, dtype)
-        got = oracle.dequant_block_avx2(blk, dtype)
+        got = decode(blk, dtype)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("flavour", FLAVOURS)
 @pytest.mark.parametrize("dtype", ALL)
-def test_avx2_matmul_matches_the_float64_yardstick(oracle, dtype):
+def test_vector_matmul_matches_the_float64_yardstick(oracle, dtype, flavour):
     """Whole blocks, a partial last block (the tail runs one element at a time), several activation
     rows, threads; unit vectors return weight columns bit for bit (every other term is +-0)."""
-    if not oracle.have_avx2():
-        pytest.skip("host without AVX2+FMA")
+    if not getattr(oracle, f"have_{flavour}")():
+        pytest.skip(f"host without {flavour}")
+    matmul = getattr(oracle, f"quantized_matmul_{flavour}")
     step = 32 if dtype == Q8_0 else 256
     for m, n, k in [(1, 33, 4096), (3, 17, 2 * step + step // 2 + 4), (2, 5, step)]:
         w, x = random_weight(dtype, n, k, seed=7), random_activations(m, k, seed=8)
         want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64)
         for threads in (1, 3):
-            got = oracle.quantized_matmul_avx2(w, x, dtype, m, n, k, threads=threads)
+            got = matmul(w, x, dtype, m, n, k, threads=threads)
             assert rel_l2(got, want) < 1e-6
             assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
     n, k = 9, 512
@@ -253,7 +260,7 @@ def test_avx2_matmul_matches_the_float64_yardstick(oracle, dtype):
     for col in (0, 7, 8, 31, 255, 256, 511):
         x = np.zeros((1, k), np.float32)
         x[0, col] = 1.0
-        y = oracle.quantized_matmul_avx2(w, x, dtype, 1, n, k)
+        y = matmul(w, x, dtype, 1, n, k)
         assert np.array_equal(y[0], deq[:, col])
 
 
