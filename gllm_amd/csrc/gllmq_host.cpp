@@ -149,6 +149,7 @@ struct Scratch {
 
 constexpr size_t kScratchArriveBytes = 4096; // MM8_SPLIT_MAX_LISTS words, padded; the chain kernel's counters behind them
 constexpr size_t kChainCountersAt = 512;     // first of its MM8C_MAX_ENTRIES + 1 words in that area
+constexpr size_t kLmHeadTicketAt = 600;      // the lm_head launch's count of finished workgroups
 constexpr size_t kScratchKeysBytes = sizeof(uint64_t) * gq::ARGMAX_MAX_ROWS * gq::ARGMAX_MAX_PARTS;
 constexpr size_t kScratchPartBytes = sizeof(float) * gq::MM8_SPLIT_PART_FLOATS;
 constexpr size_t kScratchFixedBytes = kScratchArriveBytes + kScratchKeysBytes + kScratchPartBytes;
@@ -1474,7 +1475,7 @@ int gllmq_lm_head_argmax(gllmq_ctx *ctx, const void *w, size_t w_bytes, const fl
     if (rc != GLLMQ_OK) return rc;
     // The matvec whose workgroups leave their best candidate behind, where the one-row GEMV is the
     // kernel such a matrix gets anyway (Q6_K and Q8_0, the types of GGUF output matrices) and one
-    // launch covers K; then the candidates, one per workgroup, to the token.
+    // launch covers K; the workgroup that finishes last picks among the candidates.
     const size_t rb = gllmq_row_bytes(dtype, k);
     const bool gemv_type = dtype == 14u || dtype == 8u;
     if (ctx->lm_head_fused && gemv_type && !ctx->gemv_f32 && k <= 16384) {
@@ -1488,14 +1489,10 @@ int gllmq_lm_head_argmax(gllmq_ctx *ctx, const void *w, size_t w_bytes, const fl
             P.ldy = static_cast<uint32_t>(n);
             P.x_vec = aligned(x, 16);
             P.keys = S->argmax_keys;
-            rc = launch(ctx, ctx->gemv_i8_argmax[format_index(dtype)], L.grid, L.threads, L.lds, stream, &P, sizeof P);
-            if (rc != GLLMQ_OK) return rc;
-            ArgmaxParams A{};
-            A.keys = S->argmax_keys;
-            A.parts = L.grid;
-            A.token = token;
-            A.value = value;
-            return launch(ctx, ctx->argmax_final, 1, 256, 0, stream, &A, sizeof A);
+            P.ticket = S->mm8_arrive + kLmHeadTicketAt;
+            P.token = token;
+            P.value = value;
+            return launch(ctx, ctx->gemv_i8_argmax[format_index(dtype)], L.grid, L.threads, L.lds, stream, &P, sizeof P, true);
         }
     }
     if (!logits)

@@ -33,7 +33,12 @@ struct GemvParams {
     uint32_t act_bf16;   // integer-dot kernels: round activations to bf16 before use
     uint32_t elem;       // integer-dot kernels: element type of x and y (ELEM_F32 / ELEM_F16 / ELEM_BF16)
     uint32_t glu, glu_off; // integer-dot kernels: x[i] = act(x[i]) * x[i + glu_off] (0 off, 1 SiLU, 2 SiLU behind a ReLU)
-    uint64_t *keys;      // kernels that end in the greedy token choice: one candidate per workgroup (argmax_key)
+    // kernels that end in the greedy token choice: one candidate per workgroup (argmax_key); the
+    // workgroup that finishes last (ticket counts them and is left at 0) picks among them
+    uint64_t *keys;
+    uint32_t *ticket;
+    uint32_t *token; // the choice (ARGMAX_NONE: no candidate)
+    float *value;    // null, or the chosen logit (NaN: none)
 };
 
 struct Mm8Params {

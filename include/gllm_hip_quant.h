@@ -193,8 +193,8 @@ int gllmq_reserve_matmul_elem(gllmq_ctx *ctx, uint32_t ggml_dtype, size_t m, siz
  * (build_graph.inc.rs:2661).  w_dev is [n x k] of ggml_dtype, x_dev k f32; token_dev and
  * value_dev as in gllmq_argmax (one row).  logits_dev (n f32) receives the logits; it may be
  * NULL when only the token is wanted and the matrix is Q6_K or Q8_0 with k <= 16384: there
- * every workgroup of the matvec leaves its best candidate behind and a one-workgroup launch
- * picks among them, so the logits are neither written nor read again.  Other matrices run
+ * every workgroup of the matvec leaves its best candidate behind and the one that finishes last
+ * picks among them (one launch), so the logits are neither written nor read again.  Other matrices run
  * gllmq_quantized_matmul and gllmq_argmax one after the other and need logits_dev.  The
  * logits and the token are those of the two calls made separately, bit for bit. */
 int gllmq_lm_head_argmax(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev, uint32_t ggml_dtype,
