@@ -42,12 +42,20 @@ def test_graph_replays_match_eager(hip, torch):
     logits = torch.empty(1, vocab, device="cuda")
     yb = torch.empty(16, 512, device="cuda")
     tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+    tok2 = torch.zeros(1, dtype=torch.int32, device="cuda")      # lm_head and token as one launch (a ticket counter in scratch)
+    xh = torch.empty(1, hidden, device="cuda", dtype=torch.bfloat16)
+    yh = torch.empty(1, 3 * hidden, device="cuda", dtype=torch.bfloat16)  # bf16 activations and outputs
+    wg6, wu6 = dev(random_weight(Q6_K, ffn, hidden, seed=8)), dev(random_weight(Q6_K, ffn, hidden, seed=9))
+    h6 = torch.empty(1, hidden, device="cuda")                    # gate applied in the down projection's loads
 
     def step():
         hip.quantized_matmul(wq, x, qkv, Q4_K, 1, 3 * hidden, hidden)
         hip.ffn_swiglu(wg, wu, Q4_K, wd, Q6_K, x, h, 1, hidden, ffn)
         hip.quantized_matmul(wo, h, logits, Q6_K, 1, vocab, hidden)
         hip.argmax(logits, tok)
+        hip.lm_head_argmax(wo, h, Q6_K, vocab, hidden, tok2)
+        hip.quantized_matmul(wq, xh, yh, Q4_K, 1, 3 * hidden, hidden)
+        hip.ffn_swiglu(wg6, wu6, Q6_K, wd, Q6_K, x, h6, 1, hidden, ffn)
         hip.quantized_matmul(wb, xb, yb, Q5_K, 16, 512, hidden)
         hip.quantized_matmul(ws, xs, ys, Q4_K, 2, 256, 8 * hidden)
 
@@ -55,6 +63,7 @@ def test_graph_replays_match_eager(hip, torch):
         x.copy_(torch.from_numpy(random_activations(1, hidden, seed=seed)))
         xb.copy_(torch.from_numpy(random_activations(16, hidden, seed=seed + 50)))
         xs.copy_(torch.from_numpy(random_activations(2, 8 * hidden, seed=seed + 90)))
+        xh.copy_(x.to(torch.bfloat16))
 
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
@@ -70,14 +79,17 @@ def test_graph_replays_match_eager(hip, torch):
         fill(seed)
         step()
         torch.cuda.synchronize()
-        want = [t.clone() for t in (qkv, h, logits, yb, ys, tok)]
-        for t in (qkv, h, logits, yb, ys):
+        outs = (qkv, h, logits, yb, ys, tok, tok2, yh, h6)
+        want = [t.clone() for t in outs]
+        assert int(tok2[0]) == int(tok[0])
+        for t in (qkv, h, logits, yb, ys, yh, h6):
             t.fill_(float("nan"))
         tok.fill_(-7)
+        tok2.fill_(-7)
         # eager work of the program's own between the replays
         hip.quantized_matmul(wq, x, torch.empty(1, 3 * hidden, device="cuda"), Q4_K, 1, 3 * hidden, hidden)
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        for got, exp in zip((qkv, h, logits, yb, ys, tok), want):
+        for got, exp in zip(outs, want):
             assert torch.equal(got, exp), f"replay {seed} differs from the eager run"
