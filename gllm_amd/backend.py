@@ -26,6 +26,7 @@ LIB_PATH = os.path.join(_HERE, "libgllm_hip_quant.so")
 OK, ERR_UNIMPLEMENTED, ERR_BAD_SHAPE, ERR_BAD_ALIGNMENT, ERR_HIP, ERR_INVALID = range(6)
 ACT_F32_SPLIT, ACT_BF16 = 0, 1
 DESC_AFTER_PREVIOUS = 1  # gllmq_matmul_desc.flags: the entry depends on the entries before it
+DESC_ELEM_F16, DESC_ELEM_BF16 = 0x100, 0x200  # gllmq_matmul_desc.flags: element type of the entry's x and y
 
 
 ELEM_F32, ELEM_F16, ELEM_BF16 = 0, 1, 2  # gllmq_quantized_matmul_elem: element type of activations and outputs
@@ -337,6 +338,10 @@ class HipBackend:
         arr = (MatmulDesc * len(items))()
         for i, (w, x, y, qt, m, n, k) in enumerate(items):
             flags = DESC_AFTER_PREVIOUS if after_previous is not None and after_previous(i) else 0
+            elem = self._elem_of(x.dtype)
+            if elem is None or y.dtype != x.dtype:
+                raise Unimplemented("make_batch: activations and outputs are f32, f16 or bf16, both of one type")
+            flags |= {ELEM_F32: 0, ELEM_F16: DESC_ELEM_F16, ELEM_BF16: DESC_ELEM_BF16}[elem]
             arr[i] = MatmulDesc(w.data_ptr(), w.numel() * w.element_size(), x.data_ptr(), y.data_ptr(),
                                 _dtype_id(qt), flags, m, n, k)
         return arr

@@ -1541,6 +1541,35 @@ bool elem_in_kernel(const gllmq_ctx *ctx, size_t m, size_t k)
 
 } // namespace
 
+namespace {
+
+// One validated quantized matmul over 16-bit activations and outputs with the scratch of `S`
+// (call_mutex held); elem is GLLMQ_ELEM_F16 or GLLMQ_ELEM_BF16.
+int matmul_elem_on_scratch(gllmq_ctx *ctx, Scratch &S, const void *w, size_t w_bytes, const void *x, void *y, uint32_t dtype,
+                           size_t m, size_t n, size_t k, int elem, void *stream)
+{
+    const Format *f = find_format(dtype);
+    int rc = check_matmul_args(ctx, f, w, w_bytes, static_cast<const float *>(x), static_cast<float *>(y), dtype, m, n, k);
+    if (rc >= 0) return rc;
+    if (elem_in_kernel(ctx, m, k)) {
+        ctx->call_elem = static_cast<uint32_t>(elem);
+        rc = dispatch_matmul(ctx, S, *f, static_cast<const uint8_t *>(w), static_cast<const float *>(x),
+                             static_cast<float *>(y), m, n, k, false, stream);
+        ctx->call_elem = 0;
+        return rc;
+    }
+    rc = grow_scratch(ctx, S, &S.elem, &S.elem_bytes, elem_scratch_bytes(m, n, k), stream, "quantized_matmul_elem");
+    if (rc != GLLMQ_OK) return rc;
+    float *xf = static_cast<float *>(S.elem);
+    float *yf = reinterpret_cast<float *>(static_cast<uint8_t *>(S.elem) + ((m * k * 4 + 255) & ~size_t(255)));
+    rc = convert_elems(ctx, x, xf, m * k, static_cast<uint32_t>(elem), true, stream);
+    if (rc == GLLMQ_OK) rc = dispatch_matmul(ctx, S, *f, static_cast<const uint8_t *>(w), xf, yf, m, n, k, false, stream);
+    if (rc == GLLMQ_OK) rc = convert_elems(ctx, yf, y, m * n, static_cast<uint32_t>(elem), false, stream);
+    return rc;
+}
+
+} // namespace
+
 int gllmq_quantized_matmul_elem(gllmq_ctx *ctx, const void *w, size_t w_bytes, const void *x, void *y, uint32_t dtype,
                                 size_t m, size_t n, size_t k, int elem, void *stream)
 {
@@ -1551,27 +1580,10 @@ int gllmq_quantized_matmul_elem(gllmq_ctx *ctx, const void *w, size_t w_bytes, c
                                          k, GLLMQ_ACT_F32_SPLIT, stream);
     if (elem != GLLMQ_ELEM_F16 && elem != GLLMQ_ELEM_BF16)
         return fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul_elem: unknown element type %d", elem);
-    const Format *f = find_format(dtype);
-    int rc = check_matmul_args(ctx, f, w, w_bytes, static_cast<const float *>(x), static_cast<float *>(y), dtype, m, n, k);
-    if (rc >= 0) return rc;
     Scratch *S = nullptr;
-    rc = acquire_scratch(ctx, stream, &S);
+    int rc = acquire_scratch(ctx, stream, &S);
     if (rc != GLLMQ_OK) return rc;
-    if (elem_in_kernel(ctx, m, k)) {
-        ctx->call_elem = static_cast<uint32_t>(elem);
-        rc = dispatch_matmul(ctx, *S, *f, static_cast<const uint8_t *>(w), static_cast<const float *>(x),
-                             static_cast<float *>(y), m, n, k, false, stream);
-        ctx->call_elem = 0;
-        return rc;
-    }
-    rc = grow_scratch(ctx, *S, &S->elem, &S->elem_bytes, elem_scratch_bytes(m, n, k), stream, "quantized_matmul_elem");
-    if (rc != GLLMQ_OK) return rc;
-    float *xf = static_cast<float *>(S->elem);
-    float *yf = reinterpret_cast<float *>(static_cast<uint8_t *>(S->elem) + ((m * k * 4 + 255) & ~size_t(255)));
-    rc = convert_elems(ctx, x, xf, m * k, static_cast<uint32_t>(elem), true, stream);
-    if (rc == GLLMQ_OK) rc = dispatch_matmul(ctx, *S, *f, static_cast<const uint8_t *>(w), xf, yf, m, n, k, false, stream);
-    if (rc == GLLMQ_OK) rc = convert_elems(ctx, yf, y, m * n, static_cast<uint32_t>(elem), false, stream);
-    return rc;
+    return matmul_elem_on_scratch(ctx, *S, w, w_bytes, x, y, dtype, m, n, k, elem, stream);
 }
 
 int gllmq_reserve_matmul_elem(gllmq_ctx *ctx, uint32_t dtype, size_t m, size_t n, size_t k, int elem, void *stream)
@@ -1703,15 +1715,20 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
                 continue;
             }
         }
-        if (d.flags & ~static_cast<uint32_t>(GLLMQ_DESC_AFTER_PREVIOUS)) {
+        constexpr uint32_t kElemBits = GLLMQ_DESC_ELEM_F16 | GLLMQ_DESC_ELEM_BF16;
+        if ((d.flags & ~(static_cast<uint32_t>(GLLMQ_DESC_AFTER_PREVIOUS) | kElemBits)) || (d.flags & kElemBits) == kElemBits) {
             rc = fail(ctx, GLLMQ_ERR_INVALID, "quantized_matmul_batch: unknown flag bits 0x%x in entry %zu", d.flags, i);
             break;
         }
         // an entry that depends on the ones before it starts a new group: its first launch is an
         // ordinary one
         ctx->overlap.entry_first = !(d.flags & GLLMQ_DESC_AFTER_PREVIOUS);
-        rc = matmul_on_scratch(ctx, *S, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k,
-                               GLLMQ_ACT_F32_SPLIT, stream);
+        if (d.flags & kElemBits)
+            rc = matmul_elem_on_scratch(ctx, *S, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k,
+                                        (d.flags & GLLMQ_DESC_ELEM_F16) ? GLLMQ_ELEM_F16 : GLLMQ_ELEM_BF16, stream);
+        else
+            rc = matmul_on_scratch(ctx, *S, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k,
+                                   GLLMQ_ACT_F32_SPLIT, stream);
     }
     ctx->overlap = gllmq_ctx::Overlap{};
     return rc;

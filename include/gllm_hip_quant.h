@@ -255,15 +255,18 @@ int gllmq_quantized_matmul_noalloc(gllmq_ctx *ctx, const void *w_dev, size_t w_b
  * saves the gaps between kernels and keeps the weight stream going.  An entry that does depend on the entries before it carries
  * GLLMQ_DESC_AFTER_PREVIOUS in `flags`: it starts after they have finished.  The batch as a whole
  * is ordered like any other call: it starts after the stream's earlier work and later work
- * starts after all of it. */
+ * starts after all of it.  GLLMQ_DESC_ELEM_F16 / _BF16: x_dev and y_dev of the entry hold elements
+ * of that type (as for gllmq_quantized_matmul_elem; such an entry is a launch of its own). */
 #define GLLMQ_DESC_AFTER_PREVIOUS 1u
+#define GLLMQ_DESC_ELEM_F16 0x100u
+#define GLLMQ_DESC_ELEM_BF16 0x200u
 typedef struct gllmq_matmul_desc {
     const void *w_dev;
     size_t w_bytes;
     const float *x_dev;
     float *y_dev;
     uint32_t ggml_dtype;
-    uint32_t flags; /* 0 or GLLMQ_DESC_AFTER_PREVIOUS */
+    uint32_t flags; /* 0 or GLLMQ_DESC_* bits */
     size_t m, n, k;
 } gllmq_matmul_desc;
 

@@ -20,7 +20,7 @@ pub struct gllmq_matmul_desc {
     pub x_dev: *const f32,
     pub y_dev: *mut f32,
     pub ggml_dtype: u32,
-    pub flags: u32, // 0, or GLLMQ_DESC_AFTER_PREVIOUS when the entry depends on the entries before it
+    pub flags: u32, // GLLMQ_DESC_AFTER_PREVIOUS (1): the entry depends on the entries before it; GLLMQ_DESC_ELEM_F16 (0x100) / _BF16 (0x200): x and y hold such elements
     pub m: usize,
     pub n: usize,
     pub k: usize,

@@ -140,6 +140,25 @@ def test_unaligned_rows_special_values_and_overflow(hip, torch, oracle, elem):
         assert np.isinf(npref.elem_bits_to_f32(got, elem)).any() and np.isfinite(y32).all()
 
 
+def test_batch_entries_of_mixed_element_types(hip, torch):
+    """A batch whose entries hold f32, bf16 and f16 activations: each entry's result equals the
+    single call's, bit for bit (16-bit entries are launches of their own between chained f32 ones)."""
+    print("elem in a batch", flush=True)
+    dt, n, k = Q4_K, 4096, 2048
+    ws = [torch.from_numpy(np.asarray(random_weight(dt, n, k, seed=s)).view(np.uint8).reshape(-1)).cuda() for s in range(6)]
+    kinds = [torch.float32, torch.float32, torch.bfloat16, torch.float16, torch.float32, torch.bfloat16]
+    xs = [torch.from_numpy(random_activations(1, k, seed=10 + i)).cuda().to(t) for i, t in enumerate(kinds)]
+    ys = [torch.full((1, n), float("nan"), device="cuda", dtype=t) for t in kinds]
+    hip.run_batch(hip.make_batch([(w, x, y, dt, 1, n, k) for w, x, y in zip(ws, xs, ys)]))
+    torch.cuda.synchronize()
+    for i, (w, x, y) in enumerate(zip(ws, xs, ys)):
+        alone = torch.empty_like(y)
+        hip.quantized_matmul(w, x, alone, dt, 1, n, k)
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16) if y.dtype != torch.float32 else y,
+                           alone.view(torch.int16) if y.dtype != torch.float32 else alone), f"entry {i}"
+
+
 def test_argument_errors(hip, torch):
     from gllm_amd.backend import BackendError
     print("elem errors", flush=True)
