@@ -190,6 +190,7 @@ struct gllmq_ctx {
     bool use_mm8s = true;                       // "mm8s" = 0: the fetch-and-compute kernels throughout
     bool batch_overlap = true;                  // "batch_overlap" = 0: the kernels of a batch run strictly one after the other
     bool mm8s_all = false;                      // "mm8s_all" = 1: the streamed form wherever it fits, also where another was timed faster
+    bool mm8s_areg = true;                      // "mm8s_areg" = 0: the streamed kernels never keep the digit planes in registers
     uint32_t mm8s_depth = 0;                    // "mm8s_depth": items a loader keeps unconfirmed, 0 = by item size
     uint32_t mm8s_min_rows = 8;                 // "mm8s_min_rows": fewest weight rows per CU that take the streamed form
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
@@ -591,7 +592,7 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     if (ctx->mm8s_depth) depth = std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth);
     while (depth > 2u && slots < items && slots < gq::mm8s_min_slots(depth)) --depth;
     if (slots < items && slots < gq::mm8s_min_slots(depth)) return -1;
-    const bool areg = groups <= 16 && pi <= 1;
+    const bool areg = groups <= 16 && pi <= 1 && ctx->mm8s_areg;
     // Q6_K with more than two activation rows and its operands in LDS needs more registers than
     // a wave of a twelve-wave workgroup has: left to the fetch-and-compute form
     if (kind == MM8_Q6K && pi > 0 && !areg) return -1;
@@ -607,6 +608,10 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     if (!ctx->mm8s_all) {
         if (pi == 2 || (pi == 1 && kind == MM8_Q5K)) return -1;
         if (mm >= 2 && groups > 16) return -1;
+        // one long row over fewer than 16 weight rows per CU: the K split of the other form shares
+        // the row among workgroups (Q4_K 8192 -> 2048: 7.6 against 8.6 us, 8192 -> 3072: 7.9 against
+        // 8.6; Q5_K 8192 -> 2048: 8.4 against 10.0; from 16 rows per CU on the streamed form leads)
+        if (kind != MM8_Q6K && groups > 16 && rows_per_wg < 16) return -1;
         if (kind == MM8_Q6K && !((mm == 1 && groups >= 40) || (mm == 2 && areg))) return -1;
     }
     const uint32_t steps = (((groups + 7u) / 8u + 1u) / 2u) * mm; // preparation steps per wave
@@ -1342,6 +1347,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "batch_overlap") ctx->batch_overlap = value != 0;
     else if (n == "mm8s_all") ctx->mm8s_all = value != 0;
     else if (n == "mm8s_depth") ctx->mm8s_depth = u;
+    else if (n == "mm8s_areg") ctx->mm8s_areg = value != 0;
     else if (n == "mm8s_min_rows") ctx->mm8s_min_rows = std::max(1u, u);
     else if (n == "ffn_fused") ctx->ffn_fused = value != 0;
     else if (n == "mmf_small_min_m") ctx->mmf_small_min_m = u;

@@ -91,12 +91,13 @@ def test_streamed_large_vocabulary_and_repeats(hip, torch, oracle):
 
 def test_default_choice_of_form(torch):
     """Without "mm8s_all" the streamed form runs where it was timed fastest: Q4_K single rows
-    everywhere, Q6_K for one long row or two short ones; the results stay those of the oracle's
+    except long ones over fewer than 16 weight rows per CU, Q6_K for one long row or two short ones; the results stay those of the oracle's
     bar either way (checked against the other form here)."""
     from gllm_amd.backend import HipBackend
     default, plain = HipBackend(0), HipBackend(0, options={"mm8s": 0})
     c = cus(torch)
     for dtype, m, n, k, streamed in ((Q4_K, 1, 56 * c, 4096, True), (Q4_K, 2, 16 * c, 14336, False), (Q6_K, 1, 16 * c, 14336, True),
+                                     (Q4_K, 1, 16 * c, 8192, True), (Q4_K, 1, 12 * c, 8192, False), (Q5_K, 1, 8 * c, 8192, False),
                                      (Q6_K, 1, 56 * c, 4096, False), (Q6_K, 2, 56 * c, 4096, True), (Q6_K, 2, 16 * c, 14336, False)):
         print(f"default form dtype={dtype} m={m} n={n} k={k}", flush=True)
         w, x = random_weight(dtype, n, k, seed=5), random_activations(m, k, seed=6)
