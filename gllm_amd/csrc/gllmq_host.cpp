@@ -199,6 +199,7 @@ struct gllmq_ctx {
     hipFunction_t mm8c[2] = {};                 // chains of streamed matmuls in one launch [0 = Q4_K, 1 = Q5_K]
     bool chain_dependent = false;               // "chain_dependent" = 1: entries that depend on the one before stay in the chain
     bool use_chain = true;                      // "chain" = 0: every entry of a batch is a launch of its own
+    uint32_t chain_min_rows = 1;                // "chain_min_rows": fewest weight rows in a CU's share of an entry that joins a chain
     uint32_t chain_spin_limit = 1u << 20;       // "chain_spin_limit": polls of a dependency counter before a workgroup gives up
     uint32_t *chain_error = nullptr;            // host memory the device can write: set when such a wait ran out
     bool mmfs_all = false;                      // "mmfs_all" = 1: the streamed GEMM wherever it fits, also where the other form was timed faster
@@ -969,7 +970,8 @@ bool chain_entry_ok(const gllmq_ctx *ctx, const gllmq_matmul_desc &d, const gllm
     if (!d.w_dev || !d.x_dev || !d.y_dev || !aligned(d.x_dev, 16) || !aligned(d.y_dev, 4) || !aligned(d.w_dev, f->w_align)) return false;
     const size_t rb = gllmq_row_bytes(d.ggml_dtype, d.k);
     if (rb % f->w_align != 0 || d.w_bytes < d.n * rb) return false;
-    return d.n >= static_cast<size_t>(ctx->mm8s_min_rows) * static_cast<size_t>(ctx->num_cus);
+    const size_t cus = static_cast<size_t>(ctx->num_cus);
+    return d.n > 0 && (d.n + cus - 1) / cus >= ctx->chain_min_rows; // rows of the largest share
 }
 
 size_t chain_length(const gllmq_ctx *ctx, const gllmq_matmul_desc *descs, size_t count)
@@ -1034,6 +1036,9 @@ int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t
         if (i > 0 && E.flags) P.e[i - 1].flags |= 2u;
         launched = std::max(launched, E.grid);
     }
+    bool waits = false;
+    for (size_t i = 0; i < len; ++i) waits = waits || P.e[i].flags != 0u;
+    if (!waits) P.done = nullptr; // independent entries count nothing: no counters to set back at the end
     P.launched = launched;
     return launch(ctx, ctx->mm8c[fmt], launched, (gq::MM8C_CWAVES + gq::MM8C_LOADERS) * 64, P.lds_ring + slots * P.slot_bytes,
                   stream, &P, sizeof P, true);
@@ -1339,6 +1344,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "chain") ctx->use_chain = value != 0;
     else if (n == "chain_dependent") ctx->chain_dependent = value != 0;
     else if (n == "chain_spin_limit") ctx->chain_spin_limit = u;
+    else if (n == "chain_min_rows") ctx->chain_min_rows = std::max(1u, u);
     else if (n == "lm_head_fused") ctx->lm_head_fused = value != 0;
     else if (n == "elem_fused") ctx->elem_fused = value != 0;
     else if (n == "ffn_glu_load") ctx->ffn_glu_load = value != 0;

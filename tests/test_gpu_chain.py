@@ -61,6 +61,30 @@ def test_independent_entries_of_different_heights(torch, oracle, dtype, m):
         assert np.array_equal(outs[0][i].view(np.uint32), outs[1][i].view(np.uint32)), f"entry {i}: chained and single launches differ"
 
 
+@pytest.mark.parametrize("dtype,m", [(Q4_K, 1), (Q5_K, 2)])
+def test_entries_with_few_weight_rows_join_the_chain(torch, oracle, dtype, m):
+    """Separate Q, K and V projections of a grouped-query layer (K and V have a quarter of the rows)
+    and smaller ones still, down to fewer rows than CUs: tiles of a few rows, workgroups without a
+    share of an entry.  One launch; against the oracle (a launch of its own would split K across
+    workgroups for such entries and add up in another order)."""
+    from gllm_amd.backend import HipBackend
+    hip = HipBackend(0)
+    c, k = cus(torch), 2048
+    ns = [16 * c, 4 * c, 4 * c, c + 44, 100, 33, 1, 9 * c]
+    host = [(random_weight(dtype, n, k, seed=40 + i), random_activations(m, k, seed=50 + i)) for i, n in enumerate(ns)]
+    entries = [(dev_weight(torch, w), torch.from_numpy(x).cuda(), torch.full((m * n + 64,), float("nan"), device="cuda"), dtype, m, n, k)
+               for (w, x), n in zip(host, ns)]
+    for e, n in zip(entries, ns):
+        e[2][m * n:] = 7.0
+    print(f"chain: small entries dtype={dtype} m={m}", flush=True)
+    run_batch(hip, torch, [(w, x, y[:m * n], dt, mm, n, kk) for (w, x, y, dt, mm, n, kk) in entries], after_previous=None)
+    assert hip.last_kernel_name().startswith("gq_mm8c_"), hip.last_kernel_name()
+    for i, ((w, x), n) in enumerate(zip(host, ns)):
+        got = entries[i][2].cpu().numpy()
+        assert np.all(got[m * n:] == 7.0), f"entry {i}: write past the output"
+        check_close(got[:m * n].reshape(m, n), oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=8), f"entry {i}")
+
+
 def test_every_entry_reads_the_output_of_the_one_before(torch, oracle):
     """y0 = W0 x, y1 = W1 y0, ...: every entry waits inside the launch for the workgroups of the one
     before it and reads what they stored.  Each step is checked against the oracle on the input
