@@ -257,8 +257,10 @@ struct gllmq_ctx {
     // rows call_ldx elements apart (the input of a feed-forward block's down projection); 0 = plain
     uint32_t call_glu = 0, call_glu_off = 0, call_ldx = 0;
     bool ffn_glu_load = true;   // "ffn_glu_load" = 0: the gate activation always runs as a kernel of its own
+    hipFunction_t mm8s_e16[3][6] = {};          // streamed kernels over 16-bit activations and outputs [format][p1_e1_a, p1_e2_a, p2_e4_a, p1_e2, p2_e4, p1_e4]
     hipFunction_t mm8s_glu[3][3] = {};          // streamed kernels that take gated activations [format][p1_e2, p2_e4, p1_e4]
     hipFunction_t gemv_i8_glu[kNumFormats][2] = {};
+    hipFunction_t gemv_i8_e16[kNumFormats][2] = {}; // the integer-dot GEMV over 16-bit activations and outputs
     bool elem_fused = true;     // "elem_fused" = 0: 16-bit elements always through conversion launches
     hipFunction_t convert_elem = nullptr;
     std::mutex err_mutex;
@@ -525,7 +527,10 @@ int launch_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, size_t row_by
     P.glu = ctx->call_glu;
     P.glu_off = ctx->call_glu_off;
     const int fi = format_index(f.dtype);
-    hipFunction_t fn = ctx->gemv_f32 ? ctx->gemv[fi][m - 1] : ctx->call_glu ? ctx->gemv_i8_glu[fi][m - 1] : ctx->gemv_i8[fi][m - 1];
+    hipFunction_t fn = ctx->gemv_f32 ? ctx->gemv[fi][m - 1]
+                     : ctx->call_glu ? ctx->gemv_i8_glu[fi][m - 1]
+                     : ctx->call_elem ? ctx->gemv_i8_e16[fi][m - 1]
+                                      : ctx->gemv_i8[fi][m - 1];
     return launch(ctx, fn, L.grid, L.threads, L.lds, stream, &P, sizeof P);
 }
 
@@ -624,6 +629,10 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
         const int gv = variant == 3 ? 0 : variant == 4 ? 1 : variant == 6 ? 2 : -1;
         if (gv < 0 || !glu_vector_ok(ctx)) return kNeedPlainActivations;
         fn = ctx->mm8s_glu[sfmt][gv];
+    } else if (ctx->call_elem) {
+        const int ev = variant <= 4 ? variant : variant == 6 ? 5 : -1; // no 16-bit build of p4_e4
+        if (ev < 0) return kNeedPlainActivations;
+        fn = ctx->mm8s_e16[sfmt][ev];
     }
     Mm8Params P{};
     P.glu = ctx->call_glu;
@@ -727,7 +736,7 @@ int run_mm8(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         --rows_per_pass;
     if (rows_per_pass == 0) return -1;
     if (one_pass_only && rows_per_pass < m) return -1;
-    if (ctx->call_glu) return kNeedPlainActivations;
+    if (ctx->call_glu || ctx->call_elem) return kNeedPlainActivations; // these kernels read and write f32
     for (size_t m0 = 0; m0 < m; m0 += rows_per_pass) {
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(rows_per_pass, m - m0));
         const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
@@ -741,9 +750,8 @@ int run_mm8(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         P.w2 = w2;
         P.glu_relu = glu_relu ? 1u : 0u;
         P.w = w;
-        P.elem = ctx->call_elem;
-        P.x = elem_at(ctx, x, m0 * k);
-        P.y = elem_at(ctx, y, m0 * n);
+        P.x = x + m0 * k;
+        P.y = y + m0 * n;
         P.n = static_cast<uint32_t>(n);
         P.k = static_cast<uint32_t>(k);
         P.groups = groups;
@@ -1051,6 +1059,8 @@ int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     constexpr size_t kChunk = 16384; // elements of K one launch covers (four waves of 4096)
     if (ctx->call_glu && ctx->gemv_f32) return kNeedPlainActivations;
     const uint32_t ldx = row_stride_x(ctx, k);
+    // 16-bit elements are read as aligned vectors only
+    if (ctx->call_elem && !(aligned(x, 16) && k % 64 == 0 && ldx % 8 == 0)) return kNeedPlainActivations;
     for (size_t m0 = 0; m0 < m; m0 += 2) {
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(2, m - m0));
         for (size_t k0 = 0; k0 < k; k0 += kChunk) {
@@ -1199,6 +1209,9 @@ int gllmq_init(gllmq_ctx **out, int device)
             if (rc != GLLMQ_OK) break;
             snprintf(name, sizeof name, "gq_gemv_i8_%s_m%d_glu", kFormats[i].tag, m);
             rc = get_function(ctx, &ctx->gemv_i8_glu[i][m - 1], name);
+            if (rc != GLLMQ_OK) break;
+            snprintf(name, sizeof name, "gq_gemv_i8_%s_m%d_e16", kFormats[i].tag, m);
+            rc = get_function(ctx, &ctx->gemv_i8_e16[i][m - 1], name);
         }
         if (rc != GLLMQ_OK) break;
         snprintf(name, sizeof name, "gq_gemv_i8_%s_m1_argmax", kFormats[i].tag);
@@ -1284,6 +1297,12 @@ int gllmq_init(gllmq_ctx **out, int device)
             for (int v = 0; v < 7 && rc == GLLMQ_OK; ++v) {
                 snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8s[v]);
                 rc = get_function(ctx, &ctx->mm8s[q][v], name);
+            }
+        static const char *const kMm8sE16[6] = { "p1_e1_a", "p1_e2_a", "p2_e4_a", "p1_e2", "p2_e4", "p1_e4" };
+        for (int q = 0; q < 3; ++q)
+            for (int v = 0; v < 6 && rc == GLLMQ_OK; ++v) {
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s_e16", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8sE16[v]);
+                rc = get_function(ctx, &ctx->mm8s_e16[q][v], name);
             }
         static const char *const kMm8sGlu[3] = { "p1_e2_g", "p2_e4_g", "p1_e4_g" };
         for (int q = 0; q < 3; ++q)
@@ -1568,7 +1587,7 @@ int matmul_elem_on_scratch(gllmq_ctx *ctx, Scratch &S, const void *w, size_t w_b
         rc = dispatch_matmul(ctx, S, *f, static_cast<const uint8_t *>(w), static_cast<const float *>(x),
                              static_cast<float *>(y), m, n, k, false, stream);
         ctx->call_elem = 0;
-        return rc;
+        if (rc != kNeedPlainActivations) return rc; // else: the kernel for this shape reads f32 only
     }
     rc = grow_scratch(ctx, S, &S.elem, &S.elem_bytes, elem_scratch_bytes(m, n, k), stream, "quantized_matmul_elem");
     if (rc != GLLMQ_OK) return rc;

@@ -176,10 +176,11 @@ int gllmq_argmax(gllmq_ctx *ctx, const float *logits_dev, size_t rows, size_t n,
  * x_dev holds m x k and y_dev m x n elements of type `elem`; 16-bit activations widen exactly,
  * the arithmetic is that of gllmq_quantized_matmul, and a result is rounded to the nearest
  * element, ties to even (what E::from_f32 does; NaN stays NaN, f16 overflows to infinity): y is
- * bit for bit the rounded result of the f32 call on the widened activations.  With k <= 16384
- * the kernels convert in their own loads and stores; longer rows take a widening and a rounding
- * launch around the f32 kernels, through scratch of the stream (gllmq_reserve_matmul_elem
- * before capturing such a shape).  Both pointers 4-byte aligned. */
+ * bit for bit the rounded result of the f32 call on the widened activations.  The streamed
+ * kernels, the GEMV (rows that are aligned vectors, k <= 16384) and the GEMM convert in their own
+ * loads and stores; other shapes take a widening and a rounding launch around the f32 kernels,
+ * through scratch of the stream (gllmq_reserve_matmul_elem before capturing such a shape).
+ * Both pointers 4-byte aligned. */
 #define GLLMQ_ELEM_F32 0
 #define GLLMQ_ELEM_F16 1
 #define GLLMQ_ELEM_BF16 2
