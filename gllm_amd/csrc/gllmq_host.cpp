@@ -1622,7 +1622,8 @@ int gllmq_reserve_matmul_elem(gllmq_ctx *ctx, uint32_t dtype, size_t m, size_t n
     if (!ctx) return GLLMQ_ERR_INVALID;
     std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     int rc = gllmq_reserve_matmul(ctx, dtype, m, n, k, stream);
-    if (rc != GLLMQ_OK || elem == GLLMQ_ELEM_F32 || m == 0 || n == 0 || k == 0 || elem_in_kernel(ctx, m, k)) return rc;
+    // (which kernel takes the shape also depends on the pointers' alignment: room for the widened copies either way)
+    if (rc != GLLMQ_OK || elem == GLLMQ_ELEM_F32 || m == 0 || n == 0 || k == 0) return rc;
     Scratch *S = nullptr;
     rc = acquire_scratch(ctx, stream, &S);
     if (rc != GLLMQ_OK) return rc;

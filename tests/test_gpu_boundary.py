@@ -142,6 +142,48 @@ def test_capture_needs_reserved_scratch(torch):
         assert torch.equal(y, eager), f"replay with inputs {seed} differs from the eager call"
 
 
+def test_capture_of_16_bit_elements_through_the_conversion_launches(torch):
+    """A 16-bit call whose kernel reads f32 only (few weight rows: the K-split form) needs room for
+    the widened copies: refused under capture on a fresh stream, fine after reserve_matmul with the
+    element type; replays equal the eager call."""
+    from gllm_amd.backend import BackendError, ELEM_BF16, HipBackend
+    hip = HipBackend(0)
+    dt, m, n, k = Q4_K, 2, 256, 8192
+    w = dev(torch, random_weight(dt, n, k, seed=1))
+    x = torch.from_numpy(random_activations(m, k, seed=2)).cuda().to(torch.bfloat16)
+    y = torch.zeros(m, n, device="cuda", dtype=torch.bfloat16)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    print("boundary: 16-bit capture without scratch", flush=True)
+    graph = torch.cuda.CUDAGraph()
+    refused = None
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            try:
+                hip.quantized_matmul(w, x, y, dt, m, n, k)
+            except BackendError as e:
+                refused = str(e)
+    torch.cuda.synchronize()
+    assert refused is not None and "reserve" in refused, refused
+    print("boundary: 16-bit reserve, then capture", flush=True)
+    with torch.cuda.stream(side):
+        hip.reserve_matmul(dt, m, n, k, elem=ELEM_BF16)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            hip.quantized_matmul(w, x, y, dt, m, n, k)
+    torch.cuda.synchronize()
+    eager = torch.empty_like(y)
+    for seed in (3, 4):
+        x.copy_(torch.from_numpy(random_activations(m, k, seed=seed)).to(torch.bfloat16))
+        hip.quantized_matmul(w, x, eager, dt, m, n, k)
+        torch.cuda.synchronize()
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), eager.view(torch.int16)), f"replay with inputs {seed} differs from the eager call"
+
+
 def test_host_slices_are_uploaded_once(torch, oracle):
     """The reference's signature hands over host slices on every call; the same weight slice is
     copied to the device on its first use only, until the caller says it has changed."""
