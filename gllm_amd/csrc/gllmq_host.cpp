@@ -592,9 +592,14 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     const uint32_t items = wg_tiles * groups;
     uint32_t slots = std::min(items, (160u * 1024u - std::min(fixed, 160u * 1024u)) / item_bytes);
     if (slots < items) slots -= slots % gq::MM8S_LOADERS; // a reused ring is a whole number of rounds of the loaders
-    // items a loader keeps unconfirmed: about MM8S_DEPTH_BYTES worth of them, fewer when a reused
-    // ring is too short for that many
-    uint32_t depth = std::min(gq::MM8S_MAX_DEPTH, std::max(2u, (gq::MM8S_DEPTH_BYTES + item_bytes / 2u) / item_bytes));
+    // Items a loader keeps unconfirmed.  One or two activation rows: one item (the wave requests an
+    // item, waits for the one before it and confirms that: an arithmetic wave sees an item as soon
+    // as it is there; with more outstanding the stream got no faster and the items later: one row
+    // 4096 -> 4096 5.30 against 5.95 us, 4096 -> 14336 8.46 against 8.56, 4096 -> 128256 53.5
+    // against 55.4, two rows of Q6_K 4096 -> 14336 12.7 against 13.4).  Three and four rows, whose
+    // arithmetic per item is longer, keep about MM8S_DEPTH_BYTES worth of items on their way
+    // (three rows 4096 -> 6144: 6.6 against 6.9 us with one), fewer when a reused ring is too short.
+    uint32_t depth = pi == 0 ? 1u : std::min(gq::MM8S_MAX_DEPTH, std::max(2u, (gq::MM8S_DEPTH_BYTES + item_bytes / 2u) / item_bytes));
     if (ctx->mm8s_depth) depth = std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth);
     while (depth > 2u && slots < items && slots < gq::mm8s_min_slots(depth)) --depth;
     if (slots < items && slots < gq::mm8s_min_slots(depth)) return -1;
@@ -1016,7 +1021,7 @@ int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t
     P.lds_ctrl = (prep.red + 15u) & ~15u;
     const uint32_t red = P.lds_ctrl + static_cast<uint32_t>(sizeof(gq::Mm8sCtrl)) + gq::MM8C_MAX_SLOTS * 4u;
     P.lds_ring = (red + gq::MM8C_RED_BUFS * gq::MM8C_CWAVES * 64u * 4u + 1023u) & ~1023u;
-    P.depth = 2;
+    P.depth = ctx->mm8s_depth ? std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth) : 1u; // as for the single launches of one or two rows
     if (P.lds_ring >= 160u * 1024u) return -1;
     uint32_t slots = std::min(gq::MM8C_MAX_SLOTS, (160u * 1024u - P.lds_ring) / P.slot_bytes);
     slots -= slots % gq::MM8C_LOADERS;
