@@ -906,7 +906,7 @@ MmfsPlan plan_mmfs(const gllmq_ctx *ctx, const Format &f, size_t m, size_t n, si
     const uint32_t items = L.wg_tiles * gq::MMFS_CWAVES;
     L.slots = std::min(items, (160u * 1024u - L.lds_ring) / item_bytes);
     if (L.slots < items) L.slots -= L.slots % gq::MMFS_LOADERS; // a reused ring is a whole number of rounds of the loaders
-    L.depth = std::min(gq::MM8S_MAX_DEPTH, std::max(2u, (gq::MM8S_DEPTH_BYTES + item_bytes / 2u) / item_bytes));
+    L.depth = ctx->mm8s_depth ? std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth) : 1u; // as for the one-row kernels (12.7 against 12.8 us at 32 x 4096 x 4096, 10.5 against 10.8 at 2048 x 2048)
     while (L.depth > 2u && L.slots < items && L.slots < gq::mm8s_min_slots(L.depth)) --L.depth;
     if (L.slots < items && L.slots < gq::mm8s_min_slots(L.depth)) return L;
     L.lds = L.lds_ring + L.slots * item_bytes;
