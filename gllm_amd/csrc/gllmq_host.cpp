@@ -190,6 +190,7 @@ struct gllmq_ctx {
     bool use_mm8s = true;                       // "mm8s" = 0: the fetch-and-compute kernels throughout
     bool batch_overlap = true;                  // "batch_overlap" = 0: the kernels of a batch run strictly one after the other
     bool mm8s_all = false;                      // "mm8s_all" = 1: the streamed form wherever it fits, also where another was timed faster
+    bool mm8_small_to_gemv = true;              // "mm8_small_to_gemv" = 0: one Q4_K row over few weight rows stays on the matrix-core kernels
     bool mm8s_areg = true;                      // "mm8s_areg" = 0: the streamed kernels never keep the digit planes in registers
     uint32_t mm8s_depth = 0;                    // "mm8s_depth": items a loader keeps unconfirmed, 0 = by item size
     uint32_t mm8s_min_rows = 8;                 // "mm8s_min_rows": fewest weight rows per CU that take the streamed form
@@ -582,7 +583,12 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     // the tiles are lower than the 32 rows the matrix cores multiply, which costs nothing here (the
     // stream bounds the kernel).  Below `mm8s_min_rows` rows per CU the K split of the other form,
     // which keeps whole tiles and shares their blocks between CUs, is left to do it.
-    if (n < static_cast<size_t>(ctx->mm8s_min_rows) * cus) return -1;
+    // (two rows and more: from 4 rows per CU, where the K split of the other form and the GEMV are
+    // behind: 2 x 4096 -> 1024 Q4_K 5.1-5.4 against 5.9-6.1 and 5.5-5.7 us)
+    const uint32_t min_rows = m >= 2 ? std::min(ctx->mm8s_min_rows, 4u) : ctx->mm8s_min_rows;
+    if (n < static_cast<size_t>(min_rows) * cus) return -1;
+    // one row of Q5_K over fewer than 12 weight rows per CU: the integer-dot GEMV is ahead (4096 -> 2048: 4.8-5.2 against 5.6 us)
+    if (!ctx->mm8s_all && kind == MM8_Q5K && m == 1 && n < static_cast<size_t>(12) * cus) return -1;
     const uint32_t rows_per_wg = static_cast<uint32_t>((n + cus - 1) / cus);
     const uint32_t grid = static_cast<uint32_t>((n + rows_per_wg - 1) / rows_per_wg);
     const uint32_t mm = static_cast<uint32_t>(m), pi = mm <= 2 ? 0u : (mm <= 4 ? 1u : 2u), pairs = 1u << pi;
@@ -701,6 +707,10 @@ int run_mm8(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
     if (kind == MM8_Q5K && !glu && (ctx->mm8_q5k_min_m == 0 || (m < ctx->mm8_q5k_min_m && !long_single))) return -1;
     if (kind == MM8_Q8_0 && (ctx->mm8_q8_0_min_m == 0 || (m < ctx->mm8_q8_0_min_m && !gemv_cramped))) return -1;
     if (kind == MM8_Q8_0 && k < 256) return -1; // its fetch window is one whole group of 8 blocks
+    // One row of Q4_K over at most 4 weight rows per CU: a workgroup's prologue and the meeting of
+    // the K slices outweigh what the matrix cores save, the integer-dot GEMV is ahead
+    // (4096 -> 1024: 4.5-4.7 against 5.1-5.3 us, 8192 -> 1024: 6.2-6.3 against 7.4, 14336 -> 512: 8.4 against 9.4).
+    if (kind == MM8_Q4K && m == 1 && !glu && ctx->mm8_small_to_gemv && n <= static_cast<size_t>(4) * static_cast<size_t>(ctx->num_cus)) return -1;
     if (!aligned(x, 16) || k % 8 != 0) return -1; // the kernel loads activations as aligned vectors
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
     // K split: with tiles for at most half of the CUs, 2..8 workgroups share each tile and take
@@ -1378,6 +1388,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "mm8s_all") ctx->mm8s_all = value != 0;
     else if (n == "mm8s_depth") ctx->mm8s_depth = u;
     else if (n == "mm8s_areg") ctx->mm8s_areg = value != 0;
+    else if (n == "mm8_small_to_gemv") ctx->mm8_small_to_gemv = value != 0;
     else if (n == "mm8s_min_rows") ctx->mm8s_min_rows = std::max(1u, u);
     else if (n == "ffn_fused") ctx->ffn_fused = value != 0;
     else if (n == "mmf_small_min_m") ctx->mmf_small_min_m = u;

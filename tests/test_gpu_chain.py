@@ -43,7 +43,8 @@ def test_independent_entries_of_different_heights(torch, oracle, dtype, m):
     """The matmuls of a decoder layer that share K: different numbers of weight rows, so different
     tile heights and numbers of workgroups per entry, one launch."""
     from gllm_amd.backend import HipBackend
-    hip, plain = HipBackend(0), HipBackend(0, options={"chain": 0})
+    # (single launches in the streamed form throughout: by default a short Q5_K entry would take the GEMV)
+    hip, plain = HipBackend(0), HipBackend(0, options={"chain": 0, "mm8s_all": 1})
     c, k = cus(torch), 4096
     ns = [24 * c, 16 * c, 112 * c + 5, 8 * c, 56 * c + 31]
     host = [(random_weight(dtype, n, k, seed=i), random_activations(m, k, seed=10 + i)) for i, n in enumerate(ns)]

@@ -135,7 +135,7 @@ FAMILIES = [
     ("streamed int8 long rows", {"mm8s_all": 1}, 2, lambda c: 8 * c, 14336, [Q4_K, Q6_K], lambda k: 32 + k / 2048, "gq_mm8s_"),
     ("int8 matrix cores", {"mm8s": 0, "mm8_q5k_min_m": 1, "mm8_q6k_min_m": 1, "mm8_q8_0_min_m": 1}, 4, lambda c: 300, 2048 + 256, ALL,
      lambda k: 32 + k / 2048, "gq_mm8_"),
-    ("int8 matrix cores, K split", {"mm8s": 0, "mm8_q5k_min_m": 1, "mm8_q6k_min_m": 1}, 1, lambda c: 96, 14336, [Q4_K, Q5_K, Q6_K],
+    ("int8 matrix cores, K split", {"mm8s": 0, "mm8_q5k_min_m": 1, "mm8_q6k_min_m": 1, "mm8_small_to_gemv": 0}, 1, lambda c: 96, 14336, [Q4_K, Q5_K, Q6_K],
      lambda k: 40 + k / 2048, "gq_mm8_"),
     ("integer-dot GEMV", {"mm8": 0, "mmf": 0}, 2, lambda c: 257, 4096 - 64, ALL, lambda k: 32 + k / 2048, "gq_gemv_i8_"),
     ("f32 multiply-add GEMV", {"gemv_f32": 1, "mm8": 0, "mmf": 0}, 1, lambda c: 130, 2048, ALL, lambda k: 160, "gq_gemv_"),
