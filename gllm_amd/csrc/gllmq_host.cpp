@@ -258,6 +258,8 @@ struct gllmq_ctx {
     // rows call_ldx elements apart (the input of a feed-forward block's down projection); 0 = plain
     uint32_t call_glu = 0, call_glu_off = 0, call_ldx = 0;
     bool ffn_glu_load = true;   // "ffn_glu_load" = 0: the gate activation always runs as a kernel of its own
+    hipFunction_t mm8s_gated[2][3] = {};        // streamed gate/up kernels with act(g) * u at the end of a tile pair [Q4_K, Q5_K][p1_e1_a, p1_e2_a, p2_e4_a]
+    bool ffn_streamed = true;                   // "ffn_streamed" = 0: gllmq_ffn_swiglu never uses them
     hipFunction_t mm8s_e16[3][6] = {};          // streamed kernels over 16-bit activations and outputs [format][p1_e1_a, p1_e2_a, p2_e4_a, p1_e2, p2_e4, p1_e4]
     hipFunction_t mm8s_glu[3][3] = {};          // streamed kernels that take gated activations [format][p1_e2, p2_e4, p1_e4]
     hipFunction_t gemv_i8_glu[kNumFormats][2] = {};
@@ -566,10 +568,14 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
 // Q4_K and Q5_K with up to 8 rows in the streamed form (mm8s.hip.inc): taken when the weight rows
 // give every CU at least one 32-row tile, one pass over the weights serves all activation rows and
 // the LDS ring holds enough items.  Returns -1 when the shape is not for it.
+// `w2` != null selects the gated form: `w` holds the n gate rows, `w2` the n up rows, and
+// y = act(gate . x) * (up . x) (Q4_K and Q5_K, rows of up to 4096 elements, up to four activation rows).
 int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n, size_t k,
-             bool act_bf16, void *stream)
+             bool act_bf16, void *stream, const uint8_t *w2 = nullptr, bool glu_relu = false)
 {
     const int kind = mm8_kind(f.dtype);
+    const bool glu = w2 != nullptr;
+    if (glu && ((kind != MM8_Q4K && kind != MM8_Q5K) || m > 4 || k > 4096 || ctx->call_glu || ctx->call_elem)) return -1;
     if (!ctx->use_mm8 || !ctx->use_mm8s || (kind != MM8_Q4K && kind != MM8_Q5K && kind != MM8_Q6K) || m == 0 || m > 8) return -1;
     if (kind == MM8_Q5K && ctx->mm8_q5k_min_m == 0) return -1;
     if (kind == MM8_Q6K && ctx->mm8_q6k_min_m == 0) return -1;
@@ -594,8 +600,8 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     const uint32_t mm = static_cast<uint32_t>(m), pi = mm <= 2 ? 0u : (mm <= 4 ? 1u : 2u), pairs = 1u << pi;
     const uint32_t wg_tiles = (rows_per_wg + 31u) / 32u, tile_rows = (rows_per_wg + wg_tiles - 1u) / wg_tiles;
     const uint32_t item_bytes = tile_rows * pieces * 16u; // a row of an item in LDS: its 16-byte pieces side by side
-    const uint32_t fixed = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, 0, subs).total;
-    const uint32_t items = wg_tiles * groups;
+    const uint32_t fixed = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, 0, subs, glu).total;
+    const uint32_t items = (glu ? 2u : 1u) * wg_tiles * groups; // (gated: a gate tile and an up tile per tile of rows)
     uint32_t slots = std::min(items, (160u * 1024u - std::min(fixed, 160u * 1024u)) / item_bytes);
     if (slots < items) slots -= slots % gq::MM8S_LOADERS; // a reused ring is a whole number of rounds of the loaders
     // Items a loader keeps unconfirmed.  One or two activation rows: one item (the wave requests an
@@ -622,6 +628,7 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     // for a low tile as for a full one.
     // Five to eight activation rows, and three or four of Q5_K, need more registers here than a
     // wave of a twelve-wave workgroup has (6 x 2048 -> 14336 Q4_K: 16.1 against 11.0 us).
+    if (glu && !areg) return -1;
     if (!ctx->mm8s_all) {
         if (pi == 2 || (pi == 1 && kind == MM8_Q5K)) return -1;
         if (mm >= 2 && groups > 16) return -1;
@@ -636,7 +643,9 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     if (areg) variant = pi == 1 ? 2 : (steps <= 1 ? 0 : 1);
     else variant = (pi == 0 && steps > 2) ? 6 : 3 + static_cast<int>(pi);
     hipFunction_t fn = ctx->mm8s[sfmt][variant];
-    if (ctx->call_glu) {
+    if (glu) {
+        fn = ctx->mm8s_gated[sfmt][variant]; // areg: variants 0, 1, 2
+    } else if (ctx->call_glu) {
         const int gv = variant == 3 ? 0 : variant == 4 ? 1 : variant == 6 ? 2 : -1;
         if (gv < 0 || !glu_vector_ok(ctx)) return kNeedPlainActivations;
         fn = ctx->mm8s_glu[sfmt][gv];
@@ -649,6 +658,8 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     P.glu = ctx->call_glu;
     P.glu_off = ctx->call_glu_off;
     P.w = w;
+    P.w2 = w2;
+    P.glu_relu = glu_relu ? 1u : 0u;
     P.x = x;
     P.y = y;
     P.n = static_cast<uint32_t>(n);
@@ -669,7 +680,7 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     P.wg_tiles = wg_tiles;
     P.last_wg_rows = P.n - (grid - 1u) * rows_per_wg;
     P.last_wg_tiles = (P.last_wg_rows + tile_rows - 1u) / tile_rows;
-    const gq::Mm8sLds L = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, slots, subs);
+    const gq::Mm8sLds L = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, slots, subs, glu);
     P.lds_ctrl = L.ctrl;
     P.lds_ring = L.ring;
     P.depth = depth;
@@ -1313,6 +1324,11 @@ int gllmq_init(gllmq_ctx **out, int device)
                 snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8s[v]);
                 rc = get_function(ctx, &ctx->mm8s[q][v], name);
             }
+        for (int q = 0; q < 2; ++q)
+            for (int v = 0; v < 3 && rc == GLLMQ_OK; ++v) {
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s_glu", q ? "q5k" : "q4k", kMm8s[v]);
+                rc = get_function(ctx, &ctx->mm8s_gated[q][v], name);
+            }
         static const char *const kMm8sE16[6] = { "p1_e1_a", "p1_e2_a", "p2_e4_a", "p1_e2", "p2_e4", "p1_e4" };
         for (int q = 0; q < 3; ++q)
             for (int v = 0; v < 6 && rc == GLLMQ_OK; ++v) {
@@ -1382,6 +1398,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "lm_head_fused") ctx->lm_head_fused = value != 0;
     else if (n == "elem_fused") ctx->elem_fused = value != 0;
     else if (n == "ffn_glu_load") ctx->ffn_glu_load = value != 0;
+    else if (n == "ffn_streamed") ctx->ffn_streamed = value != 0;
     else if (n == "mmfs_all") ctx->mmfs_all = value != 0;
     else if (n == "mmfs_min_rows") ctx->mmfs_min_rows = std::max(1u, u);
     else if (n == "batch_overlap") ctx->batch_overlap = value != 0;
@@ -1685,7 +1702,8 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_
 
     // gate and up in one launch with the activation in its epilogue (Q4_K / Q5_K, up to 8 rows)
     rc = -1;
-    if (ctx->ffn_fused && m <= 8) rc = run_mm8(ctx, S, *fg, gw, x, h, m, ffn, hidden, false, stream, true, uw, relu_gate != 0);
+    if (ctx->ffn_fused && ctx->ffn_streamed && m <= 4) rc = run_mm8s(ctx, *fg, gw, x, h, m, ffn, hidden, false, stream, uw, relu_gate != 0);
+    if (rc < 0 && ctx->ffn_fused && m <= 8) rc = run_mm8(ctx, S, *fg, gw, x, h, m, ffn, hidden, false, stream, true, uw, relu_gate != 0);
     if (rc > 0) return rc;
     if (rc < 0) {
         // three steps: the two products (one matmul when the up rows follow the gate rows in

@@ -170,14 +170,16 @@ struct Mm8sLds {
     uint32_t ctrl, red, ring, total;
 };
 
+// `glu`: the gated kernels keep the sums of a gate tile (pairs x 64 floats) behind the partial sums
+// until the up tile of the same rows is summed.
 GQ_HD inline Mm8sLds mm8s_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, uint32_t item_bytes, uint32_t slots,
-                                     uint32_t subs = 8u)
+                                     uint32_t subs = 8u, bool glu = false)
 {
     Mm8sLds L;
     L.prep = mm8_lds_layout(groups, m, pairs, subs, 0u);
     L.ctrl = (L.prep.red + 15u) & ~15u; // the area of mm8.hip.inc's partial sums and stages is not used here
     L.red = L.ctrl + static_cast<uint32_t>(sizeof(Mm8sCtrl));
-    L.ring = (L.red + MM8S_RED_BUFS * MM8S_CWAVES * pairs * 64u * 4u + 1023u) & ~1023u;
+    L.ring = (L.red + MM8S_RED_BUFS * MM8S_CWAVES * pairs * 64u * 4u + (glu ? pairs * 64u * 4u : 0u) + 1023u) & ~1023u;
     L.total = L.ring + slots * item_bytes;
     return L;
 }
