@@ -258,7 +258,7 @@ struct gllmq_ctx {
     // rows call_ldx elements apart (the input of a feed-forward block's down projection); 0 = plain
     uint32_t call_glu = 0, call_glu_off = 0, call_ldx = 0;
     bool ffn_glu_load = true;   // "ffn_glu_load" = 0: the gate activation always runs as a kernel of its own
-    hipFunction_t mm8s_gated[2][3] = {};        // streamed gate/up kernels with act(g) * u at the end of a tile pair [Q4_K, Q5_K][p1_e1_a, p1_e2_a, p2_e4_a]
+    hipFunction_t mm8s_gated[2][6] = {};        // streamed gate/up kernels with act(g) * u at the end of a tile pair [Q4_K, Q5_K][p1_e1_a, p1_e2_a, p2_e4_a, p1_e2, p2_e4, p1_e4]
     bool ffn_streamed = true;                   // "ffn_streamed" = 0: gllmq_ffn_swiglu never uses them
     hipFunction_t mm8s_e16[3][6] = {};          // streamed kernels over 16-bit activations and outputs [format][p1_e1_a, p1_e2_a, p2_e4_a, p1_e2, p2_e4, p1_e4]
     hipFunction_t mm8s_glu[3][3] = {};          // streamed kernels that take gated activations [format][p1_e2, p2_e4, p1_e4]
@@ -569,13 +569,13 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
 // give every CU at least one 32-row tile, one pass over the weights serves all activation rows and
 // the LDS ring holds enough items.  Returns -1 when the shape is not for it.
 // `w2` != null selects the gated form: `w` holds the n gate rows, `w2` the n up rows, and
-// y = act(gate . x) * (up . x) (Q4_K and Q5_K, rows of up to 4096 elements, up to four activation rows).
+// y = act(gate . x) * (up . x) (Q4_K and Q5_K, up to four activation rows).
 int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n, size_t k,
              bool act_bf16, void *stream, const uint8_t *w2 = nullptr, bool glu_relu = false)
 {
     const int kind = mm8_kind(f.dtype);
     const bool glu = w2 != nullptr;
-    if (glu && ((kind != MM8_Q4K && kind != MM8_Q5K) || m > 4 || k > 4096 || ctx->call_glu || ctx->call_elem)) return -1;
+    if (glu && ((kind != MM8_Q4K && kind != MM8_Q5K) || m > 4 || ctx->call_glu || ctx->call_elem)) return -1;
     if (!ctx->use_mm8 || !ctx->use_mm8s || (kind != MM8_Q4K && kind != MM8_Q5K && kind != MM8_Q6K) || m == 0 || m > 8) return -1;
     if (kind == MM8_Q5K && ctx->mm8_q5k_min_m == 0) return -1;
     if (kind == MM8_Q6K && ctx->mm8_q6k_min_m == 0) return -1;
@@ -628,7 +628,6 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     // for a low tile as for a full one.
     // Five to eight activation rows, and three or four of Q5_K, need more registers here than a
     // wave of a twelve-wave workgroup has (6 x 2048 -> 14336 Q4_K: 16.1 against 11.0 us).
-    if (glu && !areg) return -1;
     if (!ctx->mm8s_all) {
         if (pi == 2 || (pi == 1 && kind == MM8_Q5K)) return -1;
         if (mm >= 2 && groups > 16) return -1;
@@ -644,7 +643,9 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     else variant = (pi == 0 && steps > 2) ? 6 : 3 + static_cast<int>(pi);
     hipFunction_t fn = ctx->mm8s[sfmt][variant];
     if (glu) {
-        fn = ctx->mm8s_gated[sfmt][variant]; // areg: variants 0, 1, 2
+        const int gv = variant <= 4 ? variant : variant == 6 ? 5 : -1; // no gated build of p4_e4
+        if (gv < 0) return -1;
+        fn = ctx->mm8s_gated[sfmt][gv];
     } else if (ctx->call_glu) {
         const int gv = variant == 3 ? 0 : variant == 4 ? 1 : variant == 6 ? 2 : -1;
         if (gv < 0 || !glu_vector_ok(ctx)) return kNeedPlainActivations;
@@ -1324,9 +1325,10 @@ int gllmq_init(gllmq_ctx **out, int device)
                 snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8s[v]);
                 rc = get_function(ctx, &ctx->mm8s[q][v], name);
             }
+        static const char *const kMm8sGated[6] = { "p1_e1_a", "p1_e2_a", "p2_e4_a", "p1_e2", "p2_e4", "p1_e4" };
         for (int q = 0; q < 2; ++q)
-            for (int v = 0; v < 3 && rc == GLLMQ_OK; ++v) {
-                snprintf(name, sizeof name, "gq_mm8s_%s_%s_glu", q ? "q5k" : "q4k", kMm8s[v]);
+            for (int v = 0; v < 6 && rc == GLLMQ_OK; ++v) {
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s_glu", q ? "q5k" : "q4k", kMm8sGated[v]);
                 rc = get_function(ctx, &ctx->mm8s_gated[q][v], name);
             }
         static const char *const kMm8sE16[6] = { "p1_e1_a", "p1_e2_a", "p2_e4_a", "p1_e2", "p2_e4", "p1_e4" };

@@ -74,7 +74,8 @@ def test_ffn_all_format_pairs(hip, torch, oracle, t_gu, t_dn):
 @pytest.mark.parametrize("t_gu", [Q4_K, Q5_K])
 def test_ffn_ragged_shapes_and_relu_gate(hip, torch, oracle, t_gu):
     # ffn not a multiple of 32 (a partial last tile in both halves), hidden with 2 and 3 passes per tile
-    for hidden, ffn, m, relu in [(2560, 1000, 1, False), (4096, 776, 2, True), (6144, 520, 4, False), (512, 33, 7, True)]:
+    for hidden, ffn, m, relu in [(2560, 1000, 1, False), (4096, 776, 2, True), (6144, 520, 4, False), (512, 33, 7, True),
+                                 (6144, 2100, 1, True), (8192, 2048, 1, False), (1024, 2304, 3, False)]:
         print(f"ffn ragged gate/up={t_gu} hidden={hidden} ffn={ffn} m={m} relu={relu}", flush=True)
         gate, up = random_weight(t_gu, ffn, hidden, seed=ffn), random_weight(t_gu, ffn, hidden, seed=ffn + 1)
         down = random_weight(Q8_0, hidden, ffn, seed=ffn + 2)
