@@ -262,6 +262,11 @@ struct gllmq_ctx {
     bool ffn_streamed = true;                   // "ffn_streamed" = 0: gllmq_ffn_swiglu never uses them
     hipFunction_t mm8s_e16[3][6] = {};          // streamed kernels over 16-bit activations and outputs [format][p1_e1_a, p1_e2_a, p2_e4_a, p1_e2, p2_e4, p1_e4]
     hipFunction_t mm8s_glu[3][3] = {};          // streamed kernels that take gated activations [format][p1_e2, p2_e4, p1_e4]
+    // streamed kernels whose items are pairs of blocks of a tile of at most 16 weight rows (one
+    // activation row) [format][p1_e1_a, p1_e2_a, p1_e2, p1_e4, p1_e2 and p1_e4 over gated activations,
+    // the first four over a 16-bit element type]
+    hipFunction_t mm8s_fold[3][10] = {};
+    bool mm8s_fold_on = true;                   // "mm8s_fold" = 0: such tiles go block by block, half of the matrix-core columns idle
     hipFunction_t gemv_i8_glu[kNumFormats][2] = {};
     hipFunction_t gemv_i8_e16[kNumFormats][2] = {}; // the integer-dot GEMV over 16-bit activations and outputs
     bool elem_fused = true;     // "elem_fused" = 0: 16-bit elements always through conversion launches
@@ -591,17 +596,24 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     // which keeps whole tiles and shares their blocks between CUs, is left to do it.
     // (two rows and more: from 4 rows per CU, where the K split of the other form and the GEMV are
     // behind: 2 x 4096 -> 1024 Q4_K 5.1-5.4 against 5.9-6.1 and 5.5-5.7 us)
-    const uint32_t min_rows = m >= 2 ? std::min(ctx->mm8s_min_rows, 4u) : ctx->mm8s_min_rows;
+    // (one row, in pairs of blocks: likewise from 4 rows per CU, 8192 -> 1536 Q4_K 5.8 against 7.3 us,
+    // 14336 -> 1024 6.8 against 9.1, Q6_K 8.7 against 11.8)
+    const bool may_fold = ctx->mm8s_fold_on && m == 1 && !glu;
+    const uint32_t min_rows = (m >= 2 || may_fold) ? std::min(ctx->mm8s_min_rows, 4u) : ctx->mm8s_min_rows;
     if (n < static_cast<size_t>(min_rows) * cus) return -1;
-    // one row of Q5_K over fewer than 12 weight rows per CU: the integer-dot GEMV is ahead (4096 -> 2048: 4.8-5.2 against 5.6 us)
-    if (!ctx->mm8s_all && kind == MM8_Q5K && m == 1 && n < static_cast<size_t>(12) * cus) return -1;
     const uint32_t rows_per_wg = static_cast<uint32_t>((n + cus - 1) / cus);
     const uint32_t grid = static_cast<uint32_t>((n + rows_per_wg - 1) / rows_per_wg);
     const uint32_t mm = static_cast<uint32_t>(m), pi = mm <= 2 ? 0u : (mm <= 4 ? 1u : 2u), pairs = 1u << pi;
     const uint32_t wg_tiles = (rows_per_wg + 31u) / 32u, tile_rows = (rows_per_wg + wg_tiles - 1u) / wg_tiles;
-    const uint32_t item_bytes = tile_rows * pieces * 16u; // a row of an item in LDS: its 16-byte pieces side by side
+    // One activation row over tiles of at most 16 weight rows: an item is a pair of blocks of the
+    // tile, so that all 32 columns of the matrix cores carry weights (14336 -> 4096 is bound by the
+    // arithmetic, not by the stream, when half of them idle).
+    const bool fold = may_fold && tile_rows <= 16 && groups > 8; // (up to 8 blocks there is nothing to pair: a block per wave)
+    if (may_fold && !fold && n < static_cast<size_t>(ctx->mm8s_min_rows) * cus) return -1;
+    const uint32_t ipt = fold ? gq::mm8s_fold_pairs(groups) : groups; // items per tile
+    const uint32_t item_bytes = (fold ? 2u : 1u) * tile_rows * pieces * 16u; // a row of an item in LDS: its 16-byte pieces side by side
     const uint32_t fixed = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, 0, subs, glu).total;
-    const uint32_t items = (glu ? 2u : 1u) * wg_tiles * groups; // (gated: a gate tile and an up tile per tile of rows)
+    const uint32_t items = (glu ? 2u : 1u) * wg_tiles * ipt; // (gated: a gate tile and an up tile per tile of rows)
     uint32_t slots = std::min(items, (160u * 1024u - std::min(fixed, 160u * 1024u)) / item_bytes);
     if (slots < items) slots -= slots % gq::MM8S_LOADERS; // a reused ring is a whole number of rounds of the loaders
     // Items a loader keeps unconfirmed.  One or two activation rows: one item (the wave requests an
@@ -615,7 +627,7 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     if (ctx->mm8s_depth) depth = std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth);
     while (depth > 2u && slots < items && slots < gq::mm8s_min_slots(depth)) --depth;
     if (slots < items && slots < gq::mm8s_min_slots(depth)) return -1;
-    const bool areg = groups <= 16 && pi <= 1 && ctx->mm8s_areg;
+    const bool areg = ipt <= 16 && pi <= 1 && ctx->mm8s_areg && !(fold && ctx->call_glu);
     // Q6_K with more than two activation rows and its operands in LDS needs more registers than
     // a wave of a twelve-wave workgroup has: left to the fetch-and-compute form
     if (kind == MM8_Q6K && pi > 0 && !areg) return -1;
@@ -631,18 +643,35 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     if (!ctx->mm8s_all) {
         if (pi == 2 || (pi == 1 && kind == MM8_Q5K)) return -1;
         if (mm >= 2 && groups > 16) return -1;
-        // one long row over fewer than 16 weight rows per CU: the K split of the other form shares
-        // the row among workgroups (Q4_K 8192 -> 2048: 7.6 against 8.6 us, 8192 -> 3072: 7.9 against
-        // 8.6; Q5_K 8192 -> 2048: 8.4 against 10.0; from 16 rows per CU on the streamed form leads)
-        if (kind != MM8_Q6K && groups > 16 && rows_per_wg < 16) return -1;
-        if (kind == MM8_Q6K && !((mm == 1 && groups >= 40) || (mm == 2 && areg))) return -1;
+        // Tiles of fewer than 16 weight rows block by block, the matrix cores mostly idle, lose to
+        // the K split of the other form for long rows (Q4_K 8192 -> 2048: 7.6 against 8.6 us) and
+        // to the integer-dot GEMV for one row of Q5_K (4096 -> 2048: 4.8-5.2 against 5.6).  In
+        // pairs of blocks they lead (8192 -> 2048: Q4_K 5.8 against 7.5, Q5_K 5.8 against 6.8;
+        // 14336 -> 2048 Q4_K 7.1 against 9.9; Q5_K 4096 -> 2048 4.5 against 4.7).
+        if (!fold && kind != MM8_Q6K && groups > 16 && rows_per_wg < 16) return -1;
+        if (!fold && kind == MM8_Q5K && mm == 1 && n < static_cast<size_t>(12) * cus) return -1;
+        // Q6_K: one row of 40 blocks and more, in pairs of blocks from 20 (5120 -> 4096: 6.4 against 8.1 us, 6144 -> 4096: 7.3 against
+        // 8.7 us for the GEMV, 8192 -> 4096: 9.1 against 10.2; 4096 -> 4096: 6.3 against 6.0), or two short rows
+        if (kind == MM8_Q6K && !((mm == 1 && (groups >= 40 || (fold && groups >= 20))) || (mm == 2 && areg))) return -1;
+        // one short row over at most 4 weight rows per CU: the integer-dot GEMV stays ahead
+        // (4096 -> 1024: Q4_K 4.6 against 5.0 us, Q5_K 4.9 against 5.0; 8192 -> 1024 Q4_K: 6.3 against 5.9 here)
+        if (mm == 1 && rows_per_wg <= 4 && groups <= 16) return -1;
     }
     const uint32_t steps = (((groups + 7u) / 8u + 1u) / 2u) * mm; // preparation steps per wave
     int variant;
     if (areg) variant = pi == 1 ? 2 : (steps <= 1 ? 0 : 1);
     else variant = (pi == 0 && steps > 2) ? 6 : 3 + static_cast<int>(pi);
     hipFunction_t fn = ctx->mm8s[sfmt][variant];
-    if (glu) {
+    if (fold) {
+        // variants 0, 1 (registers), 3, 6 (LDS) of one activation row
+        const int fv = variant <= 1 ? variant : variant == 3 ? 2 : 3;
+        if (ctx->call_glu) {
+            if (!glu_vector_ok(ctx)) return kNeedPlainActivations;
+            fn = ctx->mm8s_fold[sfmt][fv + 2];
+        } else {
+            fn = ctx->mm8s_fold[sfmt][ctx->call_elem ? fv + 6 : fv];
+        }
+    } else if (glu) {
         const int gv = variant <= 4 ? variant : variant == 6 ? 5 : -1; // no gated build of p4_e4
         if (gv < 0) return -1;
         fn = ctx->mm8s_gated[sfmt][gv];
@@ -1069,10 +1098,12 @@ int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t
         E.last_wg_tiles = (E.last_wg_rows + E.tile_rows - 1u) / E.tile_rows;
         E.flags = i > 0 ? (d.flags & 1u) : 0u; // the chain's first entry is ordered by the stream
         if (i > 0 && E.flags) P.e[i - 1].flags |= 2u;
+        // one activation row over tiles of at most 16 weight rows: in pairs of blocks, as run_mm8s() would
+        if (ctx->mm8s_fold_on && P.m == 1 && E.tile_rows <= 16 && P.groups > 8) E.flags |= 4u;
         launched = std::max(launched, E.grid);
     }
     bool waits = false;
-    for (size_t i = 0; i < len; ++i) waits = waits || P.e[i].flags != 0u;
+    for (size_t i = 0; i < len; ++i) waits = waits || (P.e[i].flags & 3u) != 0u;
     if (!waits) P.done = nullptr; // independent entries count nothing: no counters to set back at the end
     P.launched = launched;
     return launch(ctx, ctx->mm8c[fmt], launched, (gq::MM8C_CWAVES + gq::MM8C_LOADERS) * 64, P.lds_ring + slots * P.slot_bytes,
@@ -1337,6 +1368,13 @@ int gllmq_init(gllmq_ctx **out, int device)
                 snprintf(name, sizeof name, "gq_mm8s_%s_%s_e16", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8sE16[v]);
                 rc = get_function(ctx, &ctx->mm8s_e16[q][v], name);
             }
+        static const char *const kMm8sFold[10] = { "p1_e1_a_f", "p1_e2_a_f", "p1_e2_f", "p1_e4_f", "p1_e2_g_f", "p1_e4_g_f",
+                                                   "p1_e1_a_f_e16", "p1_e2_a_f_e16", "p1_e2_f_e16", "p1_e4_f_e16" };
+        for (int q = 0; q < 3; ++q)
+            for (int v = 0; v < 10 && rc == GLLMQ_OK; ++v) {
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8sFold[v]);
+                rc = get_function(ctx, &ctx->mm8s_fold[q][v], name);
+            }
         static const char *const kMm8sGlu[3] = { "p1_e2_g", "p2_e4_g", "p1_e4_g" };
         for (int q = 0; q < 3; ++q)
             for (int v = 0; v < 3 && rc == GLLMQ_OK; ++v) {
@@ -1407,6 +1445,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "mm8s_all") ctx->mm8s_all = value != 0;
     else if (n == "mm8s_depth") ctx->mm8s_depth = u;
     else if (n == "mm8s_areg") ctx->mm8s_areg = value != 0;
+    else if (n == "mm8s_fold") ctx->mm8s_fold_on = value != 0;
     else if (n == "mm8_small_to_gemv") ctx->mm8_small_to_gemv = value != 0;
     else if (n == "mm8s_min_rows") ctx->mm8s_min_rows = std::max(1u, u);
     else if (n == "ffn_fused") ctx->ffn_fused = value != 0;

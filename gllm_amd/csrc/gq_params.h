@@ -170,6 +170,15 @@ struct Mm8sLds {
     uint32_t ctrl, red, ring, total;
 };
 
+// The folded form of the streamed kernels (one activation row, tiles of at most 16 weight rows):
+// an item is a pair of blocks of the tile, blocks 16 q + i and 16 q + 8 + i (i < 8) being pair
+// 8 q + i, so that the arithmetic wave of a pair (pair mod 8) is the wave of both of its blocks
+// (block mod 8), as in the form that goes block by block: the same wave prepares the activations
+// of a block either way.  A row whose last group of 16 blocks has 8 or fewer ends in pairs without
+// a second block.
+GQ_HD inline uint32_t mm8s_fold_pairs(uint32_t groups) { return 8u * (groups / 16u) + (groups % 16u < 8u ? groups % 16u : 8u); }
+GQ_HD inline uint32_t mm8s_fold_first(uint32_t pair) { return 16u * (pair >> 3) + (pair & 7u); }
+
 // `glu`: the gated kernels keep the sums of a gate tile (pairs x 64 floats) behind the partial sums
 // until the up tile of the same rows is summed.
 GQ_HD inline Mm8sLds mm8s_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs, uint32_t item_bytes, uint32_t slots,
@@ -259,7 +268,8 @@ struct Mm8ChainEntry {
     // the entry's geometry, worked out by the host as for the streamed kernels: weight rows per
     // workgroup, workgroups that take part, tile height, tiles of a full and of the last
     // workgroup, rows of the last workgroup; flags: bit 0 = starts after the entry before it, bit 1 =
-    // the entry behind it does (so this one says when its y is stored)
+    // the entry behind it does (so this one says when its y is stored), bit 2 = its items are pairs
+    // of blocks (one activation row, tiles of at most 16 rows)
     uint32_t rows_per_wg, grid, tile_rows, wg_tiles, last_wg_tiles, last_wg_rows, flags, pad;
 };
 struct Mm8ChainParams {

@@ -75,6 +75,44 @@ def test_streamed_equals_the_fetch_and_compute_form_bitwise(hip, torch):
             check_close(a, b, f"streamed vs GEMV dtype={dtype} m={m}")
 
 
+@pytest.mark.parametrize("dtype", [Q4_K, Q5_K, Q6_K])
+def test_pairs_of_blocks_over_low_tiles(hip, torch, oracle, dtype):
+    """One activation row over at most 16 weight rows per workgroup: an item is a pair of blocks of
+    the tile (blocks i and i + 8 of every 16).  Rows of whole sixteens of blocks and rows that end
+    in pairs without a second block (9, 10, 12, 15, 20, 24, 33 and 56 blocks), a partial last
+    block, a ragged last workgroup, operands in registers (up to 32 blocks) and in LDS, a reused
+    ring, and tiles of 16 down to 4 rows."""
+    c = cus(torch)
+    cases = [(16 * c, 4096), (16 * c, 14336), (9 * c + 5, 2304), (13 * c - 2, 2560), (8 * c, 8192), (16 * c - 7, 4096 - 8),
+             (5 * c + 1, 3072), (12 * c, 8192 + 256), (4 * c + 3, 6144), (16 * c, 5120), (7 * c, 3840 - 16)]
+    for n, k in cases:
+        print(f"pairs dtype={dtype} n={n} k={k}", flush=True)
+        w, x = random_weight(dtype, n, k, seed=n % 97), random_activations(1, k, seed=k % 89)
+        want = oracle.quantized_matmul(w, x, dtype, 1, n, k, acc=oracle.ACC_F64, threads=16)
+        got = gpu_matmul(hip, torch, w, x, dtype, 1, n, k)
+        name = hip.last_kernel_name()
+        assert name.startswith("gq_mm8s_") and name.endswith("_f"), name
+        check_close(got, want, f"pairs dtype={dtype} n={n} k={k}")
+
+
+def test_pairs_of_blocks_equal_single_blocks_within_the_bar(hip, torch):
+    """The same launches block by block (option "mm8s_fold" = 0): another order of sums, the same
+    bar; and twice in a row, the counters in LDS starting from zero."""
+    from gllm_amd.backend import HipBackend
+    single = HipBackend(0, options={"mm8s_all": 1, "mm8s_fold": 0})
+    c = cus(torch)
+    for dtype, n, k in ((Q4_K, 16 * c, 14336), (Q5_K, 11 * c, 4096), (Q6_K, 16 * c, 11008 + 256 - 11008 % 256)):
+        print(f"pairs vs single dtype={dtype} n={n} k={k}", flush=True)
+        w, x = random_weight(dtype, n, k, seed=21), random_activations(1, k, seed=22)
+        a = gpu_matmul(hip, torch, w, x, dtype, 1, n, k)
+        assert hip.last_kernel_name().endswith("_f"), hip.last_kernel_name()
+        b = gpu_matmul(single, torch, w, x, dtype, 1, n, k)
+        assert single.last_kernel_name().startswith("gq_mm8s_") and not single.last_kernel_name().endswith("_f")
+        check_close(a, b, f"pairs vs single dtype={dtype}")
+        again = gpu_matmul(hip, torch, w, x, dtype, 1, n, k)
+        assert np.array_equal(a.view(np.uint32), again.view(np.uint32))
+
+
 def test_streamed_large_vocabulary_and_repeats(hip, torch, oracle):
     """A Llama-3 vocabulary of Q4_K rows (501 rows per workgroup, 16 tiles, the ring reused eight
     times), twice in a row with different inputs: the counters in LDS start from zero every launch."""
@@ -90,14 +128,18 @@ def test_streamed_large_vocabulary_and_repeats(hip, torch, oracle):
 
 
 def test_default_choice_of_form(torch):
-    """Without "mm8s_all" the streamed form runs where it was timed fastest: Q4_K single rows
-    except long ones over fewer than 16 weight rows per CU, Q6_K for one long row or two short ones; the results stay those of the oracle's
-    bar either way (checked against the other form here)."""
+    """Without "mm8s_all" the streamed form runs where it was timed fastest: single rows of Q4_K
+    and Q5_K from 4 weight rows per CU (short rows over exactly 4 excepted), Q6_K for one row of
+    20 blocks and more over at most 16 weight rows per CU, of 40 and more over any number, or two
+    short ones; the results stay those of the oracle's bar either way (checked against the other
+    form here)."""
     from gllm_amd.backend import HipBackend
     default, plain = HipBackend(0), HipBackend(0, options={"mm8s": 0})
     c = cus(torch)
     for dtype, m, n, k, streamed in ((Q4_K, 1, 56 * c, 4096, True), (Q4_K, 2, 16 * c, 14336, False), (Q6_K, 1, 16 * c, 14336, True),
-                                     (Q4_K, 1, 16 * c, 8192, True), (Q4_K, 1, 12 * c, 8192, False), (Q5_K, 1, 8 * c, 8192, False),
+                                     (Q4_K, 1, 16 * c, 8192, True), (Q4_K, 1, 12 * c, 8192, True), (Q5_K, 1, 8 * c, 8192, True),
+                                     (Q4_K, 1, 4 * c, 4096, False), (Q4_K, 1, 4 * c, 8192, True), (Q5_K, 1, 8 * c, 4096, True),
+                                     (Q6_K, 1, 16 * c, 4096, False), (Q6_K, 1, 16 * c, 5120, True), (Q6_K, 1, 24 * c, 5120, False),
                                      (Q6_K, 1, 56 * c, 4096, False), (Q6_K, 2, 56 * c, 4096, True), (Q6_K, 2, 16 * c, 14336, False)):
         print(f"default form dtype={dtype} m={m} n={n} k={k}", flush=True)
         w, x = random_weight(dtype, n, k, seed=5), random_activations(m, k, seed=6)
