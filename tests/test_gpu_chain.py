@@ -86,6 +86,35 @@ def test_entries_with_few_weight_rows_join_the_chain(torch, oracle, dtype, m):
         check_close(got[:m * n].reshape(m, n), oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=8), f"entry {i}")
 
 
+@pytest.mark.parametrize("dtype,m", [(Q4_K, 1), (Q5_K, 1), (Q4_K, 2)])
+def test_entries_that_share_their_activations(torch, oracle, dtype, m):
+    """Q, K and V read the same x, gate and up another, a last entry the first again: a workgroup
+    prepares an x once for the entries in a row that share it (also one that skipped an entry it
+    has no rows of).  Equal to single launches bit for bit, and against the oracle."""
+    from gllm_amd.backend import HipBackend
+    hip, plain = HipBackend(0), HipBackend(0, options={"chain": 0, "mm8s_all": 1})
+    c, k = cus(torch), 4096
+    ns = [16 * c, 4 * c, c // 2, 4 * c + 3, 56 * c, 56 * c, 16 * c]
+    which_x = [0, 0, 0, 0, 1, 1, 0]
+    xs_host = [random_activations(m, k, seed=40 + i) for i in range(2)]
+    ws_host = [random_weight(dtype, n, k, seed=50 + i) for i, n in enumerate(ns)]
+    outs = []
+    for backend in (hip, plain):
+        xs = [torch.from_numpy(x).cuda() for x in xs_host]
+        entries = [(dev_weight(torch, w), xs[xi], torch.full((m, n), float("nan"), device="cuda"), dtype, m, n, k)
+                   for w, n, xi in zip(ws_host, ns, which_x)]
+        print(f"chain: shared x dtype={dtype} m={m} chain={backend is hip}", flush=True)
+        run_batch(backend, torch, entries, after_previous=None)
+        if backend is hip:
+            assert backend.last_kernel_name().startswith("gq_mm8c_"), backend.last_kernel_name()
+        outs.append([e[2].cpu().numpy() for e in entries])
+    for i, (w, n, xi) in enumerate(zip(ws_host, ns, which_x)):
+        want = oracle.quantized_matmul(w, xs_host[xi], dtype, m, n, k, acc=oracle.ACC_F64, threads=16)
+        check_close(outs[0][i], want, f"entry {i}")
+        if n >= 4 * c:  # (fewer rows: a launch of its own splits K across workgroups, another order of sums)
+            assert np.array_equal(outs[0][i].view(np.uint32), outs[1][i].view(np.uint32)), f"entry {i}: chained and single launches differ"
+
+
 def test_every_entry_reads_the_output_of_the_one_before(torch, oracle):
     """y0 = W0 x, y1 = W1 y0, ...: every entry waits inside the launch for the workgroups of the one
     before it and reads what they stored.  Each step is checked against the oracle on the input
