@@ -266,6 +266,10 @@ struct gllmq_ctx {
     // activation row) [format][p1_e1_a, p1_e2_a, p1_e2, p1_e4, p1_e2 and p1_e4 over gated activations,
     // the first four over a 16-bit element type]
     hipFunction_t mm8s_fold[3][10] = {};
+    // streamed kernels whose workgroups share a row range and take a slice of K each (two to four
+    // activation rows over few weight rows) [format][p1_e4, p2_e4][plain, gated activations]
+    hipFunction_t mm8s_split[3][2][2] = {};
+    bool mm8s_split_on = true;                  // "mm8s_split" = 0: such shapes stay on the fetch-and-compute form
     bool mm8s_fold_on = true;                   // "mm8s_fold" = 0: such tiles go block by block, half of the matrix-core columns idle
     hipFunction_t gemv_i8_glu[kNumFormats][2] = {};
     hipFunction_t gemv_i8_e16[kNumFormats][2] = {}; // the integer-dot GEMV over 16-bit activations and outputs
@@ -575,8 +579,10 @@ int check_matmul_args(gllmq_ctx *ctx, const Format *f, const void *w, size_t w_b
 // the LDS ring holds enough items.  Returns -1 when the shape is not for it.
 // `w2` != null selects the gated form: `w` holds the n gate rows, `w2` the n up rows, and
 // y = act(gate . x) * (up . x) (Q4_K and Q5_K, up to four activation rows).
+// `S` != null lets few weight rows under two to four rows of long activations share a row range
+// among workgroups, a slice of K each (the sums meet in S->mm8_part).
 int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n, size_t k,
-             bool act_bf16, void *stream, const uint8_t *w2 = nullptr, bool glu_relu = false)
+             bool act_bf16, void *stream, const uint8_t *w2 = nullptr, bool glu_relu = false, Scratch *S = nullptr)
 {
     const int kind = mm8_kind(f.dtype);
     const bool glu = w2 != nullptr;
@@ -601,18 +607,31 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     const bool may_fold = ctx->mm8s_fold_on && m == 1 && !glu;
     const uint32_t min_rows = (m >= 2 || may_fold) ? std::min(ctx->mm8s_min_rows, 4u) : ctx->mm8s_min_rows;
     if (n < static_cast<size_t>(min_rows) * cus) return -1;
-    const uint32_t rows_per_wg = static_cast<uint32_t>((n + cus - 1) / cus);
-    const uint32_t grid = static_cast<uint32_t>((n + rows_per_wg - 1) / rows_per_wg);
     const uint32_t mm = static_cast<uint32_t>(m), pi = mm <= 2 ? 0u : (mm <= 4 ? 1u : 2u), pairs = 1u << pi;
+    // K split: two to four activation rows of at least 32 blocks over 32-row tiles for at most half
+    // of the CUs.  Every workgroup prepares the activations it multiplies, so whole rows of K per
+    // workgroup cost rows x K of preparation in each (and four rows of 14336 do not fit the LDS);
+    // `ksplit` workgroups share a tile and take a slice of at least 16 blocks each.
+    uint32_t ksplit = 1;
+    // (Q6_K: two rows; with three and four the fetch-and-compute form stays ahead, 14336 -> 4096 at
+    // three rows 19.8 against 22.5 us)
+    if (S && ctx->mm8s_split_on && !glu && !ctx->call_elem && mm >= 2 && mm <= (kind == MM8_Q6K && !ctx->mm8s_all ? 2u : 4u) &&
+        groups >= 32 && tiles * 2u <= cus && tiles <= gq::MM8_SPLIT_MAX_LISTS)
+        ksplit = std::min(cus / tiles, groups / 16u);
+    while (ksplit > 1 && static_cast<size_t>(ksplit) * mm * n > gq::MM8_SPLIT_PART_FLOATS) --ksplit;
+    const bool split = ksplit > 1;
+    const uint32_t kslice = (groups + ksplit - 1u) / ksplit, lds_groups = split ? kslice : groups; // blocks a workgroup prepares
+    const uint32_t rows_per_wg = split ? 32u : static_cast<uint32_t>((n + cus - 1) / cus);
+    const uint32_t grid = static_cast<uint32_t>((n + rows_per_wg - 1) / rows_per_wg);
     const uint32_t wg_tiles = (rows_per_wg + 31u) / 32u, tile_rows = (rows_per_wg + wg_tiles - 1u) / wg_tiles;
     // One activation row over tiles of at most 16 weight rows: an item is a pair of blocks of the
     // tile, so that all 32 columns of the matrix cores carry weights (14336 -> 4096 is bound by the
     // arithmetic, not by the stream, when half of them idle).
     const bool fold = may_fold && tile_rows <= 16 && groups > 8; // (up to 8 blocks there is nothing to pair: a block per wave)
     if (may_fold && !fold && n < static_cast<size_t>(ctx->mm8s_min_rows) * cus) return -1;
-    const uint32_t ipt = fold ? gq::mm8s_fold_pairs(groups) : groups; // items per tile
+    const uint32_t ipt = fold ? gq::mm8s_fold_pairs(groups) : lds_groups; // items per tile
     const uint32_t item_bytes = (fold ? 2u : 1u) * tile_rows * pieces * 16u; // a row of an item in LDS: its 16-byte pieces side by side
-    const uint32_t fixed = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, 0, subs, glu).total;
+    const uint32_t fixed = gq::mm8s_lds_layout(lds_groups, mm, pairs, item_bytes, 0, subs, glu).total;
     const uint32_t items = (glu ? 2u : 1u) * wg_tiles * ipt; // (gated: a gate tile and an up tile per tile of rows)
     uint32_t slots = std::min(items, (160u * 1024u - std::min(fixed, 160u * 1024u)) / item_bytes);
     if (slots < items) slots -= slots % gq::MM8S_LOADERS; // a reused ring is a whole number of rounds of the loaders
@@ -625,12 +644,9 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     // (three rows 4096 -> 6144: 6.6 against 6.9 us with one), fewer when a reused ring is too short.
     uint32_t depth = pi == 0 ? 1u : std::min(gq::MM8S_MAX_DEPTH, std::max(2u, (gq::MM8S_DEPTH_BYTES + item_bytes / 2u) / item_bytes));
     if (ctx->mm8s_depth) depth = std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth);
-    while (depth > 2u && slots < items && slots < gq::mm8s_min_slots(depth)) --depth;
+    while (depth > (split ? 1u : 2u) && slots < items && slots < gq::mm8s_min_slots(depth)) --depth;
     if (slots < items && slots < gq::mm8s_min_slots(depth)) return -1;
-    const bool areg = ipt <= 16 && pi <= 1 && ctx->mm8s_areg && !(fold && ctx->call_glu);
-    // Q6_K with more than two activation rows and its operands in LDS needs more registers than
-    // a wave of a twelve-wave workgroup has: left to the fetch-and-compute form
-    if (kind == MM8_Q6K && pi > 0 && !areg) return -1;
+    const bool areg = ipt <= 16 && pi <= 1 && ctx->mm8s_areg && !(fold && ctx->call_glu) && !split;
     // Where the other kernels were timed faster (rows of 14336 and of 4096 elements over 4096 to
     // 128256 weight rows): several activation rows of long weight rows, whose preparation every
     // workgroup repeats in full (Q4_K 2 x 14336 -> 4096: 13.0 against 12.2 us); Q6_K other than
@@ -641,8 +657,8 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     // Five to eight activation rows, and three or four of Q5_K, need more registers here than a
     // wave of a twelve-wave workgroup has (6 x 2048 -> 14336 Q4_K: 16.1 against 11.0 us).
     if (!ctx->mm8s_all) {
-        if (pi == 2 || (pi == 1 && kind == MM8_Q5K)) return -1;
-        if (mm >= 2 && groups > 16) return -1;
+        if (pi == 2 || (pi == 1 && kind == MM8_Q5K && !split)) return -1;
+        if (mm >= 2 && groups > 16 && !split) return -1;
         // Tiles of fewer than 16 weight rows block by block, the matrix cores mostly idle, lose to
         // the K split of the other form for long rows (Q4_K 8192 -> 2048: 7.6 against 8.6 us) and
         // to the integer-dot GEMV for one row of Q5_K (4096 -> 2048: 4.8-5.2 against 5.6).  In
@@ -652,7 +668,7 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
         if (!fold && kind == MM8_Q5K && mm == 1 && n < static_cast<size_t>(12) * cus) return -1;
         // Q6_K: one row of 40 blocks and more, in pairs of blocks from 20 (5120 -> 4096: 6.4 against 8.1 us, 6144 -> 4096: 7.3 against
         // 8.7 us for the GEMV, 8192 -> 4096: 9.1 against 10.2; 4096 -> 4096: 6.3 against 6.0), or two short rows
-        if (kind == MM8_Q6K && !((mm == 1 && (groups >= 40 || (fold && groups >= 20))) || (mm == 2 && areg))) return -1;
+        if (kind == MM8_Q6K && !((mm == 1 && (groups >= 40 || (fold && groups >= 20))) || (mm == 2 && areg) || split)) return -1;
         // one short row over at most 4 weight rows per CU: the integer-dot GEMV stays ahead
         // (4096 -> 1024: Q4_K 4.6 against 5.0 us, Q5_K 4.9 against 5.0; 8192 -> 1024 Q4_K: 6.3 against 5.9 here)
         if (mm == 1 && rows_per_wg <= 4 && groups <= 16) return -1;
@@ -662,7 +678,10 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     if (areg) variant = pi == 1 ? 2 : (steps <= 1 ? 0 : 1);
     else variant = (pi == 0 && steps > 2) ? 6 : 3 + static_cast<int>(pi);
     hipFunction_t fn = ctx->mm8s[sfmt][variant];
-    if (fold) {
+    if (split) {
+        if (ctx->call_glu && !glu_vector_ok(ctx)) return kNeedPlainActivations;
+        fn = ctx->mm8s_split[sfmt][pi][ctx->call_glu ? 1 : 0];
+    } else if (fold) {
         // variants 0, 1 (registers), 3, 6 (LDS) of one activation row
         const int fv = variant <= 1 ? variant : variant == 3 ? 2 : 3;
         if (ctx->call_glu) {
@@ -710,12 +729,18 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     P.wg_tiles = wg_tiles;
     P.last_wg_rows = P.n - (grid - 1u) * rows_per_wg;
     P.last_wg_tiles = (P.last_wg_rows + tile_rows - 1u) / tile_rows;
-    const gq::Mm8sLds L = gq::mm8s_lds_layout(groups, mm, pairs, item_bytes, slots, subs, glu);
+    const gq::Mm8sLds L = gq::mm8s_lds_layout(lds_groups, mm, pairs, item_bytes, slots, subs, glu);
     P.lds_ctrl = L.ctrl;
     P.lds_ring = L.ring;
     P.depth = depth;
     const uint32_t lds = L.total;
-    return launch(ctx, fn, grid, (gq::MM8S_CWAVES + gq::MM8S_LOADERS) * 64, lds, stream, &P, sizeof P);
+    if (split) {
+        P.ksplit = ksplit;
+        P.kslice_groups = kslice;
+        P.part = S->mm8_part;
+        P.arrive = S->mm8_arrive;
+    }
+    return launch(ctx, fn, grid * ksplit, (gq::MM8S_CWAVES + gq::MM8S_LOADERS) * 64, lds, stream, &P, sizeof P, split);
 }
 
 // Q4_K, Q5_K and Q6_K on the int8 matrix cores, activation rows in passes of at most 8 (a pass keeps
@@ -1141,7 +1166,7 @@ int dispatch_matmul(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *
     rc = run_mmf(ctx, S, f, w, x, y, m, n, k, bf16, stream);
     if (rc >= 0 || rc == kNeedPlainActivations) return rc;
     // up to 8 rows: the int8 kernels when one pass over the weights does it, else the GEMM
-    rc = run_mm8s(ctx, f, w, x, y, m, n, k, bf16, stream);
+    rc = run_mm8s(ctx, f, w, x, y, m, n, k, bf16, stream, nullptr, false, &S);
     if (rc >= 0 || rc == kNeedPlainActivations) return rc;
     rc = run_mm8(ctx, S, f, w, x, y, m, n, k, bf16, stream, true);
     if (rc >= 0 || rc == kNeedPlainActivations) return rc;
@@ -1375,6 +1400,11 @@ int gllmq_init(gllmq_ctx **out, int device)
                 snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8sFold[v]);
                 rc = get_function(ctx, &ctx->mm8s_fold[q][v], name);
             }
+        for (int q = 0; q < 3; ++q)
+            for (int v = 0; v < 4 && rc == GLLMQ_OK; ++v) {
+                snprintf(name, sizeof name, "gq_mm8s_%s_p%d_e4%s_s", q == 2 ? "q6k" : q ? "q5k" : "q4k", 1 + (v & 1), (v & 2) ? "_g" : "");
+                rc = get_function(ctx, &ctx->mm8s_split[q][v & 1][v >> 1], name);
+            }
         static const char *const kMm8sGlu[3] = { "p1_e2_g", "p2_e4_g", "p1_e4_g" };
         for (int q = 0; q < 3; ++q)
             for (int v = 0; v < 3 && rc == GLLMQ_OK; ++v) {
@@ -1446,6 +1476,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "mm8s_depth") ctx->mm8s_depth = u;
     else if (n == "mm8s_areg") ctx->mm8s_areg = value != 0;
     else if (n == "mm8s_fold") ctx->mm8s_fold_on = value != 0;
+    else if (n == "mm8s_split") ctx->mm8s_split_on = value != 0;
     else if (n == "mm8_small_to_gemv") ctx->mm8_small_to_gemv = value != 0;
     else if (n == "mm8s_min_rows") ctx->mm8s_min_rows = std::max(1u, u);
     else if (n == "ffn_fused") ctx->ffn_fused = value != 0;

@@ -160,7 +160,8 @@ struct Mm8sCtrl {                    // counters in LDS, all start at zero
     uint32_t done[MM8S_CWAVES];      // per arithmetic wave: items consumed
     uint32_t arrived[MM8S_RED_BUFS]; // per partial-sum buffer: waves that left their sums
     uint32_t reduced;                // tiles summed and stored
-    uint32_t pad[3];
+    uint32_t finished;               // K split: arithmetic waves whose slice sums have reached coherent memory
+    uint32_t pad[2];
 };
 
 // LDS carve-up of the streamed kernels: the preparation's planes, sums and scales as in

@@ -91,7 +91,7 @@ def test_ffn_layer_shape(hip, torch, oracle):
     print("ffn 4096/14336", flush=True)
     gate, up = random_weight(Q4_K, ffn, hidden, seed=21), random_weight(Q4_K, ffn, hidden, seed=22)
     down = random_weight(Q6_K, hidden, ffn, seed=23)
-    for m in (1, 16):
+    for m in (1, 2, 4, 16):  # (two to four rows: the down projection's workgroups share slices of K)
         x = random_activations(m, hidden, seed=24 + m)
         want = oracle.ffn_swiglu(gate, up, Q4_K, down, Q6_K, x, m, hidden, ffn, acc=oracle.ACC_F64, threads=16)
         got = run_ffn(hip, torch, gate, up, Q4_K, down, Q6_K, x, m, hidden, ffn, stacked=True)
@@ -116,6 +116,8 @@ def test_ffn_three_step_form(torch, oracle):
 @pytest.mark.parametrize("t_gu,t_dn,hidden,ffn,ms", [
     (Q6_K, Q6_K, 2048, 4352, (1, 2, 4, 8)),    # GEMV gate/up; streamed down projection that reads the gated product
     (Q8_0, Q4_K, 2048, 4608, (1, 3)),          # Q8_0 gate/up, streamed Q4_K down
+    (Q6_K, Q6_K, 2048, 8192, (2, 4)),          # the down projection's workgroups share slices of K and read the gated product
+    (Q8_0, Q5_K, 1024, 8448, (3,)),
     (Q6_K, Q8_0, 1024, 1536, (1, 2, 5)),       # GEMV down projection (two rows at a time)
     (Q4_K, Q5_K, 2048, 5120, (16, 40)),        # GEMM: the preparation launch of the down projection applies the gate
     (Q6_K, Q6_K, 512, 776, (1, 9)),            # ragged ffn

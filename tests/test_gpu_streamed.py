@@ -19,7 +19,9 @@ Q4_K, Q5_K, Q6_K = 12, 13, 14
 def hip():
     # "mm8s_all": the streamed form wherever the shape fits, not only where it was timed fastest
     from gllm_amd.backend import HipBackend
-    return HipBackend(0, options={"mm8s_all": 1})
+    # ("mm8s_split" = 0: whole rows of K per workgroup also where slices of K would be shared; that
+    # form has its own test below)
+    return HipBackend(0, options={"mm8s_all": 1, "mm8s_split": 0})
 
 
 @pytest.fixture(scope="module")
@@ -113,6 +115,29 @@ def test_pairs_of_blocks_equal_single_blocks_within_the_bar(hip, torch):
         assert np.array_equal(a.view(np.uint32), again.view(np.uint32))
 
 
+@pytest.mark.parametrize("dtype", [Q4_K, Q5_K, Q6_K])
+def test_slices_of_k_shared_among_workgroups(torch, oracle, dtype):
+    """Two to four rows of long activations over few weight rows (a down projection of a small
+    batch): the workgroups of a 32-row tile take a slice of K each and the one that finishes last
+    adds the slices up.  Two to four slices, a last slice that is shorter, a ragged last tile, a
+    partial last block; twice in a row (the arrival counters are left at zero)."""
+    from gllm_amd.backend import HipBackend
+    hip = HipBackend(0, options={"mm8s_all": 1})  # (by default three and four rows of Q6_K stay on the other form)
+    c = cus(torch)
+    cases = [(2, 16 * c, 14336), (4, 16 * c, 11008 + 256 - 11008 % 256), (3, 16 * c - 9, 11008 + 256 - 11008 % 256), (4, 8 * c + 5, 8192 + 512 - 8),
+             (2, 4 * c, 14336), (3, 10 * c, 9216)]
+    for m, n, k in cases:
+        print(f"k split dtype={dtype} m={m} n={n} k={k}", flush=True)
+        w, x = random_weight(dtype, n, k, seed=n % 89 + m), random_activations(m, k, seed=k % 83 + m)
+        want = oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=16)
+        got = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+        name = hip.last_kernel_name()
+        assert name.startswith("gq_mm8s_") and name.endswith("_s"), name
+        check_close(got, want, f"k split dtype={dtype} m={m} n={n} k={k}")
+        again = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+        assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+
+
 def test_streamed_large_vocabulary_and_repeats(hip, torch, oracle):
     """A Llama-3 vocabulary of Q4_K rows (501 rows per workgroup, 16 tiles, the ring reused eight
     times), twice in a row with different inputs: the counters in LDS start from zero every launch."""
@@ -131,16 +156,19 @@ def test_default_choice_of_form(torch):
     """Without "mm8s_all" the streamed form runs where it was timed fastest: single rows of Q4_K
     and Q5_K from 4 weight rows per CU (short rows over exactly 4 excepted), Q6_K for one row of
     20 blocks and more over at most 16 weight rows per CU, of 40 and more over any number, or two
-    short ones; the results stay those of the oracle's bar either way (checked against the other
-    form here)."""
+    short ones; two to four rows of 32 blocks and more over 32-row tiles for at most half of the
+    CUs (slices of K shared among workgroups); the results stay those of the oracle's bar either
+    way (checked against the other form here)."""
     from gllm_amd.backend import HipBackend
     default, plain = HipBackend(0), HipBackend(0, options={"mm8s": 0})
     c = cus(torch)
-    for dtype, m, n, k, streamed in ((Q4_K, 1, 56 * c, 4096, True), (Q4_K, 2, 16 * c, 14336, False), (Q6_K, 1, 16 * c, 14336, True),
+    for dtype, m, n, k, streamed in ((Q4_K, 1, 56 * c, 4096, True), (Q4_K, 2, 16 * c, 14336, True), (Q6_K, 1, 16 * c, 14336, True),
                                      (Q4_K, 1, 16 * c, 8192, True), (Q4_K, 1, 12 * c, 8192, True), (Q5_K, 1, 8 * c, 8192, True),
                                      (Q4_K, 1, 4 * c, 4096, False), (Q4_K, 1, 4 * c, 8192, True), (Q5_K, 1, 8 * c, 4096, True),
                                      (Q6_K, 1, 16 * c, 4096, False), (Q6_K, 1, 16 * c, 5120, True), (Q6_K, 1, 24 * c, 5120, False),
-                                     (Q6_K, 1, 56 * c, 4096, False), (Q6_K, 2, 56 * c, 4096, True), (Q6_K, 2, 16 * c, 14336, False)):
+                                     (Q6_K, 1, 56 * c, 4096, False), (Q6_K, 2, 56 * c, 4096, True), (Q6_K, 2, 16 * c, 14336, True),
+                                     (Q4_K, 2, 40 * c, 14336, False), (Q6_K, 4, 16 * c, 14336, False), (Q5_K, 4, 16 * c, 14336, True),
+                                     (Q4_K, 5, 16 * c, 14336, False)):
         print(f"default form dtype={dtype} m={m} n={n} k={k}", flush=True)
         w, x = random_weight(dtype, n, k, seed=5), random_activations(m, k, seed=6)
         a = gpu_matmul(default, torch, w, x, dtype, m, n, k)
