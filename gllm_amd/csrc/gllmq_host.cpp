@@ -654,10 +654,13 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     // short ones (4096 -> 14336: 12.9 against 16.0), the integer-dot GEMV being ahead for one short
     // row (4096 -> 14336: 11.5 against 12.8 us) and the arithmetic of a Q6_K item costing the same
     // for a low tile as for a full one.
-    // Five to eight activation rows, and three or four of Q5_K, need more registers here than a
-    // wave of a twelve-wave workgroup has (6 x 2048 -> 14336 Q4_K: 16.1 against 11.0 us).
+    // Five to eight activation rows lead over at most 32 weight rows per CU or rows of at most 8
+    // blocks (Q4_K 6 x 4096 -> 6144: 9.9 against 10.2 us, 8 x 2048 -> 14336: 10.6 against 12.0; 6 x
+    // 4096 -> 14336: 15.0 against 14.3, 6 x 4096 -> 28672: 24.7 against 21.6), Q6_K over at most 32
+    // weight rows per CU (5 x 4096 -> 4096: 11.7 against 12.0; 5 x 2048 -> 14336: 13.6 against 12.9).
+    const bool few_rows = n <= static_cast<size_t>(32) * cus;
     if (!ctx->mm8s_all) {
-        if (pi == 2 || (pi == 1 && kind == MM8_Q5K && !split)) return -1;
+        if (pi == 2 && !(few_rows || (groups <= 8 && kind != MM8_Q6K))) return -1;
         if (mm >= 2 && groups > 16 && !split) return -1;
         // Tiles of fewer than 16 weight rows block by block, the matrix cores mostly idle, lose to
         // the K split of the other form for long rows (Q4_K 8192 -> 2048: 7.6 against 8.6 us) and
@@ -668,7 +671,11 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
         if (!fold && kind == MM8_Q5K && mm == 1 && n < static_cast<size_t>(12) * cus) return -1;
         // Q6_K: one row of 40 blocks and more, in pairs of blocks from 20 (5120 -> 4096: 6.4 against 8.1 us, 6144 -> 4096: 7.3 against
         // 8.7 us for the GEMV, 8192 -> 4096: 9.1 against 10.2; 4096 -> 4096: 6.3 against 6.0), or two short rows
-        if (kind == MM8_Q6K && !((mm == 1 && (groups >= 40 || (fold && groups >= 20))) || (mm == 2 && areg) || split)) return -1;
+        // three rows of K <= 4096 (4096 -> 14336: 14.7 against 16.6 us), four over at most 32 weight rows per
+        // CU or rows of at most 8 blocks (4096 -> 6144: 8.7 against 10.4; 4096 -> 14336: 17.4 against 16.7)
+        if (kind == MM8_Q6K && !((mm == 1 && (groups >= 40 || (fold && groups >= 20))) || ((mm == 2 || mm == 3) && areg) ||
+                                 (mm == 4 && areg && (few_rows || groups <= 8)) || pi == 2 || split))
+            return -1;
         // one short row over at most 4 weight rows per CU: the integer-dot GEMV stays ahead
         // (4096 -> 1024: Q4_K 4.6 against 5.0 us, Q5_K 4.9 against 5.0; 8192 -> 1024 Q4_K: 6.3 against 5.9 here)
         if (mm == 1 && rows_per_wg <= 4 && groups <= 16) return -1;
