@@ -47,6 +47,11 @@ def test_graph_replays_match_eager(hip, torch):
     yh = torch.empty(1, 3 * hidden, device="cuda", dtype=torch.bfloat16)  # bf16 activations and outputs
     wg6, wu6 = dev(random_weight(Q6_K, ffn, hidden, seed=8)), dev(random_weight(Q6_K, ffn, hidden, seed=9))
     h6 = torch.empty(1, hidden, device="cuda")                    # gate applied in the down projection's loads
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    wf = dev(random_weight(Q5_K, 12 * cus, 4 * hidden, seed=10))  # one row over low tiles: pairs of blocks
+    xf, yf = torch.empty(1, 4 * hidden, device="cuda"), torch.empty(1, 12 * cus, device="cuda")
+    wk = dev(random_weight(Q4_K, 8 * cus, 8 * hidden + 256, seed=11))  # three long rows over few weight rows: streamed slices of K
+    xk, yk = torch.empty(3, 8 * hidden + 256, device="cuda"), torch.empty(3, 8 * cus, device="cuda")
 
     def step():
         hip.quantized_matmul(wq, x, qkv, Q4_K, 1, 3 * hidden, hidden)
@@ -58,12 +63,18 @@ def test_graph_replays_match_eager(hip, torch):
         hip.ffn_swiglu(wg6, wu6, Q6_K, wd, Q6_K, x, h6, 1, hidden, ffn)
         hip.quantized_matmul(wb, xb, yb, Q5_K, 16, 512, hidden)
         hip.quantized_matmul(ws, xs, ys, Q4_K, 2, 256, 8 * hidden)
+        hip.quantized_matmul(wf, xf, yf, Q5_K, 1, 12 * cus, 4 * hidden)
+        assert hip.last_kernel_name().endswith("_f"), hip.last_kernel_name()
+        hip.quantized_matmul(wk, xk, yk, Q4_K, 3, 8 * cus, 8 * hidden + 256)
+        assert hip.last_kernel_name().endswith("_s"), hip.last_kernel_name()
 
     def fill(seed):
         x.copy_(torch.from_numpy(random_activations(1, hidden, seed=seed)))
         xb.copy_(torch.from_numpy(random_activations(16, hidden, seed=seed + 50)))
         xs.copy_(torch.from_numpy(random_activations(2, 8 * hidden, seed=seed + 90)))
         xh.copy_(x.to(torch.bfloat16))
+        xf.copy_(torch.from_numpy(random_activations(1, 4 * hidden, seed=seed + 120)))
+        xk.copy_(torch.from_numpy(random_activations(3, 8 * hidden + 256, seed=seed + 150)))
 
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
@@ -79,10 +90,10 @@ def test_graph_replays_match_eager(hip, torch):
         fill(seed)
         step()
         torch.cuda.synchronize()
-        outs = (qkv, h, logits, yb, ys, tok, tok2, yh, h6)
+        outs = (qkv, h, logits, yb, ys, tok, tok2, yh, h6, yf, yk)
         want = [t.clone() for t in outs]
         assert int(tok2[0]) == int(tok[0])
-        for t in (qkv, h, logits, yb, ys, yh, h6):
+        for t in (qkv, h, logits, yb, ys, yh, h6, yf, yk):
             t.fill_(float("nan"))
         tok.fill_(-7)
         tok2.fill_(-7)
