@@ -24,7 +24,9 @@ F16, BF16 = npref.ELEM_F16, npref.ELEM_BF16
 SHAPES = [(Q4_K, 1, 4096, 2048), (Q5_K, 4, 3072, 1024), (Q6_K, 2, 4096, 4096), (Q4_K, 8, 2048, 1024),
           (Q4_K, 3, 300, 512), (Q4_K, 2, 256, 8192), (Q6_K, 1, 96, 14336), (Q5_K, 1, 128, 11008),
           (Q8_0, 1, 500, 1024), (Q8_0, 2, 333, 1056), (Q6_K, 2, 1000, 768), (Q8_0, 5, 300, 2048), (Q6_K, 7, 64, 12288),
-          (Q4_K, 16, 512, 1024), (Q4_K, 32, 4096, 4096), (Q6_K, 1, 64, 16640), (Q8_0, 40, 100, 512)]
+          (Q4_K, 16, 512, 1024), (Q4_K, 32, 4096, 4096), (Q6_K, 1, 64, 16640), (Q8_0, 40, 100, 512),
+          # one row over low tiles (pairs of blocks), registers and LDS operands; slices of K fall back to conversions
+          (Q4_K, 1, 4096, 4096), (Q5_K, 1, 3000, 8192), (Q6_K, 1, 4096, 14336), (Q4_K, 1, 2048, 11008), (Q4_K, 3, 4096, 9216)]
 
 
 @pytest.fixture(scope="module")
