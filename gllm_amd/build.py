@@ -20,7 +20,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 BUILD = os.path.join(CSRC, "build")
-KERNEL_UNITS = ["codec", "mm8", "mm8s", "mm8c", "mm8_q6k_q8_0", "mmf", "mmfs", "moe"]  # csrc/kernels_<unit>.hip, one code object each
+KERNEL_UNITS = ["codec", "mm8", "mm8s", "mm8s_q8_0", "mm8c", "mm8_q6k_q8_0", "mmf", "mmfs", "moe"]  # csrc/kernels_<unit>.hip, one code object each
 LIB = os.path.join(HERE, "libgllm_hip_quant.so")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")

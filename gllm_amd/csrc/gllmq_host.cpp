@@ -36,6 +36,7 @@
 GLLMQ_EMBED(codec)
 GLLMQ_EMBED(mm8)
 GLLMQ_EMBED(mm8s)
+GLLMQ_EMBED(mm8s_q8_0)
 GLLMQ_EMBED(mm8c)
 GLLMQ_EMBED(mm8_q6k_q8_0)
 GLLMQ_EMBED(mmf)
@@ -166,7 +167,7 @@ struct CachedWeights {
 
 struct gllmq_ctx {
     int device = 0;
-    hipModule_t modules[8] = {}; // one per embedded code object
+    hipModule_t modules[9] = {}; // one per embedded code object
     hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
     hipFunction_t gather[kNumFormats][2] = {};  // quantized embedding lookup [format][0 = scalar stores, 1 = float4 stores]
     // gated form of the int8 kernels (gate and up rows in one launch, act(gate) * up out):
@@ -179,14 +180,19 @@ struct gllmq_ctx {
     hipFunction_t dequant_wave_q5k = nullptr;   // the same for Q5_K
     hipFunction_t gemv[kNumFormats][2] = {};    // [format][m - 1], f32 multiply-add flavour
     hipFunction_t gemv_i8[kNumFormats][2] = {}; // [format][m - 1], integer-dot flavour (default)
+    // call_mutex held: launches are only counted and the last kernel noted, nothing is enqueued
+    // (gllmq_lm_head_argmax asks which kernel the one-row matmul of its shape would get)
+    bool probe = false;
+    uint32_t probe_launches = 0;
+    hipFunction_t probe_fn = nullptr;
     hipFunction_t gemv_i8_argmax[kNumFormats] = {}; // one row, ending in the candidates of the greedy token choice
     // int8 matrix-core kernels [Mm8Kind][pairs 1,2,4][early steps 1,2,4], and the same with
     // register-resident activation operands [Mm8Kind][pairs 1,2][early][passes per tile - 1]
     hipFunction_t mm8[MM8_KINDS][3][3] = {};
     hipFunction_t mm8_areg[MM8_KINDS][2][3][2] = {};
-    // streamed form (loader waves + arithmetic waves) [0 = Q4_K, 1 = Q5_K, 2 = Q6_K][variant]: register
+    // streamed form (loader waves + arithmetic waves) [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][variant]: register
     // operands p1_e1, p1_e2, p2_e4, then LDS operands p1_e2, p2_e4, p4_e4
-    hipFunction_t mm8s[3][7] = {};
+    hipFunction_t mm8s[4][7] = {};
     bool use_mm8s = true;                       // "mm8s" = 0: the fetch-and-compute kernels throughout
     bool batch_overlap = true;                  // "batch_overlap" = 0: the kernels of a batch run strictly one after the other
     bool mm8s_all = false;                      // "mm8s_all" = 1: the streamed form wherever it fits, also where another was timed faster
@@ -260,15 +266,16 @@ struct gllmq_ctx {
     bool ffn_glu_load = true;   // "ffn_glu_load" = 0: the gate activation always runs as a kernel of its own
     hipFunction_t mm8s_gated[2][6] = {};        // streamed gate/up kernels with act(g) * u at the end of a tile pair [Q4_K, Q5_K][p1_e1_a, p1_e2_a, p2_e4_a, p1_e2, p2_e4, p1_e4]
     bool ffn_streamed = true;                   // "ffn_streamed" = 0: gllmq_ffn_swiglu never uses them
-    hipFunction_t mm8s_e16[3][6] = {};          // streamed kernels over 16-bit activations and outputs [format][p1_e1_a, p1_e2_a, p2_e4_a, p1_e2, p2_e4, p1_e4]
-    hipFunction_t mm8s_glu[3][3] = {};          // streamed kernels that take gated activations [format][p1_e2, p2_e4, p1_e4]
+    hipFunction_t mm8s_e16[4][6] = {};          // streamed kernels over 16-bit activations and outputs [format][p1_e1_a, p1_e2_a, p2_e4_a, p1_e2, p2_e4, p1_e4]
+    hipFunction_t mm8s_glu[4][3] = {};          // streamed kernels that take gated activations [format][p1_e2, p2_e4, p1_e4]
     // streamed kernels whose items are pairs of blocks of a tile of at most 16 weight rows (one
     // activation row) [format][p1_e1_a, p1_e2_a, p1_e2, p1_e4, p1_e2 and p1_e4 over gated activations,
     // the first four over a 16-bit element type]
-    hipFunction_t mm8s_fold[3][10] = {};
+    hipFunction_t mm8s_fold[4][10] = {};
     // streamed kernels whose workgroups share a row range and take a slice of K each (two to four
     // activation rows over few weight rows) [format][p1_e4, p2_e4][plain, gated activations]
-    hipFunction_t mm8s_split[3][2][2] = {};
+    hipFunction_t mm8s_split[4][2][2] = {};
+    bool mm8s_q8_0 = true;                      // "mm8s_q8_0" = 0: Q8_0 never takes the streamed form
     bool mm8s_split_on = true;                  // "mm8s_split" = 0: such shapes stay on the fetch-and-compute form
     bool mm8s_fold_on = true;                   // "mm8s_fold" = 0: such tiles go block by block, half of the matrix-core columns idle
     hipFunction_t gemv_i8_glu[kNumFormats][2] = {};
@@ -433,6 +440,11 @@ int grow_scratch(gllmq_ctx *ctx, const Scratch &S, void **buf, size_t *have, siz
 int launch2d(gllmq_ctx *ctx, hipFunction_t f, uint32_t grid_x, uint32_t grid_y, uint32_t block, uint32_t lds,
              void *stream, void *params, size_t params_size, bool uses_scratch = false)
 {
+    if (ctx->probe) {
+        ++ctx->probe_launches;
+        ctx->probe_fn = f;
+        return GLLMQ_OK;
+    }
     void *config[] = { HIP_LAUNCH_PARAM_BUFFER_POINTER, params, HIP_LAUNCH_PARAM_BUFFER_SIZE,
                        &params_size, HIP_LAUNCH_PARAM_END };
     gllmq_ctx::Overlap &ov = ctx->overlap;
@@ -587,12 +599,14 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     const int kind = mm8_kind(f.dtype);
     const bool glu = w2 != nullptr;
     if (glu && ((kind != MM8_Q4K && kind != MM8_Q5K) || m > 4 || ctx->call_glu || ctx->call_elem)) return -1;
-    if (!ctx->use_mm8 || !ctx->use_mm8s || (kind != MM8_Q4K && kind != MM8_Q5K && kind != MM8_Q6K) || m == 0 || m > 8) return -1;
+    if (!ctx->use_mm8 || !ctx->use_mm8s || (kind != MM8_Q4K && kind != MM8_Q5K && kind != MM8_Q6K && kind != MM8_Q8_0) || m == 0 || m > 8) return -1;
     if (kind == MM8_Q5K && ctx->mm8_q5k_min_m == 0) return -1;
     if (kind == MM8_Q6K && ctx->mm8_q6k_min_m == 0) return -1;
-    const int sfmt = kind == MM8_Q6K ? 2 : kind == MM8_Q5K ? 1 : 0;
-    const uint32_t pieces = sfmt == 2 ? gq::Mm8sFormat<2>::PIECES : sfmt == 1 ? gq::Mm8sFormat<1>::PIECES : gq::Mm8sFormat<0>::PIECES;
-    const uint32_t subs = sfmt == 2 ? 16u : 8u;
+    // Q8_0: an item is a group of 8 blocks, so rows of whole groups only
+    if (kind == MM8_Q8_0 && (ctx->mm8_q8_0_min_m == 0 || !ctx->mm8s_q8_0 || k % 256 != 0)) return -1;
+    const int sfmt = kind == MM8_Q8_0 ? 3 : kind == MM8_Q6K ? 2 : kind == MM8_Q5K ? 1 : 0;
+    const uint32_t pieces = sfmt == 3 ? gq::Mm8sFormat<3>::PIECES : sfmt == 2 ? gq::Mm8sFormat<2>::PIECES : sfmt == 1 ? gq::Mm8sFormat<1>::PIECES : gq::Mm8sFormat<0>::PIECES;
+    const uint32_t subs = sfmt == 3 ? 0u : sfmt == 2 ? 16u : 8u;
     if (!aligned(x, 16) || k % 8 != 0) return -1;
     const uint32_t cus = static_cast<uint32_t>(ctx->num_cus);
     const uint32_t groups = static_cast<uint32_t>((k + 255) / 256), tiles = static_cast<uint32_t>((n + 31) / 32);
@@ -619,6 +633,9 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
         groups >= 32 && tiles * 2u <= cus && tiles <= gq::MM8_SPLIT_MAX_LISTS)
         ksplit = std::min(cus / tiles, groups / 16u);
     while (ksplit > 1 && static_cast<size_t>(ksplit) * mm * n > gq::MM8_SPLIT_PART_FLOATS) --ksplit;
+    // (slices for fewer than three quarters of the CUs leave too many of them idle: Q8_0 8192 -> 1024
+    // at two rows 10.9 against 9.6 us for the GEMV)
+    if (ksplit > 1 && !ctx->mm8s_all && ksplit * tiles * 4u < cus * 3u) ksplit = 1;
     const bool split = ksplit > 1;
     const uint32_t kslice = (groups + ksplit - 1u) / ksplit, lds_groups = split ? kslice : groups; // blocks a workgroup prepares
     const uint32_t rows_per_wg = split ? 32u : static_cast<uint32_t>((n + cus - 1) / cus);
@@ -676,6 +693,8 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
         if (kind == MM8_Q6K && !((mm == 1 && (groups >= 40 || (fold && groups >= 20))) || ((mm == 2 || mm == 3) && areg) ||
                                  (mm == 4 && areg && (few_rows || groups <= 8)) || pi == 2 || split))
             return -1;
+        // Q8_0, two rows over at most 8 weight rows per CU: its GEMV stays ahead (4096 -> 1024: 5.9 against 7.1 us)
+        if (kind == MM8_Q8_0 && mm == 2 && n <= static_cast<size_t>(8) * cus) return -1;
         // one short row over at most 4 weight rows per CU: the integer-dot GEMV stays ahead
         // (4096 -> 1024: Q4_K 4.6 against 5.0 us, Q5_K 4.9 against 5.0; 8192 -> 1024 Q4_K: 6.3 against 5.9 here)
         if (mm == 1 && rows_per_wg <= 4 && groups <= 16) return -1;
@@ -1264,9 +1283,9 @@ int gllmq_init(gllmq_ctx **out, int device)
             return GLLMQ_ERR_UNIMPLEMENTED;
         }
     }
-    const unsigned char *const images[8] = { gllmq_co_codec, gllmq_co_mm8, gllmq_co_mm8s, gllmq_co_mm8c, gllmq_co_mm8_q6k_q8_0,
-                                             gllmq_co_mmf, gllmq_co_mmfs, gllmq_co_moe };
-    for (int i = 0; i < 8; ++i) {
+    const unsigned char *const images[9] = { gllmq_co_codec, gllmq_co_mm8, gllmq_co_mm8s, gllmq_co_mm8s_q8_0, gllmq_co_mm8c,
+                                             gllmq_co_mm8_q6k_q8_0, gllmq_co_mmf, gllmq_co_mmfs, gllmq_co_moe };
+    for (int i = 0; i < 9; ++i) {
         e = hipModuleLoadData(&ctx->modules[i], images[i]);
         if (e != hipSuccess) {
             fprintf(stderr, "gllmq_init: hipModuleLoadData: %s\n", hipGetErrorString(e));
@@ -1382,10 +1401,11 @@ int gllmq_init(gllmq_ctx **out, int device)
                 }
             }
         if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->glu_act, "gq_glu_act");
+        static const char *const kMm8sFormat[4] = { "q4k", "q5k", "q6k", "q8_0" };
         static const char *const kMm8s[7] = { "p1_e1_a", "p1_e2_a", "p2_e4_a", "p1_e2", "p2_e4", "p4_e4", "p1_e4" };
-        for (int q = 0; q < 3; ++q)
+        for (int q = 0; q < 4; ++q)
             for (int v = 0; v < 7 && rc == GLLMQ_OK; ++v) {
-                snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8s[v]);
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s", kMm8sFormat[q], kMm8s[v]);
                 rc = get_function(ctx, &ctx->mm8s[q][v], name);
             }
         static const char *const kMm8sGated[6] = { "p1_e1_a", "p1_e2_a", "p2_e4_a", "p1_e2", "p2_e4", "p1_e4" };
@@ -1395,27 +1415,27 @@ int gllmq_init(gllmq_ctx **out, int device)
                 rc = get_function(ctx, &ctx->mm8s_gated[q][v], name);
             }
         static const char *const kMm8sE16[6] = { "p1_e1_a", "p1_e2_a", "p2_e4_a", "p1_e2", "p2_e4", "p1_e4" };
-        for (int q = 0; q < 3; ++q)
+        for (int q = 0; q < 4; ++q)
             for (int v = 0; v < 6 && rc == GLLMQ_OK; ++v) {
-                snprintf(name, sizeof name, "gq_mm8s_%s_%s_e16", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8sE16[v]);
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s_e16", kMm8sFormat[q], kMm8sE16[v]);
                 rc = get_function(ctx, &ctx->mm8s_e16[q][v], name);
             }
         static const char *const kMm8sFold[10] = { "p1_e1_a_f", "p1_e2_a_f", "p1_e2_f", "p1_e4_f", "p1_e2_g_f", "p1_e4_g_f",
                                                    "p1_e1_a_f_e16", "p1_e2_a_f_e16", "p1_e2_f_e16", "p1_e4_f_e16" };
-        for (int q = 0; q < 3; ++q)
+        for (int q = 0; q < 4; ++q)
             for (int v = 0; v < 10 && rc == GLLMQ_OK; ++v) {
-                snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8sFold[v]);
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s", kMm8sFormat[q], kMm8sFold[v]);
                 rc = get_function(ctx, &ctx->mm8s_fold[q][v], name);
             }
-        for (int q = 0; q < 3; ++q)
+        for (int q = 0; q < 4; ++q)
             for (int v = 0; v < 4 && rc == GLLMQ_OK; ++v) {
-                snprintf(name, sizeof name, "gq_mm8s_%s_p%d_e4%s_s", q == 2 ? "q6k" : q ? "q5k" : "q4k", 1 + (v & 1), (v & 2) ? "_g" : "");
+                snprintf(name, sizeof name, "gq_mm8s_%s_p%d_e4%s_s", kMm8sFormat[q], 1 + (v & 1), (v & 2) ? "_g" : "");
                 rc = get_function(ctx, &ctx->mm8s_split[q][v & 1][v >> 1], name);
             }
         static const char *const kMm8sGlu[3] = { "p1_e2_g", "p2_e4_g", "p1_e4_g" };
-        for (int q = 0; q < 3; ++q)
+        for (int q = 0; q < 4; ++q)
             for (int v = 0; v < 3 && rc == GLLMQ_OK; ++v) {
-                snprintf(name, sizeof name, "gq_mm8s_%s_%s", q == 2 ? "q6k" : q ? "q5k" : "q4k", kMm8sGlu[v]);
+                snprintf(name, sizeof name, "gq_mm8s_%s_%s", kMm8sFormat[q], kMm8sGlu[v]);
                 rc = get_function(ctx, &ctx->mm8s_glu[q][v], name);
             }
     }
@@ -1484,6 +1504,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "mm8s_areg") ctx->mm8s_areg = value != 0;
     else if (n == "mm8s_fold") ctx->mm8s_fold_on = value != 0;
     else if (n == "mm8s_split") ctx->mm8s_split_on = value != 0;
+    else if (n == "mm8s_q8_0") ctx->mm8s_q8_0 = value != 0;
     else if (n == "mm8_small_to_gemv") ctx->mm8_small_to_gemv = value != 0;
     else if (n == "mm8s_min_rows") ctx->mm8s_min_rows = std::max(1u, u);
     else if (n == "ffn_fused") ctx->ffn_fused = value != 0;
@@ -1616,12 +1637,23 @@ int gllmq_lm_head_argmax(gllmq_ctx *ctx, const void *w, size_t w_bytes, const fl
     Scratch *S = nullptr;
     rc = acquire_scratch(ctx, stream, &S);
     if (rc != GLLMQ_OK) return rc;
-    // The matvec whose workgroups leave their best candidate behind, where the one-row GEMV is the
-    // kernel such a matrix gets anyway (Q6_K and Q8_0, the types of GGUF output matrices) and one
-    // launch covers K; the workgroup that finishes last picks among the candidates.
+    // The matvec whose workgroups leave their best candidate behind: the one-row GEMV of Q6_K and
+    // Q8_0 (the types of GGUF output matrices) where one launch covers K; the workgroup that
+    // finishes last picks among the candidates.  With a logits buffer it runs where the GEMV is
+    // the kernel gllmq_quantized_matmul gives the shape anyway (asked by a dry run of the
+    // dispatch), so that the logits are that call's bit for bit; without one, always.
     const size_t rb = gllmq_row_bytes(dtype, k);
     const bool gemv_type = dtype == 14u || dtype == 8u;
-    if (ctx->lm_head_fused && gemv_type && !ctx->gemv_f32 && k <= 16384) {
+    bool gemv_anyway = true;
+    if (ctx->lm_head_fused && gemv_type && !ctx->gemv_f32 && k <= 16384 && logits) {
+        ctx->probe = true;
+        ctx->probe_launches = 0;
+        ctx->probe_fn = nullptr;
+        const int prc = dispatch_matmul(ctx, *S, *f, static_cast<const uint8_t *>(w), x, logits, 1, n, k, false, stream);
+        ctx->probe = false;
+        gemv_anyway = prc == GLLMQ_OK && ctx->probe_launches == 1 && ctx->probe_fn == ctx->gemv_i8[format_index(dtype)][0];
+    }
+    if (ctx->lm_head_fused && gemv_type && !ctx->gemv_f32 && k <= 16384 && gemv_anyway) {
         GemvPlan L = plan_gemv(ctx, 1, static_cast<uint32_t>(n), static_cast<uint32_t>(k), rb, ctx->gemv_waves);
         if (L.grid <= gq::ARGMAX_MAX_PARTS * gq::ARGMAX_MAX_ROWS) {
             GemvParams &P = L.P;

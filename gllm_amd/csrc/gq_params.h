@@ -107,6 +107,7 @@ template <int FMT> struct Mm8sFormat;
 template <> struct Mm8sFormat<0> { static constexpr uint32_t BLOCK = 144, PIECES = 9, SUBS = 8; };   // Q4_K
 template <> struct Mm8sFormat<1> { static constexpr uint32_t BLOCK = 176, PIECES = 11, SUBS = 8; };  // Q5_K
 template <> struct Mm8sFormat<2> { static constexpr uint32_t BLOCK = 210, PIECES = 14, SUBS = 16; }; // Q6_K
+template <> struct Mm8sFormat<3> { static constexpr uint32_t BLOCK = 272, PIECES = 17, SUBS = 0; };   // Q8_0: a group of 8 blocks of 34 bytes (K a multiple of 256)
 GQ_HD constexpr uint32_t mm8s_piece_offset(int fmt, uint32_t piece) { return (fmt == 2 && piece == 13u) ? 194u : 16u * piece; }
 
 // LDS carve-up (bytes) of the int8 matrix-core kernels.

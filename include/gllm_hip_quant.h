@@ -196,8 +196,12 @@ int gllmq_reserve_matmul_elem(gllmq_ctx *ctx, uint32_t ggml_dtype, size_t m, siz
  * NULL when only the token is wanted and the matrix is Q6_K or Q8_0 with k <= 16384: there
  * every workgroup of the matvec leaves its best candidate behind and the one that finishes last
  * picks among them (one launch), so the logits are neither written nor read again.  Other matrices run
- * gllmq_quantized_matmul and gllmq_argmax one after the other and need logits_dev.  The
- * logits and the token are those of the two calls made separately, bit for bit. */
+ * gllmq_quantized_matmul and gllmq_argmax one after the other and need logits_dev, and so do
+ * shapes with a logits buffer for which gllmq_quantized_matmul has a faster kernel than that
+ * matvec (Q8_0 rows of whole 256-element groups, a few long Q6_K rows).  With logits_dev the
+ * logits and the token are those of the two calls made separately, bit for bit; without it the
+ * token is the choice among that matvec's own logits, which agree with the other kernels' to the
+ * matmul's tolerance. */
 int gllmq_lm_head_argmax(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev, uint32_t ggml_dtype,
                          size_t n, size_t k, float *logits_dev, uint32_t *token_dev, float *value_dev, void *stream);
 

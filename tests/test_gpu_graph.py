@@ -50,8 +50,8 @@ def test_graph_replays_match_eager(hip, torch):
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     wf = dev(random_weight(Q5_K, 12 * cus, 4 * hidden, seed=10))  # one row over low tiles: pairs of blocks
     xf, yf = torch.empty(1, 4 * hidden, device="cuda"), torch.empty(1, 12 * cus, device="cuda")
-    wk = dev(random_weight(Q4_K, 8 * cus, 8 * hidden + 256, seed=11))  # three long rows over few weight rows: streamed slices of K
-    xk, yk = torch.empty(3, 8 * hidden + 256, device="cuda"), torch.empty(3, 8 * cus, device="cuda")
+    wk = dev(random_weight(Q4_K, 16 * cus, 8 * hidden + 256, seed=11))  # three long rows over few weight rows: streamed slices of K
+    xk, yk = torch.empty(3, 8 * hidden + 256, device="cuda"), torch.empty(3, 16 * cus, device="cuda")
 
     def step():
         hip.quantized_matmul(wq, x, qkv, Q4_K, 1, 3 * hidden, hidden)
@@ -65,7 +65,7 @@ def test_graph_replays_match_eager(hip, torch):
         hip.quantized_matmul(ws, xs, ys, Q4_K, 2, 256, 8 * hidden)
         hip.quantized_matmul(wf, xf, yf, Q5_K, 1, 12 * cus, 4 * hidden)
         assert hip.last_kernel_name().endswith("_f"), hip.last_kernel_name()
-        hip.quantized_matmul(wk, xk, yk, Q4_K, 3, 8 * cus, 8 * hidden + 256)
+        hip.quantized_matmul(wk, xk, yk, Q4_K, 3, 16 * cus, 8 * hidden + 256)
         assert hip.last_kernel_name().endswith("_s"), hip.last_kernel_name()
 
     def fill(seed):

@@ -138,6 +138,31 @@ def test_slices_of_k_shared_among_workgroups(torch, oracle, dtype):
         assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
 
 
+def test_q8_0_in_groups_of_eight_blocks(torch, oracle):
+    """Q8_0 rows of whole 256-element groups take the streamed form too (an item is a group of 8
+    blocks of a tile, 272 bytes per row): one to eight rows, registers and LDS operands, pairs of
+    groups over low tiles, slices of K; rows with a partial group stay on the other kernels."""
+    from gllm_amd.backend import HipBackend
+    Q8_0 = 8
+    hip = HipBackend(0, options={"mm8s_all": 1})
+    c = cus(torch)
+    cases = [(1, 56 * c, 4096, ""), (1, 16 * c, 14336, "_f"), (2, 33 * c + 5, 2048, ""), (1, 9 * c + 3, 2304, "_f"),
+             (3, 40 * c, 1024, ""), (4, 16 * c - 7, 8192 + 256, "_s"), (1, 64 * c + 3, 256, ""), (8, 32 * c, 1024, ""),
+             (1, 12 * c, 4096, "_f"), (2, 56 * c, 4096, ""), (5, 32 * c + 5, 1536, ""), (1, 32 * c, 4096 + 32, None),
+             (2, 40 * c, 1000, None)]
+    for m, n, k, suffix in cases:
+        print(f"streamed Q8_0 m={m} n={n} k={k}", flush=True)
+        w, x = random_weight(Q8_0, n, k, seed=m + n), random_activations(m, k, seed=k + m)
+        want = oracle.quantized_matmul(w, x, Q8_0, m, n, k, acc=oracle.ACC_F64, threads=16)
+        got = gpu_matmul(hip, torch, w, x, Q8_0, m, n, k)
+        name = hip.last_kernel_name()
+        if suffix is None:
+            assert not name.startswith("gq_mm8s_"), name
+        else:
+            assert name.startswith("gq_mm8s_q8_0_") and (name.endswith(suffix) if suffix else name[-2:] not in ("_f", "_s")), name
+        check_close(got, want, f"streamed Q8_0 m={m} n={n} k={k}")
+
+
 def test_streamed_large_vocabulary_and_repeats(hip, torch, oracle):
     """A Llama-3 vocabulary of Q4_K rows (501 rows per workgroup, 16 tiles, the ring reused eight
     times), twice in a row with different inputs: the counters in LDS start from zero every launch."""
