@@ -197,13 +197,14 @@ def run_other(args):
         return region
 
     if name in ("gemv_q4k_4096", "gemv_q6k", "gemm_m16", "gemm_m32", "gemm_m64", "layer_mix", "layer_mix_m4", "layer_mix_m32",
-                "lm_head_q6k", "down_q6k", "down_q4k", "down_q6k_m2", "down_q4k_m4"):
+                "lm_head_q6k", "down_q6k", "down_q4k", "down_q6k_m2", "down_q4k_m4", "gemv_q8_0", "gemv_q5k"):
         if name.startswith("layer_mix"):
             mm = int(name.split("_m")[2]) if name.count("_m") == 2 else 1  # decode, or batched decode of 4 / 32 sequences
             ops = [(12, 6144, 4096, mm), (12, 4096, 4096, mm), (12, 2 * 14336, 4096, mm), (14, 4096, 14336, mm)]
             copies = 3
         else:
             dtype, n, k, m = {"gemv_q4k_4096": (12, 4096, 4096, 1), "gemv_q6k": (14, 14336, 4096, 1),
+                              "gemv_q8_0": (8, 14336, 4096, 1), "gemv_q5k": (13, 14336, 4096, 1),
                               "gemm_m16": (12, 14336, 4096, 16), "gemm_m32": (12, 14336, 4096, 32),
                               "gemm_m64": (12, 14336, 4096, 64),
                               # the down projection of the layer: few weight rows (16 per CU), long rows
@@ -456,7 +457,7 @@ def main():
     ap.add_argument("--no-context", action="store_true",
                     help="skip the cache-resident and copy-rate context runs (profiling: only the timed kernel launches)")
     ap.add_argument("--workload", default="gemv_q4k",
-                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q6k, layer_mix, layer_mix_m4, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, down_q6k, down_q4k, down_q6k_m2, down_q4k_m4, lm_head_q6k, lm_head_argmax_q6k, lm_head_then_argmax_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
+                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q5k, gemv_q6k, gemv_q8_0, layer_mix, layer_mix_m4, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, down_q6k, down_q4k, down_q6k_m2, down_q4k_m4, lm_head_q6k, lm_head_argmax_q6k, lm_head_then_argmax_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
                          "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="kernel-family option of the library for this run (repeatable), e.g. mm8s=0")
