@@ -203,7 +203,7 @@ struct gllmq_ctx {
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmfs[2][2] = {};              // its streamed form [0 = Q4_K, 1 = Q5_K][bf16 mode]
-    hipFunction_t mm8c[2] = {};                 // chains of streamed matmuls in one launch [0 = Q4_K, 1 = Q5_K]
+    hipFunction_t mm8c[3] = {};                 // chains of streamed matmuls in one launch [0 = Q4_K, 1 = Q5_K, 2 = Q8_0]
     bool chain_dependent = false;               // "chain_dependent" = 1: entries that depend on the one before stay in the chain
     bool use_chain = true;                      // "chain" = 0: every entry of a batch is a launch of its own
     uint32_t chain_min_rows = 1;                // "chain_min_rows": fewest weight rows in a CU's share of an entry that joins a chain
@@ -1078,8 +1078,9 @@ int run_mmfs(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, cons
 bool chain_entry_ok(const gllmq_ctx *ctx, const gllmq_matmul_desc &d, const gllmq_matmul_desc &first)
 {
     const Format *f = find_format(d.ggml_dtype);
-    if (!f || (f->dtype != T_Q4_K && f->dtype != T_Q5_K)) return false;
+    if (!f || (f->dtype != T_Q4_K && f->dtype != T_Q5_K && f->dtype != T_Q8_0)) return false;
     if (f->dtype == T_Q5_K && ctx->mm8_q5k_min_m == 0) return false;
+    if (f->dtype == T_Q8_0 && (ctx->mm8_q8_0_min_m == 0 || !ctx->mm8s_q8_0 || d.k % 256 != 0)) return false; // whole groups of 8 blocks
     if (d.ggml_dtype != first.ggml_dtype || d.m != first.m || d.k != first.k) return false;
     if (d.m == 0 || d.m > 2 || d.k == 0 || d.k % 8 != 0 || (d.k + 255) / 256 > 16 || d.n > 0x7FFFFFFFu) return false;
     if (!d.w_dev || !d.x_dev || !d.y_dev || !aligned(d.x_dev, 16) || !aligned(d.y_dev, 4) || !aligned(d.w_dev, f->w_align)) return false;
@@ -1105,7 +1106,7 @@ size_t chain_length(const gllmq_ctx *ctx, const gllmq_matmul_desc *descs, size_t
 int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t len, void *stream)
 {
     const Format &f = *find_format(descs[0].ggml_dtype);
-    const int fmt = f.dtype == T_Q5_K ? 1 : 0;
+    const int fmt = f.dtype == T_Q8_0 ? 2 : f.dtype == T_Q5_K ? 1 : 0;
     const uint32_t cus = static_cast<uint32_t>(ctx->num_cus);
     const size_t k = descs[0].k;
     Mm8ChainParams P{};
@@ -1116,10 +1117,10 @@ int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t
     P.m = static_cast<uint32_t>(descs[0].m);
     P.ldx = P.k;
     P.act_bf16 = 0;
-    const uint32_t pieces = fmt == 1 ? gq::Mm8sFormat<1>::PIECES : gq::Mm8sFormat<0>::PIECES;
+    const uint32_t pieces = fmt == 2 ? gq::Mm8sFormat<3>::PIECES : fmt == 1 ? gq::Mm8sFormat<1>::PIECES : gq::Mm8sFormat<0>::PIECES;
     P.slot_bytes = 32u * pieces * 16u; // a slot holds an item of any entry: 32 rows of one block
     // LDS: the preparation's planes, sums and scales; the counters; the partial sums; the ring
-    const gq::Mm8Lds prep = gq::mm8_lds_layout(P.groups, P.m, 1u, 8u, 0u);
+    const gq::Mm8Lds prep = gq::mm8_lds_layout(P.groups, P.m, 1u, fmt == 2 ? 0u : 8u, 0u);
     P.lds_ctrl = (prep.red + 15u) & ~15u;
     const uint32_t red = P.lds_ctrl + static_cast<uint32_t>(sizeof(gq::Mm8sCtrl)) + gq::MM8C_MAX_SLOTS * 4u;
     P.lds_ring = (red + gq::MM8C_RED_BUFS * gq::MM8C_CWAVES * 64u * 4u + 1023u) & ~1023u;
@@ -1340,6 +1341,7 @@ int gllmq_init(gllmq_ctx **out, int device)
             }
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8c[0], "gq_mm8c_q4k");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8c[1], "gq_mm8c_q5k");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8c[2], "gq_mm8c_q8_0");
     for (int q = 0; q < 2 && rc == GLLMQ_OK; ++q)
         for (int b = 0; b < 2 && rc == GLLMQ_OK; ++b) {
             snprintf(name, sizeof name, "gq_mmfs_%s%s", q ? "q5k" : "q4k", b ? "_bf16" : "");

@@ -11,6 +11,8 @@
 #define GQ_TEMPLATES_ONLY
 #include "mm8.hip.inc"
 #include "mm8_q6k.hip.inc"
+#include "mm8_q8_0.hip.inc"
+#define GQ_MM8S_Q8_0 // the Q8_0 item of mm8s.hip.inc
 #include "mm8s.hip.inc"
 #undef GQ_TEMPLATES_ONLY
 

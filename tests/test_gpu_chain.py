@@ -14,7 +14,7 @@ from tests.test_gpu_parity import check_close
 
 pytestmark = pytest.mark.gpu
 
-Q4_K, Q5_K = 12, 13
+Q4_K, Q5_K, Q8_0 = 12, 13, 8
 
 
 @pytest.fixture(scope="module")
@@ -38,7 +38,7 @@ def run_batch(hip, torch, entries, after_previous):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("dtype,m", [(Q4_K, 1), (Q5_K, 1), (Q4_K, 2), (Q5_K, 2)])
+@pytest.mark.parametrize("dtype,m", [(Q4_K, 1), (Q5_K, 1), (Q4_K, 2), (Q5_K, 2), (Q8_0, 1), (Q8_0, 2)])
 def test_independent_entries_of_different_heights(torch, oracle, dtype, m):
     """The matmuls of a decoder layer that share K: different numbers of weight rows, so different
     tile heights and numbers of workgroups per entry, one launch."""
@@ -62,7 +62,7 @@ def test_independent_entries_of_different_heights(torch, oracle, dtype, m):
         assert np.array_equal(outs[0][i].view(np.uint32), outs[1][i].view(np.uint32)), f"entry {i}: chained and single launches differ"
 
 
-@pytest.mark.parametrize("dtype,m", [(Q4_K, 1), (Q5_K, 2)])
+@pytest.mark.parametrize("dtype,m", [(Q4_K, 1), (Q5_K, 2), (Q8_0, 1)])
 def test_entries_with_few_weight_rows_join_the_chain(torch, oracle, dtype, m):
     """Separate Q, K and V projections of a grouped-query layer (K and V have a quarter of the rows)
     and smaller ones still, down to fewer rows than CUs: tiles of a few rows, workgroups without a
@@ -86,7 +86,7 @@ def test_entries_with_few_weight_rows_join_the_chain(torch, oracle, dtype, m):
         check_close(got[:m * n].reshape(m, n), oracle.quantized_matmul(w, x, dtype, m, n, k, acc=oracle.ACC_F64, threads=8), f"entry {i}")
 
 
-@pytest.mark.parametrize("dtype,m", [(Q4_K, 1), (Q5_K, 1), (Q4_K, 2)])
+@pytest.mark.parametrize("dtype,m", [(Q4_K, 1), (Q5_K, 1), (Q4_K, 2), (Q8_0, 1)])
 def test_entries_that_share_their_activations(torch, oracle, dtype, m):
     """Q, K and V read the same x, gate and up another, a last entry the first again: a workgroup
     prepares an x once for the entries in a row that share it (also one that skipped an entry it
