@@ -203,7 +203,7 @@ struct gllmq_ctx {
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmfs[2][2] = {};              // its streamed form [0 = Q4_K, 1 = Q5_K][bf16 mode]
-    hipFunction_t mm8c[3] = {};                 // chains of streamed matmuls in one launch [0 = Q4_K, 1 = Q5_K, 2 = Q8_0]
+    hipFunction_t mm8c[3][2] = {};              // chains of streamed matmuls in one launch [0 = Q4_K, 1 = Q5_K, 2 = Q8_0][some entry in pairs of blocks]
     bool chain_dependent = false;               // "chain_dependent" = 1: entries that depend on the one before stay in the chain
     bool use_chain = true;                      // "chain" = 0: every entry of a batch is a launch of its own
     uint32_t chain_min_rows = 1;                // "chain_min_rows": fewest weight rows in a CU's share of an entry that joins a chain
@@ -1154,11 +1154,14 @@ int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t
         if (ctx->mm8s_fold_on && P.m == 1 && E.tile_rows <= 16 && P.groups > 8) E.flags |= 4u;
         launched = std::max(launched, E.grid);
     }
-    bool waits = false;
-    for (size_t i = 0; i < len; ++i) waits = waits || (P.e[i].flags & 3u) != 0u;
+    bool waits = false, folds = false;
+    for (size_t i = 0; i < len; ++i) {
+        waits = waits || (P.e[i].flags & 3u) != 0u;
+        folds = folds || (P.e[i].flags & 4u) != 0u;
+    }
     if (!waits) P.done = nullptr; // independent entries count nothing: no counters to set back at the end
     P.launched = launched;
-    return launch(ctx, ctx->mm8c[fmt], launched, (gq::MM8C_CWAVES + gq::MM8C_LOADERS) * 64, P.lds_ring + slots * P.slot_bytes,
+    return launch(ctx, ctx->mm8c[fmt][folds ? 1 : 0], launched, (gq::MM8C_CWAVES + gq::MM8C_LOADERS) * 64, P.lds_ring + slots * P.slot_bytes,
                   stream, &P, sizeof P, true);
 }
 
@@ -1339,9 +1342,9 @@ int gllmq_init(gllmq_ctx **out, int device)
                 snprintf(name, sizeof name, "gq_mmf_%s_t%d%s", q == 3 ? "q8_0" : q == 2 ? "q6k" : q == 1 ? "q5k" : "q4k", t + 1, b ? "_bf16" : "");
                 rc = get_function(ctx, &ctx->mmf_q4k[q][t][b], name);
             }
-    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8c[0], "gq_mm8c_q4k");
-    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8c[1], "gq_mm8c_q5k");
-    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8c[2], "gq_mm8c_q8_0");
+    static const char *const kMm8c[3][2] = { { "gq_mm8c_q4k", "gq_mm8c_q4k_f" }, { "gq_mm8c_q5k", "gq_mm8c_q5k_f" }, { "gq_mm8c_q8_0", "gq_mm8c_q8_0_f" } };
+    for (int q = 0; q < 3; ++q)
+        for (int v = 0; v < 2 && rc == GLLMQ_OK; ++v) rc = get_function(ctx, &ctx->mm8c[q][v], kMm8c[q][v]);
     for (int q = 0; q < 2 && rc == GLLMQ_OK; ++q)
         for (int b = 0; b < 2 && rc == GLLMQ_OK; ++b) {
             snprintf(name, sizeof name, "gq_mmfs_%s%s", q ? "q5k" : "q4k", b ? "_bf16" : "");

@@ -131,7 +131,7 @@ def test_every_entry_reads_the_output_of_the_one_before(torch, oracle):
         entries = [(wd[i], bufs[i], bufs[i + 1], Q4_K, 1, k, k) for i in range(steps)]
         print(f"chain: dependent entries, attempt {attempt}", flush=True)
         run_batch(hip, torch, entries, after_previous=lambda i: i > 0)
-        assert hip.last_kernel_name() == "gq_mm8c_q4k"
+        assert hip.last_kernel_name().startswith("gq_mm8c_q4k")
         got = [b.cpu().numpy() for b in bufs]
         for i in range(steps):
             assert np.isfinite(got[i + 1]).all(), f"step {i}: an entry started before its input was complete"
