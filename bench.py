@@ -524,13 +524,21 @@ def main():
         free = hip.make_batch([(ws[i % COPIES], x, ys[i % COPIES], DTYPE, M, N, K_DIM) for i in range(steps + COPIES)])
         t2 = measure(torch, lambda r: hip.run_batch(free, (r * steps) % COPIES, steps), steps, args.warmup)
         free_kernel = hip.last_kernel_name()
+        # (those entries share one activation row, as the Q, K and V projections of a token do, and
+        # a workgroup of the chained launch prepares a shared row once; with a row of its own per
+        # entry every entry is prepared)
+        xs = [torch.randn(M, K_DIM, device="cuda", generator=g) for _ in range(COPIES)]
+        own = hip.make_batch([(ws[i % COPIES], xs[i % COPIES], ys[i % COPIES], DTYPE, M, N, K_DIM) for i in range(steps + COPIES)])
+        t3 = measure(torch, lambda r: hip.run_batch(own, (r * steps) % COPIES, steps), steps, args.warmup)
         context = {"cache_resident_us_per_call": round(t1["us"], 3),
                    "device_copy_gbs_read_plus_write": round(2 * nb / tc["us"] / 1e3, 1),
                    "independent_entries": {"us_per_call": round(t2["us"], 3), "p10_us": round(t2["p10_us"], 3),
                                            "p90_us": round(t2["p90_us"], 3),
                                            "gbs": round(bytes_per_call / (t2["us"] * 1e-6) / 1e9, 1),
                                            "frac": round(bytes_per_call / (t2["us"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                                           "kernel": free_kernel}}
+                                           "kernel": free_kernel, "activations": "one row shared by all entries",
+                                           "own_row_per_entry_us_per_call": round(t3["us"], 3),
+                                           "own_row_per_entry_frac": round(bytes_per_call / (t3["us"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}}
     log(f"Q4_K GEMV 1x{K_DIM}x{N}: {us_per_call:.2f} us/call (p10 {t['p10_us']:.2f}, p90 {t['p90_us']:.2f}; "
         f"{t['regions']} regions of {steps} calls), {gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS * 100:.1f}% of 8 TB/s), "
         f"{2 * N * K_DIM / (us_per_call * 1e-6) / 1e12:.2f} TFLOP/s")
@@ -538,7 +546,8 @@ def main():
         log(f"  same weights every call (cache resident): {context['cache_resident_us_per_call']:.2f} us/call")
         ie = context["independent_entries"]
         log(f"  as independent entries of one batch call ({ie['kernel']}): {ie['us_per_call']:.2f} us/call, "
-            f"{ie['gbs']:.0f} GB/s ({ie['frac'] * 100:.1f}% of 8 TB/s)")
+            f"{ie['gbs']:.0f} GB/s ({ie['frac'] * 100:.1f}% of 8 TB/s); with an activation row of its own per entry "
+            f"{ie['own_row_per_entry_us_per_call']:.2f} us/call ({ie['own_row_per_entry_frac'] * 100:.1f}%)")
         log(f"  plain device-to-device copy of the same 33 MB buffers: {context['device_copy_gbs_read_plus_write']:.0f} GB/s read+write")
 
     result = {
