@@ -237,6 +237,7 @@ struct gllmq_ctx {
     bool moe_mm8 = true;                        // "moe_mm8" = 0: expert rows stay on the GEMV kernels
     bool moe_mm8_q6k = true;                    // "moe_mm8_q6k" = 0: Q6_K expert rows stay there
     bool moe_glu = true;                        // "moe_glu" = 0: gate/up results to memory, activation as a kernel of its own
+    uint32_t moe_slices = 0;                    // "moe_slices": workgroups that share a job's row tiles (0 = by the number of pairs and experts)
     bool moe_mm8_rows = true;                   // "moe_mm8_rows" = 0: no wave-per-tile kernel for short Q6_K rows
 
     // One lock over every enqueue on this context: calls from several threads take turns on the
@@ -1522,6 +1523,7 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "moe_mm8_q6k") ctx->moe_mm8_q6k = value != 0;
     else if (n == "moe_mm8_rows") ctx->moe_mm8_rows = value != 0;
     else if (n == "moe_glu") ctx->moe_glu = value != 0;
+    else if (n == "moe_slices") ctx->moe_slices = u;
     else if (n == "weights_cache_mib") ctx->weights_cache_limit = static_cast<size_t>(u) << 20;
     else return fail(ctx, GLLMQ_ERR_INVALID, "set_option: unknown option %s", name);
     return GLLMQ_OK;
@@ -2120,6 +2122,7 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate, size_t gate_bytes, size_t
         // upper bound of the jobs: one per expert hit, plus one per eight further pairs
         const uint64_t max_jobs = std::min<uint64_t>(pairs, experts + pairs / 8);
         uint32_t slices = std::max<uint32_t>(1u, (3u * static_cast<uint32_t>(ctx->num_cus)) / (2u * static_cast<uint32_t>(std::min<uint64_t>(pairs, experts))));
+        if (ctx->moe_slices) slices = ctx->moe_slices;
         const uint32_t ppt = (groups + 7u) / 8u;
         hipFunction_t fn = glu ? ctx->moe_mm8_glu_fn[kind][ppt - 1] : ctx->moe_mm8_fn[kind][ppt - 1];
         uint32_t units = Q.g.tiles; // what the slices of a job share: tiles, or groups of eight tiles
