@@ -50,8 +50,17 @@ def test_two_calls_in_a_row_second_smaller(hip, torch, dtype):
     for m, n, k in ((4, 1024, 8192), (2, 256, 4096), (4, 1024, 8192)):
         print(f"noalloc K split dtype={dtype} m={m} n={n} k={k}", flush=True)
         both(hip, torch, dtype, m, n, k, seed=5 * m)
-    # shapes without scratch go through the same entry point
+    # the streamed kernels' slices of K (sums and counters in the scratch as well): 32-row tiles
+    # for half of the CUs, long rows; then smaller; then again
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    for m, n, k in ((2, 16 * cus, 8192 + 512), (3, 16 * cus - 40, 8192), (2, 16 * cus, 8192 + 512)):
+        print(f"noalloc streamed K split dtype={dtype} m={m} n={n} k={k}", flush=True)
+        both(hip, torch, dtype, m, n, k, seed=7 * m)
+        if dtype != Q6_K or m == 2:
+            assert hip.last_kernel_name().endswith("_s"), hip.last_kernel_name()
+    # shapes without scratch go through the same entry point (also one row in pairs of blocks)
     both(hip, torch, dtype, 1, 777, 1024, seed=9)
+    both(hip, torch, dtype, 1, 12 * cus, 4096, seed=10)
 
 
 def test_baseline_shapes_fit(hip, torch):
