@@ -219,6 +219,7 @@ struct gllmq_ctx {
     hipFunction_t moe_gemv[kNumFormats] = {};
     hipFunction_t moe_mm8_fn[MM8_KINDS][2] = {}; // grouped int8 matrix-core kernels [Mm8Kind][passes per tile - 1]
     hipFunction_t moe_mm8_q6k_rows = nullptr;   // Q6_K rows of at most 8 blocks: a wave per 32-row tile
+    hipFunction_t moe_mm8s_fn[MM8_MOE_KINDS][2] = {}; // the grouped kernels in the streamed form [Mm8Kind][plain, gated]
     uint32_t *identity_rows = nullptr;          // device: 0..7, the activation rows of an ungathered matmul
 
     // Kernel-family choices (gllmq_set_option).  The defaults are the measured best; the tests
@@ -239,6 +240,8 @@ struct gllmq_ctx {
     bool moe_glu = true;                        // "moe_glu" = 0: gate/up results to memory, activation as a kernel of its own
     uint32_t moe_slices = 0;                    // "moe_slices": workgroups that share a job's row tiles (0 = by the number of pairs and experts)
     bool moe_mm8_rows = true;                   // "moe_mm8_rows" = 0: no wave-per-tile kernel for short Q6_K rows
+    uint32_t moe_streamed = 1;                  // "moe_streamed": the grouped kernels in the streamed form: 0 never, 1 while experts see few tokens each, 2 always
+    uint32_t moe_depth = 0;                     // "moe_depth": items a loader of the streamed grouped kernels keeps unconfirmed (0 = as the dense launches)
 
     // One lock over every enqueue on this context: calls from several threads take turns on the
     // host (the kernels they enqueue overlap as their streams allow).
@@ -1365,6 +1368,11 @@ int gllmq_init(gllmq_ctx **out, int device)
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[2][0], "gq_moe_mm8_q5k_a1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_fn[2][1], "gq_moe_mm8_q5k_a2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_q6k_rows, "gq_moe_mm8_q6k_rows");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8s_fn[MM8_Q4K][0], "gq_moe_mm8s_q4k");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8s_fn[MM8_Q5K][0], "gq_moe_mm8s_q5k");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8s_fn[MM8_Q6K][0], "gq_moe_mm8s_q6k");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8s_fn[MM8_Q4K][1], "gq_moe_mm8s_glu_q4k");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8s_fn[MM8_Q5K][1], "gq_moe_mm8s_glu_q5k");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_glu_fn[MM8_Q4K][0], "gq_moe_mm8_glu_q4k_a1");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_glu_fn[MM8_Q4K][1], "gq_moe_mm8_glu_q4k_a2");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_mm8_glu_fn[MM8_Q5K][0], "gq_moe_mm8_glu_q5k_a1");
@@ -1523,6 +1531,8 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "moe_mm8_q6k") ctx->moe_mm8_q6k = value != 0;
     else if (n == "moe_mm8_rows") ctx->moe_mm8_rows = value != 0;
     else if (n == "moe_glu") ctx->moe_glu = value != 0;
+    else if (n == "moe_streamed") ctx->moe_streamed = u;
+    else if (n == "moe_depth") ctx->moe_depth = u;
     else if (n == "moe_slices") ctx->moe_slices = u;
     else if (n == "weights_cache_mib") ctx->weights_cache_limit = static_cast<size_t>(u) << 20;
     else return fail(ctx, GLLMQ_ERR_INVALID, "set_option: unknown option %s", name);
@@ -2054,10 +2064,16 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate, size_t gate_bytes, size_t
     float *h = reinterpret_cast<float *>(ws + W.h);
     float *o = reinterpret_cast<float *>(ws + W.o);
 
+    // The streamed grouped kernels take up to four tokens per job (their ring shares the LDS with the
+    // tokens' digit planes), the others up to eight.  An expert with more tokens is read once per
+    // job, so the streamed form is for calls whose experts see few tokens each (at most two on
+    // average: decode batches); with more, jobs of eight read the weights half as often.
+    const bool streamed_jobs = ctx->use_mm8s && (ctx->moe_streamed == 2 || (ctx->moe_streamed == 1 && pairs <= 2 * experts));
+    const uint32_t job_shift = streamed_jobs ? 2u : 3u;
     const uint32_t fast = pairs <= 4096 ? 1u : 0u; // per-pair placement: quadratic in the pairs, but without serial LDS walks
     {
         MoePlanParams P{ route_expert, route_len, pair_src, pair_pos, jobs, jobs8, counters, static_cast<uint32_t>(tokens),
-                         static_cast<uint32_t>(top_k), static_cast<uint32_t>(experts), static_cast<uint32_t>(pairs), fast };
+                         static_cast<uint32_t>(top_k), static_cast<uint32_t>(experts), static_cast<uint32_t>(pairs), fast, job_shift };
         const uint32_t lds = static_cast<uint32_t>((pairs + 4 * experts + 4 + (fast ? 2 * pairs : 0)) * 4);
         rc = launch(ctx, ctx->moe_plan, 1, 256, lds, stream, &P, sizeof P);
         if (rc != GLLMQ_OK) return rc;
@@ -2119,8 +2135,8 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate, size_t gate_bytes, size_t
         Q.y_stride = y_stride;
         Q.g.glu_relu = relu_gate ? 1u : 0u;
         Q.rows = by_token ? nullptr : ctx->identity_rows;
-        // upper bound of the jobs: one per expert hit, plus one per eight further pairs
-        const uint64_t max_jobs = std::min<uint64_t>(pairs, experts + pairs / 8);
+        // upper bound of the jobs: one per expert hit, plus one per eight (four) further pairs
+        const uint64_t max_jobs = std::min<uint64_t>(pairs, experts + (pairs >> job_shift));
         uint32_t slices = std::max<uint32_t>(1u, (3u * static_cast<uint32_t>(ctx->num_cus)) / (2u * static_cast<uint32_t>(std::min<uint64_t>(pairs, experts))));
         if (ctx->moe_slices) slices = ctx->moe_slices;
         const uint32_t ppt = (groups + 7u) / 8u;
@@ -2129,6 +2145,32 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate, size_t gate_bytes, size_t
         if (q6k && groups <= 8 && ctx->moe_mm8_rows) {
             fn = ctx->moe_mm8_q6k_rows;
             units = (Q.g.tiles + 7u) / 8u;
+        }
+        // The streamed form (loader waves and arithmetic waves, a workgroup per CU): a slice is a range
+        // of whole tiles, and the ring is worked out per job in the kernel; it must exist for two and
+        // for four rows (a job of more rows runs as passes of four).
+        if (streamed_jobs && ctx->moe_mm8s_fn[kind][glu ? 1 : 0] && aligned(xin, 16)) {
+            const uint32_t sfmt = kind == MM8_Q6K ? 2u : kind == MM8_Q5K ? 1u : 0u;
+            const uint32_t pieces = sfmt == 2 ? gq::Mm8sFormat<2>::PIECES : sfmt == 1 ? gq::Mm8sFormat<1>::PIECES : gq::Mm8sFormat<0>::PIECES;
+            const uint32_t subs = sfmt == 2 ? 16u : 8u, item_bytes = 32u * pieces * 16u, lds_bytes = 160u * 1024u;
+            const uint32_t wg_tiles = (Q.g.tiles + std::min(slices, Q.g.tiles) - 1u) / std::min(slices, Q.g.tiles);
+            const uint32_t ranges = (Q.g.tiles + wg_tiles - 1u) / wg_tiles;
+            const uint32_t items = (glu ? 2u : 1u) * wg_tiles * groups;
+            gq::Mm8sLds L2, L4;
+            uint32_t slots, depth;
+            if (gq::mm8s_ring(groups, 2, item_bytes, items, subs, glu, lds_bytes, ctx->moe_depth, L2, slots, depth) &&
+                gq::mm8s_ring(groups, 4, item_bytes, items, subs, glu, lds_bytes, ctx->moe_depth, L4, slots, depth)) {
+                Q.slices = ranges;
+                Q.g.tile_rows = 32;
+                Q.g.rows_per_wg = 32u * wg_tiles;
+                Q.g.wg_tiles = wg_tiles;
+                Q.g.last_wg_rows = n - (ranges - 1u) * Q.g.rows_per_wg;
+                Q.g.last_wg_tiles = (Q.g.last_wg_rows + 31u) / 32u;
+                Q.g.lds_ring = lds_bytes; // the kernel carves it up per job
+                Q.g.depth = ctx->moe_depth;
+                return launch(ctx, ctx->moe_mm8s_fn[kind][glu ? 1 : 0], static_cast<uint32_t>(max_jobs * ranges),
+                              (gq::MM8S_CWAVES + gq::MM8S_LOADERS) * 64, lds_bytes, stream, &Q, sizeof Q);
+            }
         }
         slices = std::min(slices, units);
         Q.slices = slices;

@@ -195,6 +195,30 @@ GQ_HD inline Mm8sLds mm8s_lds_layout(uint32_t groups, uint32_t m, uint32_t pairs
     return L;
 }
 
+// Ring and loader depth of a streamed launch for `m` activation rows (1..4) whose items, `items`
+// per workgroup of `item_bytes` each, share `lds_bytes` of LDS with the preparation of `groups`
+// blocks: one or two rows keep one item per loader unconfirmed, three and four about
+// MM8S_DEPTH_BYTES.  False when the ring would be too short for the loaders to run ahead.
+// `want_depth` != 0: that many items per loader instead (a long stream gains from more of them).
+GQ_HD inline bool mm8s_ring(uint32_t groups, uint32_t m, uint32_t item_bytes, uint32_t items, uint32_t subs, bool glu,
+                            uint32_t lds_bytes, uint32_t want_depth, Mm8sLds &L, uint32_t &slots, uint32_t &depth)
+{
+    const uint32_t pairs = m <= 2u ? 1u : 2u;
+    L = mm8s_lds_layout(groups, m, pairs, item_bytes, 0u, subs, glu);
+    if (L.total + item_bytes > lds_bytes) return false;
+    slots = (lds_bytes - L.total) / item_bytes;
+    if (slots >= items) slots = items;
+    else slots -= slots % MM8S_LOADERS; // a reused ring is a whole number of rounds of the loaders
+    depth = 1u;
+    if (pairs > 1u) {
+        depth = (MM8S_DEPTH_BYTES + item_bytes / 2u) / item_bytes;
+        depth = depth < 2u ? 2u : (depth > MM8S_MAX_DEPTH ? MM8S_MAX_DEPTH : depth);
+    }
+    if (want_depth) depth = want_depth > MM8S_MAX_DEPTH ? MM8S_MAX_DEPTH : want_depth;
+    while (depth > (pairs > 1u ? 2u : 1u) && slots < items && slots < mm8s_min_slots(depth)) --depth;
+    return slots >= items || slots >= mm8s_min_slots(depth);
+}
+
 // Q6_K flavour (mm8_q6k.hip.inc)
 constexpr int MM8Q6_LOADS = 7;             // 16-byte loads per lane for one 32-row block tile (32 x 14 pieces)
 constexpr int MM8Q6_ROW_STRIDE = 240;      // bytes between rows in the stage: 224 used, padded against bank conflicts
@@ -359,7 +383,7 @@ struct MoeJob {
     uint32_t t0, t1; // their tokens (t1 = t0 when m = 1)
 };
 
-// All tokens of one expert, up to eight at a time: a job of the int8 matrix-core kernel.
+// All tokens of one expert, up to eight (or four) at a time: a job of the int8 matrix-core kernels.
 struct MoeJob8 {
     uint32_t expert;
     uint32_t p0;     // sorted position of the job's first pair
@@ -378,6 +402,7 @@ struct MoePlanParams {
     uint32_t *counters; // [0] jobs, [1] routed pairs, [2] eight-token jobs
     uint32_t tokens, top_k, experts, pairs;
     uint32_t fast; // pairs are few enough for the per-pair placement (LDS has two more arrays of `pairs` words)
+    uint32_t job_shift; // a matrix-core job takes up to 1 << job_shift tokens of an expert (3, or 2 for the streamed kernels)
 };
 
 constexpr uint32_t MOE_NONE = 0xFFFFFFFFu;

@@ -13,6 +13,7 @@
 #include "gemv_i8.hip.inc"
 #include "mm8.hip.inc"
 #include "mm8_q6k.hip.inc"
+#include "mm8s.hip.inc"
 #undef GQ_TEMPLATES_ONLY
 
 #include "moe.hip.inc"

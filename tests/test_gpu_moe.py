@@ -208,19 +208,24 @@ def test_moe_more_than_eight_tokens_per_expert(hip, torch, oracle, hidden, ffn):
     want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
     got = run_gpu(hip, torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, *dev)
     check_close(got, want, f"moe hidden={hidden} ffn={ffn}")
+    # the streamed grouped kernels (by default for experts with few tokens each): jobs of four tokens
+    from gllm_amd.backend import HipBackend
+    got = run_gpu(HipBackend(0, options={"moe_streamed": 2}), torch, gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, *dev)
+    check_close(got, want, f"moe streamed hidden={hidden} ffn={ffn}")
 
 
 def test_moe_grouped_kernel_alternatives(hip, torch, oracle):
-    """The grouped kernels the default dispatch does not pick for this shape: Q6_K down rows on
-    the tile-split matrix-core kernel and on the integer-dot GEMV, gate/up results through memory
-    with the activation as a kernel of its own."""
+    """The grouped kernels the default dispatch does not pick for this shape: the matrix-core
+    kernels whose waves fetch and multiply (a wave per tile and tile-split for the Q6_K down rows),
+    the integer-dot GEMV, gate/up results through memory with the activation as a kernel of its own."""
     from gllm_amd.backend import HipBackend
     experts, tokens, top_k, hidden, ffn = 6, 20, 3, 512, 1024
     gu, dn = expert_weights(Q4_K, Q6_K, experts, hidden, ffn, seed=95)
     x = random_activations(tokens, hidden, seed=96)
     dev, r = route_gpu(hip, torch, oracle, random_gate_logits(tokens, experts, seed=97), top_k, float(experts))
     want = oracle.moe_ffn(gu, Q4_K, dn, Q6_K, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
-    for options in ({"moe_mm8_rows": 0}, {"moe_mm8_q6k": 0}, {"moe_mm8": 0}, {"moe_glu": 0}):
+    for options in ({"moe_streamed": 0}, {"moe_streamed": 0, "moe_mm8_rows": 0}, {"moe_mm8_rows": 0}, {"moe_mm8_q6k": 0}, {"moe_mm8": 0},
+                    {"moe_glu": 0}, {"moe_streamed": 0, "moe_glu": 0}):
         hip2 = HipBackend(0, options=options)
         for split in (False, True):
             print(f"moe alternatives {options} split={split}", flush=True)
@@ -231,6 +236,8 @@ def test_moe_grouped_kernel_alternatives(hip, torch, oracle):
 def test_moe_random_shapes_sweep(hip, torch, oracle):
     """Sixteen seeded MoE shapes: formats in every role, expert counts from 2 to 40, top-k from 1
     to 6, ragged hidden/ffn sizes on both sides of the matrix-core kernels' limits."""
+    from gllm_amd.backend import HipBackend
+    streamed = HipBackend(0, options={"moe_streamed": 2})  # also where experts see many tokens each
     rng = np.random.default_rng(77)
     fmts = [Q4_K, Q5_K, Q6_K, Q8_0]
     for case in range(16):
@@ -248,6 +255,8 @@ def test_moe_random_shapes_sweep(hip, torch, oracle):
         want = oracle.moe_ffn(gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], threads=8)
         got = run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, *dev, split=bool(case & 1))
         check_close(got, want, f"moe sweep case {case}")
+        got = run_gpu(streamed, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, *dev, split=bool(case & 1))
+        check_close(got, want, f"moe sweep case {case}, streamed grouped kernels")
 
 
 def test_moe_many_pairs(hip, torch, oracle):
