@@ -2146,29 +2146,24 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate, size_t gate_bytes, size_t
             fn = ctx->moe_mm8_q6k_rows;
             units = (Q.g.tiles + 7u) / 8u;
         }
-        // The streamed form (loader waves and arithmetic waves, a workgroup per CU): a slice is a range
-        // of whole tiles, and the ring is worked out per job in the kernel; it must exist for two and
-        // for four rows (a job of more rows runs as passes of four).
-        if (streamed_jobs && ctx->moe_mm8s_fn[kind][glu ? 1 : 0] && aligned(xin, 16)) {
+        // The streamed form (loader waves and arithmetic waves, a workgroup per CU): the kernel cuts the
+        // tiles of all jobs into one run per workgroup and works the ring out per job; it must exist for
+        // two and for four rows over a run of any length.
+        if (streamed_jobs && ctx->moe_mm8s_fn[kind][glu ? 1 : 0] && aligned(xin, 16) && max_jobs * Q.g.tiles < 0x7FFFFFFFull) {
             const uint32_t sfmt = kind == MM8_Q6K ? 2u : kind == MM8_Q5K ? 1u : 0u;
             const uint32_t pieces = sfmt == 2 ? gq::Mm8sFormat<2>::PIECES : sfmt == 1 ? gq::Mm8sFormat<1>::PIECES : gq::Mm8sFormat<0>::PIECES;
             const uint32_t subs = sfmt == 2 ? 16u : 8u, item_bytes = 32u * pieces * 16u, lds_bytes = 160u * 1024u;
-            const uint32_t wg_tiles = (Q.g.tiles + std::min(slices, Q.g.tiles) - 1u) / std::min(slices, Q.g.tiles);
-            const uint32_t ranges = (Q.g.tiles + wg_tiles - 1u) / wg_tiles;
-            const uint32_t items = (glu ? 2u : 1u) * wg_tiles * groups;
+            const uint32_t items = (glu ? 2u : 1u) * Q.g.tiles * groups; // the longest piece: all tiles of a job
             gq::Mm8sLds L2, L4;
             uint32_t slots, depth;
             if (gq::mm8s_ring(groups, 2, item_bytes, items, subs, glu, lds_bytes, ctx->moe_depth, L2, slots, depth) &&
                 gq::mm8s_ring(groups, 4, item_bytes, items, subs, glu, lds_bytes, ctx->moe_depth, L4, slots, depth)) {
-                Q.slices = ranges;
+                Q.slices = 1;
                 Q.g.tile_rows = 32;
-                Q.g.rows_per_wg = 32u * wg_tiles;
-                Q.g.wg_tiles = wg_tiles;
-                Q.g.last_wg_rows = n - (ranges - 1u) * Q.g.rows_per_wg;
-                Q.g.last_wg_tiles = (Q.g.last_wg_rows + 31u) / 32u;
                 Q.g.lds_ring = lds_bytes; // the kernel carves it up per job
                 Q.g.depth = ctx->moe_depth;
-                return launch(ctx, ctx->moe_mm8s_fn[kind][glu ? 1 : 0], static_cast<uint32_t>(max_jobs * ranges),
+                const uint64_t wgs = std::min<uint64_t>(static_cast<uint64_t>(ctx->num_cus), max_jobs * Q.g.tiles);
+                return launch(ctx, ctx->moe_mm8s_fn[kind][glu ? 1 : 0], static_cast<uint32_t>(wgs),
                               (gq::MM8S_CWAVES + gq::MM8S_LOADERS) * 64, lds_bytes, stream, &Q, sizeof Q);
             }
         }
