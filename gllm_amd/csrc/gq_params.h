@@ -425,7 +425,7 @@ struct MoeMm8Params {
     uint64_t expert_stride;  // bytes between experts in g.w
     const uint8_t *up;       // gated form: the up rows of expert 0 (g.w then holds the gate rows)
     uint64_t up_stride;      // bytes between experts in `up`
-    uint32_t slices;         // workgroups that share one job's tiles
+    uint32_t slices;         // workgroups that share one job's tiles (the streamed kernels cut runs of tiles across jobs instead)
     uint32_t y_stride;       // elements between output rows (by sorted position)
     const uint32_t *rows;    // null: the activation rows are the job's tokens; else this table (0, 1, ...)
                              // counts from the job's first sorted position
