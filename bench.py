@@ -449,6 +449,7 @@ def cpu_baseline(budget_s: float = 12.0, simd_budget_s: float = 5.0):
 
 
 def main():
+    global COPIES
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
@@ -461,6 +462,10 @@ def main():
                          "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="kernel-family option of the library for this run (repeatable), e.g. mm8s=0")
+    ap.add_argument("--copies", type=int, default=COPIES,
+                    help="weight copies the headline workload rotates over (default 16 = 504 MiB, past every cache; fewer "
+                         "shows what the caches give: 2 copies fit the memory-side cache but no L2)")
+    ap.add_argument("--real-chain", action="store_true", help="every matmul reads the first K outputs of the one before it")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch plain device-to-device copies of one 33 MB weight buffer (counter calibration)")
     args = ap.parse_args()
@@ -484,6 +489,7 @@ def main():
         run_other(args)
         return
     hip = HipBackend(0, options=parse_options(args))
+    COPIES = max(1, args.copies)  # (module-level name: the helpers below read it)
     g = torch.Generator(device="cuda")
     g.manual_seed(0)
     ws = [device_weight_any(torch, g, DTYPE, N, K_DIM) for _ in range(COPIES)]
@@ -497,8 +503,13 @@ def main():
     # One list of steps + COPIES descriptors; region r is one C call over `steps` consecutive
     # entries starting where region r - 1 stopped in the rotation.
     # every entry is a call of its own: it starts after the one before it has finished
-    rotating = hip.make_batch([(ws[i % COPIES], x, ys[i % COPIES], DTYPE, M, N, K_DIM) for i in range(steps + COPIES)],
-                              after_previous=lambda i: True)
+    if args.real_chain:
+        ys = [torch.zeros(M, N, device="cuda") for _ in range(steps + COPIES)]
+        rotating = hip.make_batch([(ws[i % COPIES], x if i == 0 else ys[i - 1], ys[i], DTYPE, M, N, K_DIM) for i in range(steps + COPIES)],
+                                  after_previous=lambda i: True)
+    else:
+        rotating = hip.make_batch([(ws[i % COPIES], x, ys[i % COPIES], DTYPE, M, N, K_DIM) for i in range(steps + COPIES)],
+                                  after_previous=lambda i: True)
     resident = hip.make_batch([(ws[0], x, ys[0], DTYPE, M, N, K_DIM)] * steps, after_previous=lambda i: True)
 
     if args.copy_probe:

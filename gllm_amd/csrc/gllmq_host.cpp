@@ -20,6 +20,7 @@
 #include <string>
 #include <type_traits>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 // The code objects built from the kernels_*.hip translation units, placed in .rodata by the
@@ -146,10 +147,10 @@ struct Scratch {
     size_t moe_bytes = 0;
     void *elem = nullptr;        // 16-bit activations and outputs as f32, for the kernels that do not convert themselves
     size_t elem_bytes = 0;
+    void *box = nullptr;         // the chained launch's mailbox [kChainBoxPairs] of 64-bit words, zero when allocated
 };
 
 constexpr size_t kScratchArriveBytes = 4096; // MM8_SPLIT_MAX_LISTS words, padded; the chain kernel's counters behind them
-constexpr size_t kChainCountersAt = 512;     // first of its MM8C_MAX_ENTRIES + 1 words in that area
 constexpr size_t kLmHeadTicketAt = 600;      // the lm_head launch's count of finished workgroups
 constexpr size_t kScratchKeysBytes = sizeof(uint64_t) * gq::ARGMAX_MAX_ROWS * gq::ARGMAX_MAX_PARTS;
 constexpr size_t kScratchPartBytes = sizeof(float) * gq::MM8_SPLIT_PART_FLOATS;
@@ -204,7 +205,8 @@ struct gllmq_ctx {
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmfs[2][2] = {};              // its streamed form [0 = Q4_K, 1 = Q5_K][bf16 mode]
     hipFunction_t mm8c[3][2] = {};              // chains of streamed matmuls in one launch [0 = Q4_K, 1 = Q5_K, 2 = Q8_0][some entry in pairs of blocks]
-    bool chain_dependent = false;               // "chain_dependent" = 1: entries that depend on the one before stay in the chain
+    bool chain_dependent = false;               // "chain_dependent" = 1: an entry that reads the output of the one before it stays in the chained launch (measured slower than a launch of its own)
+    uint32_t chain_epoch = 1;                   // epochs handed to chained entries so far (see Mm8ChainParams::box)
     bool use_chain = true;                      // "chain" = 0: every entry of a batch is a launch of its own
     uint32_t chain_min_rows = 1;                // "chain_min_rows": fewest weight rows in a CU's share of an entry that joins a chain
     uint32_t chain_spin_limit = 1u << 20;       // "chain_spin_limit": polls of a dependency counter before a workgroup gives up
@@ -286,6 +288,24 @@ struct gllmq_ctx {
     hipFunction_t gemv_i8_e16[kNumFormats][2] = {}; // the integer-dot GEMV over 16-bit activations and outputs
     bool elem_fused = true;     // "elem_fused" = 0: 16-bit elements always through conversion launches
     hipFunction_t convert_elem = nullptr;
+    // Weight prefetch beside the dependent launches of a batch (touch.hip.inc).  Launches that
+    // take part are numbered per context; a kernel of `announces` raises *progress to its number
+    // when it starts, and the prefetch launch, on a stream of the context's own, reads the weights
+    // of launch s while launch s - 1 runs.
+    bool prefetch = false;                      // "prefetch" = 1: on (measured slower: the prefetch shares every CU's memory pipeline with the launch it runs beside)
+    uint32_t prefetch_wgs = 0;                  // "prefetch_wgs": workgroups of the prefetch launch (0 = one per CU)
+    uint32_t prefetch_threads = 64;             // "prefetch_threads": threads of each (64 .. 256)
+    uint32_t prefetch_timeout_us = 200;         // "prefetch_timeout_us": longest wait for the launch before an entry's
+    uint32_t prefetch_flags = 0;                // "prefetch_flags": TouchParams::flags
+    bool prefetch_announce = true;              // "prefetch_announce" = 0: the launches stay silent (for measurements)
+    uint32_t prefetch_min_kib = 4096;           // "prefetch_min_kib": smallest weight matrix worth a prefetch
+    hipFunction_t touch = nullptr;
+    hipStream_t side_stream = nullptr;
+    hipEvent_t side_event = nullptr;
+    unsigned long long *progress = nullptr;     // device
+    unsigned long long launch_seq = 0;          // number of the last launch that was given one
+    unsigned long long call_seq = 0;            // number the launch being enqueued announces itself under (0: none)
+    std::unordered_set<hipFunction_t> announces;
     std::mutex err_mutex;
     std::string err;
 };
@@ -366,6 +386,7 @@ void free_scratch(Scratch &S)
     if (S.ffn) (void)hipFree(S.ffn);
     if (S.moe) (void)hipFree(S.moe);
     if (S.elem) (void)hipFree(S.elem);
+    if (S.box) (void)hipFree(S.box);
     S = Scratch{};
 }
 
@@ -763,6 +784,8 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     P.lds_ctrl = L.ctrl;
     P.lds_ring = L.ring;
     P.depth = depth;
+    P.progress = ctx->call_seq && ctx->prefetch_announce ? ctx->progress : nullptr;
+    P.progress_seq = ctx->call_seq;
     const uint32_t lds = L.total;
     if (split) {
         P.ksplit = ksplit;
@@ -1094,14 +1117,50 @@ bool chain_entry_ok(const gllmq_ctx *ctx, const gllmq_matmul_desc &d, const gllm
     return d.n > 0 && (d.n + cus - 1) / cus >= ctx->chain_min_rows; // rows of the largest share
 }
 
+// Whether [a, a + an) and [b, b + bn) share a byte.
+bool ranges_meet(const void *a, size_t an, const void *b, size_t bn)
+{
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+    return a0 < b0 + bn && b0 < a0 + an;
+}
+
+constexpr size_t kChainBoxPairs = size_t(1) << 19; // 64-bit words of the mailbox (4 MiB per stream that runs such chains)
+
+// Whether entry `d`, flagged as starting after `prev`, reads (part of) prev's output and nothing
+// else, so that it can take its activations from what prev posts: one activation row anywhere
+// inside prev's output row, or all rows of an output whose rows are exactly as long as d's.
+bool chain_reads_previous(const gllmq_matmul_desc &d, const gllmq_matmul_desc &prev)
+{
+    const uintptr_t x = reinterpret_cast<uintptr_t>(d.x_dev), y = reinterpret_cast<uintptr_t>(prev.y_dev);
+    if (x < y || (x - y) % 4 != 0) return false;
+    const size_t at = (x - y) / 4;
+    if (d.m == 1) return at + d.k <= prev.n; // (the chain's entries share m)
+    return at == 0 && d.k == prev.n;
+}
+
 size_t chain_length(const gllmq_ctx *ctx, const gllmq_matmul_desc *descs, size_t count)
 {
     if (!ctx->use_chain || !ctx->use_mm8 || !ctx->use_mm8s || count < 2) return 0;
-    size_t len = 0;
+    size_t len = 0, posted = 0; // entries so far, and the mailbox places their posting entries take
     while (len < count && len < gq::MM8C_MAX_ENTRIES && !(descs[len].flags & ~1u) && chain_entry_ok(ctx, descs[len], descs[0])) {
-        // an entry that depends on the one before it starts a launch of its own unless told otherwise:
-        // waiting inside a launch costs more than the launch boundary
-        if (len > 0 && (descs[len].flags & 1u) && !ctx->chain_dependent) break;
+        const gllmq_matmul_desc &d = descs[len];
+        const size_t xb = d.m * d.k * 4, yb = d.m * d.n * 4;
+        const bool reads_prev = len > 0 && (d.flags & 1u) && ctx->chain_dependent && chain_reads_previous(d, descs[len - 1]) &&
+                                posted + descs[len - 1].m * descs[len - 1].n <= kChainBoxPairs;
+        // An entry that starts after the one before it and does not simply read its output begins a
+        // launch of its own: the launch boundary is the one wait that covers every case.
+        if (len > 0 && (d.flags & 1u) && !reads_prev) break;
+        // Workgroups run through the entries at their own pace: nothing an entry writes may be
+        // anything another entry of the launch reads from memory or writes.
+        bool clash = false;
+        for (size_t j = 0; j < len && !clash; ++j) {
+            const gllmq_matmul_desc &o = descs[j];
+            const bool o_reads_prev = j > 0 && (o.flags & 1u); // (then it reads the mailbox, not memory)
+            clash = ranges_meet(d.y_dev, yb, o.y_dev, o.m * o.n * 4) || (!o_reads_prev && ranges_meet(d.y_dev, yb, o.x_dev, o.m * o.k * 4)) ||
+                    (!reads_prev && ranges_meet(d.x_dev, xb, o.y_dev, o.m * o.n * 4));
+        }
+        if (clash || ranges_meet(d.y_dev, yb, d.x_dev, xb)) break;
+        if (reads_prev) posted += descs[len - 1].m * descs[len - 1].n;
         ++len;
     }
     return len;
@@ -1135,9 +1194,11 @@ int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t
     if (slots < gq::mm8s_min_slots(P.depth)) return -1;
     P.ring_slots = slots;
     P.spin_limit = ctx->chain_spin_limit;
-    P.done = S.mm8_arrive + kChainCountersAt;
+    P.epoch0 = ctx->chain_epoch;
     P.error = ctx->chain_error;
-    uint32_t launched = 0;
+    P.progress = ctx->call_seq ? ctx->progress : nullptr;
+    P.progress_seq = ctx->call_seq;
+    uint32_t launched = 0, box_used = 0;
     for (size_t i = 0; i < len; ++i) {
         const gllmq_matmul_desc &d = descs[i];
         Mm8ChainEntry &E = P.e[i];
@@ -1153,7 +1214,14 @@ int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t
         E.last_wg_rows = E.n - (E.grid - 1u) * E.rows_per_wg;
         E.last_wg_tiles = (E.last_wg_rows + E.tile_rows - 1u) / E.tile_rows;
         E.flags = i > 0 ? (d.flags & 1u) : 0u; // the chain's first entry is ordered by the stream
-        if (i > 0 && E.flags) P.e[i - 1].flags |= 2u;
+        if (i > 0 && E.flags) { // (chain_length() has checked that it reads the output of the entry before and that the places fit)
+            Mm8ChainEntry &B = P.e[i - 1];
+            B.flags |= 2u;
+            B.box_at = box_used;
+            box_used += P.m * B.n;
+            E.x_at = B.box_at + static_cast<uint32_t>((static_cast<const float *>(d.x_dev) - static_cast<const float *>(descs[i - 1].y_dev)));
+            E.x_ld = B.n;
+        }
         // one activation row over tiles of at most 16 weight rows: in pairs of blocks, as run_mm8s() would
         if (ctx->mm8s_fold_on && P.m == 1 && E.tile_rows <= 16 && P.groups > 8) E.flags |= 4u;
         launched = std::max(launched, E.grid);
@@ -1163,7 +1231,19 @@ int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t
         waits = waits || (P.e[i].flags & 3u) != 0u;
         folds = folds || (P.e[i].flags & 4u) != 0u;
     }
-    if (!waits) P.done = nullptr; // independent entries count nothing: no counters to set back at the end
+    if (waits) {
+        if (box_used > kChainBoxPairs) return -1;
+        if (!S.box) {
+            // first chain of this kind on the stream: the mailbox, all zero (epochs start at 1).  Not
+            // during a capture and not from a block of fixed size: the entries then take a launch each.
+            if (S.fixed || stream_is_capturing(stream)) return -1;
+            GLLMQ_HIP(ctx, hipSetDevice(ctx->device));
+            GLLMQ_HIP(ctx, hipMalloc(&S.box, kChainBoxPairs * 8));
+            GLLMQ_HIP(ctx, hipMemset(S.box, 0, kChainBoxPairs * 8));
+        }
+        P.box = static_cast<unsigned long long *>(S.box);
+        ctx->chain_epoch += static_cast<uint32_t>(len);
+    }
     P.launched = launched;
     return launch(ctx, ctx->mm8c[fmt][folds ? 1 : 0], launched, (gq::MM8C_CWAVES + gq::MM8C_LOADERS) * 64, P.lds_ring + slots * P.slot_bytes,
                   stream, &P, sizeof P, true);
@@ -1392,6 +1472,14 @@ int gllmq_init(gllmq_ctx **out, int device)
         if (he == hipSuccess) *ctx->chain_error = 0u;
         else rc = fail(ctx, GLLMQ_ERR_HIP, "error word: %s", hipGetErrorString(he));
     }
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->touch, "gq_touch");
+    if (rc == GLLMQ_OK) {
+        hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->progress), 256);
+        if (he == hipSuccess) he = hipMemset(ctx->progress, 0, 256);
+        if (he == hipSuccess) he = hipStreamCreateWithFlags(&ctx->side_stream, hipStreamNonBlocking);
+        if (he == hipSuccess) he = hipEventCreateWithFlags(&ctx->side_event, hipEventDisableTiming);
+        if (he != hipSuccess) rc = fail(ctx, GLLMQ_ERR_HIP, "prefetch stream: %s", hipGetErrorString(he));
+    }
     {
         static const struct { int pi, ei; const char *tag; } kMm8[] = {
             { 0, 0, "p1_e1" }, { 0, 1, "p1_e2" }, { 0, 2, "p1_e4" }, { 1, 1, "p2_e2" }, { 1, 2, "p2_e4" }, { 2, 2, "p4_e4" },
@@ -1453,6 +1541,20 @@ int gllmq_init(gllmq_ctx **out, int device)
                 rc = get_function(ctx, &ctx->mm8s_glu[q][v], name);
             }
     }
+    if (rc == GLLMQ_OK) {
+        // the kernels that say when they start (the streamed forms and their chain)
+        auto add = [&](hipFunction_t f) { if (f) ctx->announces.insert(f); };
+        for (auto &q : ctx->mm8s) for (hipFunction_t f : q) add(f);
+        for (auto &q : ctx->mm8s_gated) for (hipFunction_t f : q) add(f);
+        for (auto &q : ctx->mm8s_e16) for (hipFunction_t f : q) add(f);
+        for (auto &q : ctx->mm8s_glu) for (hipFunction_t f : q) add(f);
+        for (auto &q : ctx->mm8s_fold) for (hipFunction_t f : q) add(f);
+        for (auto &q : ctx->mm8s_split) for (auto &r : q) for (hipFunction_t f : r) add(f);
+        for (auto &q : ctx->mm8c) for (hipFunction_t f : q) add(f);
+    }
+    // the scratch array of the entry point that allocates nothing: found (and thereby placed on
+    // this device) now, while allocating is allowed
+    if (rc == GLLMQ_OK) rc = gq_noalloc_init(ctx, device);
     if (rc != GLLMQ_OK) {
         fprintf(stderr, "gllmq_init: %s\n", ctx->err.c_str());
         for (hipModule_t mod : ctx->modules)
@@ -1473,6 +1575,12 @@ void gllmq_destroy(gllmq_ctx *ctx)
         if (W.dev) (void)hipFree(W.dev);
     if (ctx->identity_rows) (void)hipFree(ctx->identity_rows);
     if (ctx->chain_error) (void)hipHostFree(ctx->chain_error);
+    if (ctx->side_stream) {
+        (void)hipStreamSynchronize(ctx->side_stream);
+        (void)hipStreamDestroy(ctx->side_stream);
+    }
+    if (ctx->side_event) (void)hipEventDestroy(ctx->side_event);
+    if (ctx->progress) (void)hipFree(ctx->progress);
     for (hipModule_t mod : ctx->modules)
         if (mod) (void)hipModuleUnload(mod);
     delete ctx;
@@ -1534,6 +1642,13 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "moe_streamed") ctx->moe_streamed = u;
     else if (n == "moe_depth") ctx->moe_depth = u;
     else if (n == "moe_slices") ctx->moe_slices = u;
+    else if (n == "prefetch") ctx->prefetch = value != 0;
+    else if (n == "prefetch_wgs") ctx->prefetch_wgs = u;
+    else if (n == "prefetch_threads") ctx->prefetch_threads = std::min(256u, std::max(64u, u & ~63u));
+    else if (n == "prefetch_timeout_us") ctx->prefetch_timeout_us = u;
+    else if (n == "prefetch_flags") ctx->prefetch_flags = u;
+    else if (n == "prefetch_announce") ctx->prefetch_announce = value != 0;
+    else if (n == "prefetch_min_kib") ctx->prefetch_min_kib = u;
     else if (n == "weights_cache_mib") ctx->weights_cache_limit = static_cast<size_t>(u) << 20;
     else return fail(ctx, GLLMQ_ERR_INVALID, "set_option: unknown option %s", name);
     return GLLMQ_OK;
@@ -1880,6 +1995,82 @@ int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w, size_t w_bytes, const 
     return gllmq_quantized_matmul_ex(ctx, w, w_bytes, x, y, dtype, m, n, k, GLLMQ_ACT_F32_SPLIT, stream);
 }
 
+namespace {
+
+// One launch (or chained launch) of a batch, as gllmq_quantized_matmul_batch will enqueue it.
+struct BatchUnit {
+    size_t first, len;
+    bool ordered;   // starts after everything before it
+    bool announces; // its kernel says when it starts
+    unsigned long long seq;
+};
+
+int batch_entry(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc &d, void *stream)
+{
+    constexpr uint32_t kElemBits = GLLMQ_DESC_ELEM_F16 | GLLMQ_DESC_ELEM_BF16;
+    if (d.flags & kElemBits)
+        return matmul_elem_on_scratch(ctx, S, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k,
+                                      (d.flags & GLLMQ_DESC_ELEM_F16) ? GLLMQ_ELEM_F16 : GLLMQ_ELEM_BF16, stream);
+    return matmul_on_scratch(ctx, S, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k, GLLMQ_ACT_F32_SPLIT, stream);
+}
+
+// The launches a batch will make, and which of them get their weights prefetched: an ordered
+// launch whose kernel and whose predecessor's kernel both say when they start (the predecessor's
+// start is the prefetch's cue, its own start tells a late prefetch to give up).  Nothing is
+// enqueued here: single entries go through the dispatch in counting mode.
+void plan_prefetch(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t count, void *stream,
+                   std::vector<BatchUnit> &units, std::vector<gq::TouchEntry> &touch)
+{
+    constexpr uint32_t kKnown = GLLMQ_DESC_AFTER_PREVIOUS | GLLMQ_DESC_ELEM_F16 | GLLMQ_DESC_ELEM_BF16;
+    for (size_t i = 0; i < count;) {
+        BatchUnit u{ i, 1, true, false, 0 };
+        const size_t chain = chain_length(ctx, descs + i, count - i);
+        if (chain >= 2) {
+            u.len = chain;
+            u.announces = true;
+        } else if (!(descs[i].flags & ~kKnown)) {
+            u.ordered = (descs[i].flags & GLLMQ_DESC_AFTER_PREVIOUS) != 0 || i == 0 || !ctx->batch_overlap;
+            ctx->probe = true;
+            ctx->probe_launches = 0;
+            ctx->probe_fn = nullptr;
+            const int rc = batch_entry(ctx, S, descs[i], stream);
+            ctx->probe = false;
+            u.announces = rc == GLLMQ_OK && ctx->probe_launches == 1 && ctx->announces.count(ctx->probe_fn) != 0;
+        }
+        u.seq = ++ctx->launch_seq;
+        units.push_back(u);
+        i += u.len;
+    }
+    for (size_t j = 1; j < units.size(); ++j) {
+        const BatchUnit &u = units[j];
+        const gllmq_matmul_desc &d = descs[u.first]; // (of a chain: its first matrix; the chain's own stream carries on from there)
+        if (!u.ordered || !u.announces || !units[j - 1].announces || !d.w_dev) continue;
+        const size_t bytes = std::min(d.w_bytes, d.n * gllmq_row_bytes(d.ggml_dtype, d.k));
+        if (bytes < (static_cast<size_t>(ctx->prefetch_min_kib) << 10)) continue;
+        touch.push_back(gq::TouchEntry{ static_cast<const uint8_t *>(d.w_dev), bytes, u.seq });
+    }
+}
+
+int launch_prefetch(gllmq_ctx *ctx, const std::vector<gq::TouchEntry> &touch)
+{
+    const uint32_t wgs = ctx->prefetch_wgs ? ctx->prefetch_wgs : static_cast<uint32_t>(ctx->num_cus);
+    for (size_t at = 0; at < touch.size(); at += gq::TOUCH_MAX_ENTRIES) {
+        gq::TouchParams T{};
+        T.progress = ctx->progress;
+        T.sink = nullptr;
+        T.count = static_cast<uint32_t>(std::min<size_t>(gq::TOUCH_MAX_ENTRIES, touch.size() - at));
+        T.timeout_ticks = ctx->prefetch_timeout_us * 100u; // wall_clock64() counts at 100 MHz
+        T.flags = ctx->prefetch_flags;
+        for (uint32_t i = 0; i < T.count; ++i) T.e[i] = touch[at + i];
+        size_t size = sizeof T;
+        void *config[] = { HIP_LAUNCH_PARAM_BUFFER_POINTER, &T, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END };
+        GLLMQ_HIP(ctx, hipModuleLaunchKernel(ctx->touch, wgs, 1, 1, ctx->prefetch_threads, 1, 1, 0, ctx->side_stream, nullptr, config));
+    }
+    return GLLMQ_OK;
+}
+
+} // namespace
+
 int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs, size_t count, void *stream)
 {
     if (!ctx) return GLLMQ_ERR_INVALID;
@@ -1895,8 +2086,21 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
         return fail(ctx, GLLMQ_ERR_HIP, "quantized_matmul_batch: an earlier chained launch timed out waiting for the entry before "
                                         "(option chain_spin_limit; is the device shared?): its outputs are invalid");
     }
+    // The prefetch launch goes first, on the context's own stream (never into a capture: it is not
+    // part of the caller's stream).
+    std::vector<BatchUnit> units;
+    std::vector<gq::TouchEntry> touch;
+    if (ctx->prefetch && count >= 2 && !stream_is_capturing(stream)) plan_prefetch(ctx, *S, descs, count, stream, units, touch);
+    if (!touch.empty()) {
+        rc = launch_prefetch(ctx, touch);
+        if (rc != GLLMQ_OK) return rc;
+    }
+    size_t unit = 0;
     for (size_t i = 0; i < count && rc == GLLMQ_OK; ++i) {
         const gllmq_matmul_desc &d = descs[i];
+        while (unit < units.size() && units[unit].first < i) ++unit;
+        const bool planned = !touch.empty() && unit < units.size() && units[unit].first == i && units[unit].announces;
+        ctx->call_seq = planned ? units[unit].seq : 0ull;
         // consecutive one-row matmuls of one kind run as one launch whose weight stream never stops
         const size_t chain = chain_length(ctx, descs + i, count - i);
         if (chain >= 2) {
@@ -1917,14 +2121,17 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
         // an entry that depends on the ones before it starts a new group: its first launch is an
         // ordinary one
         ctx->overlap.entry_first = !(d.flags & GLLMQ_DESC_AFTER_PREVIOUS);
-        if (d.flags & kElemBits)
-            rc = matmul_elem_on_scratch(ctx, *S, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k,
-                                        (d.flags & GLLMQ_DESC_ELEM_F16) ? GLLMQ_ELEM_F16 : GLLMQ_ELEM_BF16, stream);
-        else
-            rc = matmul_on_scratch(ctx, *S, d.w_dev, d.w_bytes, d.x_dev, d.y_dev, d.ggml_dtype, d.m, d.n, d.k,
-                                   GLLMQ_ACT_F32_SPLIT, stream);
+        rc = batch_entry(ctx, *S, d, stream);
     }
+    ctx->call_seq = 0;
     ctx->overlap = gllmq_ctx::Overlap{};
+    if (!touch.empty()) {
+        // The caller's stream ends behind the prefetch: whoever waits for the stream may free the
+        // weights, which the prefetch must then be through with.
+        hipError_t e = hipEventRecord(ctx->side_event, ctx->side_stream);
+        if (e == hipSuccess) e = hipStreamWaitEvent(static_cast<hipStream_t>(stream), ctx->side_event, 0);
+        if (e != hipSuccess && rc == GLLMQ_OK) rc = fail(ctx, GLLMQ_ERR_HIP, "prefetch: %s", hipGetErrorString(e));
+    }
     return rc;
 }
 

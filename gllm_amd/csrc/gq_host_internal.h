@@ -21,4 +21,8 @@ extern "C" GQ_INTERNAL int gq_quantized_matmul_on_block(gllmq_ctx *ctx, const vo
                                                         float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,
                                                         void *block_dev, size_t block_bytes, void *stream);
 
+// Looks up, once per device, the address of the device array behind gllmq_quantized_matmul_noalloc
+// (`device` must be current).  Called by gllmq_init, so that the entry point never has to.
+extern "C" GQ_INTERNAL int gq_noalloc_init(gllmq_ctx *ctx, int device);
+
 #endif

@@ -76,6 +76,30 @@ struct Mm8Params {
     // activations that are the gated product of two f32 vectors (the input of a feed-forward
     // block's down projection): x[i] = act(x[i]) * x[i + glu_off]; glu = 0 off, 1 SiLU, 2 SiLU behind a ReLU
     uint32_t glu, glu_off;
+    // streamed kernels: null, or the word that says which launch of the context has started (the
+    // weight prefetch of the launch behind this one waits for it): workgroup 0 raises it to
+    // `progress_seq` on its way in
+    unsigned long long *progress;
+    unsigned long long progress_seq;
+};
+
+// The weight prefetch that runs beside a sequence of dependent launches (touch.hip.inc): for each
+// entry, in order, wait until launch number `seq - 1` of the context has started (`progress`, see
+// Mm8Params), then pull the entry's bytes into the memory-side cache by reading one word of every
+// 128-byte line.  An entry whose own launch has already started, or whose wait runs out after
+// `timeout_ticks` of the 100 MHz clock, is skipped: the prefetch never holds anything up.
+constexpr uint32_t TOUCH_MAX_ENTRIES = 32;
+struct TouchEntry {
+    const uint8_t *w;
+    unsigned long long bytes;
+    unsigned long long seq;
+};
+struct TouchParams {
+    const unsigned long long *progress;
+    uint32_t *sink;          // null (a place the words read would go to if they were ever needed)
+    uint32_t count, timeout_ticks;
+    uint32_t flags, pad;     // bit 0: wait as usual but read nothing (for measurements)
+    TouchEntry e[TOUCH_MAX_ENTRIES];
 };
 
 constexpr uint32_t MM8_SPLIT_MAX_LISTS = 256;        // tile lists (workgroups per slice) of a K-split launch
@@ -293,17 +317,31 @@ struct Mm8ChainEntry {
     uint32_t n, ldy;
     // the entry's geometry, worked out by the host as for the streamed kernels: weight rows per
     // workgroup, workgroups that take part, tile height, tiles of a full and of the last
-    // workgroup, rows of the last workgroup; flags: bit 0 = starts after the entry before it, bit 1 =
-    // the entry behind it does (so this one says when its y is stored), bit 2 = its items are pairs
-    // of blocks (one activation row, tiles of at most 16 rows)
-    uint32_t rows_per_wg, grid, tile_rows, wg_tiles, last_wg_tiles, last_wg_rows, flags, pad;
+    // workgroup, rows of the last workgroup; flags: bit 0 = its x is (part of) the y of the entry
+    // before it, read from the mailbox, bit 1 = the entry behind it reads this one's y (so this one
+    // posts its outputs there), bit 2 = its items are pairs of blocks (one activation row, tiles
+    // of at most 16 rows)
+    uint32_t rows_per_wg, grid, tile_rows, wg_tiles, last_wg_tiles, last_wg_rows, flags;
+    // mailbox places (in pairs, see Mm8ChainParams::box): where this entry posts output row 0 (rows
+    // `n` apart), and where its own activation row 0 was posted by the entry before (rows `x_ld` apart)
+    uint32_t box_at, x_at, x_ld, pad;
 };
 struct Mm8ChainParams {
     uint32_t count, launched;     // entries, workgroups of the launch (the largest `grid`)
     uint32_t k, groups, row_bytes, m, ldx, act_bf16;
     uint32_t ring_slots, slot_bytes, depth, lds_ctrl, lds_ring, spin_limit;
-    uint32_t *done;               // [MM8C_MAX_ENTRIES + 1] workgroups through with each entry, and with the launch; zero at rest
-    uint32_t *error;              // host-visible word, set to 1 when a wait for `done` ran out
+    // Entries that read the output of the one before them inside the launch: every output of such
+    // a producer is also posted as one 64-bit word (epoch << 32 | value bits) with a device-scope
+    // store, entry e under epoch `epoch0 + e`; a reader loads the words it needs until all carry the
+    // producer's epoch.  A word says by itself that its value is there, so nobody waits for stores
+    // to be acknowledged, nothing is counted, and nothing is set back: epochs are the context's own
+    // count of chained entries, no earlier launch used them, and every entry of a launch has places
+    // of its own.  Null when no entry waits.
+    unsigned long long *box;
+    uint32_t epoch0, pad0;
+    uint32_t *error;              // host-visible word, set to 1 when a reader's wait ran out
+    unsigned long long *progress; // as in Mm8Params
+    unsigned long long progress_seq;
     Mm8ChainEntry e[MM8C_MAX_ENTRIES];
 };
 

@@ -14,3 +14,4 @@
 #include "ffn.hip.inc"
 #include "route.hip.inc"
 #include "convert.hip.inc"
+#include "touch.hip.inc"

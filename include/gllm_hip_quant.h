@@ -88,9 +88,11 @@ const char *gllmq_version(void);
  * int8 kernels), "mm8s_min_rows" (fewest weight rows per CU that take it), "mm8s_all" (1: that form wherever the
  * shape fits it, also where another kernel was timed faster), "mm8s_depth" (items a loader wave
  * keeps in flight; 0: by item size), "mmfs" / "mmfs_all" / "mmfs_min_rows" (the same three for the loader-wave
- * form of the f16 GEMM), "chain" (0: every entry of a batch is a launch of its own), "chain_dependent" (1: entries
- * that wait for the one before them stay inside a chained launch and wait there), "chain_spin_limit" (polls of such
- * a wait before a workgroup gives up and the next batch call reports it), "batch_overlap" (0: the kernels of a
+ * form of the f16 GEMM), "chain" (0: every entry of a batch is a launch of its own), "chain_dependent" (1: an entry
+ * whose activations are the output of the entry before it stays inside a chained launch and takes them from a mailbox
+ * in device memory as they are stored), "chain_spin_limit" (looks at that mailbox before a wave gives up and the next
+ * batch call reports it), "prefetch" (1: a launch on a stream of the context's own pulls the weights of each
+ * dependent launch of a batch into the memory-side cache while the launch before it runs; measured slower), "batch_overlap" (0: the kernels of a
  * batch run strictly one after the other), "ffn_fused" (0: the
  * feed-forward block in three steps), "mm8_q5k_min_m" / "mm8_q6k_min_m" / "mm8_q8_0_min_m"
  * (fewest rows that take the int8 matrix-core kernel; 0 = never), "mmf_small_min_m" (fewest rows
@@ -239,14 +241,16 @@ int gllmq_quantized_matmul_ex(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes,
  * capture, tight serving loops, harnesses that forbid allocation.  Same arguments, same kernels
  * and bit-identical results as gllmq_quantized_matmul, but the scratch (arrival counters and slice
  * sums of the K split, activation images and partial sums of the GEMM) is one array of
- * GLLMQ_NOALLOC_SCRATCH_BYTES in device memory that exists from the moment the library is loaded
- * (every GPU the library runs on holds its own copy until the process ends); the call allocates
- * and frees nothing.  A shape whose scratch does not fit (the GEMM's: about 72 KiB per 256
+ * GLLMQ_NOALLOC_SCRATCH_BYTES in device memory whose address gllmq_init looks up for the context's
+ * device (that lookup is what places the array there, so init fails if it cannot; every GPU the
+ * library runs on holds its own copy until the process ends); the call itself allocates and frees
+ * nothing and may be the first call on a fresh context, also under stream capture.  A shape whose scratch does not fit (the GEMM's: about 72 KiB per 256
  * elements of K for up to 64 rows plus ksplit * min(m, 64) * n * 4 bytes of partial sums, in
  * 27.9 MiB) returns GLLMQ_ERR_BAD_SHAPE with the two sizes in gllmq_last_error; every baseline
  * shape up to 64 rows fits.  All calls on one GPU share that GPU's array, whatever their context
  * or stream: calls that overlap in time on one GPU race, so keep them on one stream or order them
- * yourself.  The context's device must be the calling thread's current device. */
+ * yourself.  The context's device must be the calling thread's current device (checked on every
+ * call). */
 #define GLLMQ_NOALLOC_SCRATCH_BYTES (32u << 20)
 int gllmq_quantized_matmul_noalloc(gllmq_ctx *ctx, const void *w_dev, size_t w_bytes, const float *x_dev,
                                    float *y_dev, uint32_t ggml_dtype, size_t m, size_t n, size_t k,

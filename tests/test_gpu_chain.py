@@ -120,7 +120,7 @@ def test_every_entry_reads_the_output_of_the_one_before(torch, oracle):
     before it and reads what they stored.  Each step is checked against the oracle on the input
     the GPU actually had; twice, so the counters are seen to be back at zero."""
     from gllm_amd.backend import HipBackend
-    hip = HipBackend(0, options={"chain_dependent": 1})  # by default a dependent entry starts a launch of its own
+    hip = HipBackend(0, options={"chain_dependent": 1})  # by default such an entry starts a launch of its own
     k = 4096
     steps = 7
     ws = [random_weight(Q4_K, k, k, seed=20 + i) for i in range(steps)]
@@ -181,7 +181,7 @@ def many_entries(hip, torch, oracle):
 
 
 def test_a_wait_that_runs_out_is_reported_and_the_launch_still_ends(torch):
-    """With no polls allowed a workgroup that finds the entry before it unfinished gives up at once:
+    """With no repeats allowed a wave that finds its activations not yet posted gives up at once:
     the launch ends (nothing hangs), the next batch call reports the failure once, and the call
     after that works again."""
     from gllm_amd.backend import BackendError, HipBackend
@@ -190,9 +190,11 @@ def test_a_wait_that_runs_out_is_reported_and_the_launch_still_ends(torch):
     n = 56 * c
     wd = dev_weight(torch, random_weight(Q4_K, n, k, seed=1))
     x = torch.from_numpy(random_activations(1, k, seed=2)).cuda()
-    entries = [(wd, x, torch.empty(1, n, device="cuda"), Q4_K, 1, n, k) for _ in range(6)]
+    ys = [torch.empty(1, n, device="cuda") for _ in range(6)]
+    entries = [(wd, x if i == 0 else ys[i - 1], ys[i], Q4_K, 1, n, k) for i in range(6)]  # each reads the first k outputs of the one before
     print("chain: waits that run out", flush=True)
     run_batch(hip, torch, entries, after_previous=lambda i: i > 0)
+    assert hip.last_kernel_name().startswith("gq_mm8c_q4k")
     with pytest.raises(BackendError, match="timed out"):
         run_batch(hip, torch, entries, after_previous=lambda i: i > 0)
     hip.set_option("chain_spin_limit", 1 << 20)

@@ -83,3 +83,59 @@ def test_too_large_a_shape_is_refused_and_nothing_runs(hip, torch):
     assert bool((y == 5.0).all())
     # and the entry point still works afterwards
     both(hip, torch, Q4_K, 16, 520, 2048, seed=11)
+
+
+def test_first_call_of_a_fresh_context_under_capture_allocates_nothing(torch):
+    """A new context whose very first call is the no-alloc entry point, made while its stream is
+    being captured: the scratch array was placed at init, so the call records kernels only; the
+    replays (with a smaller shape in the same graph) give the bits of the allocating entry point.
+    (The capture runs in torch's default mode, in which an allocation by the capturing thread is an
+    error.)  And the very first, eager, call of another new context leaves the device's free memory
+    where it was: nothing is placed on the device by the call itself."""
+    from gllm_amd.backend import HipBackend
+    fresh = HipBackend(0)
+    ref = HipBackend(0)
+    shapes = ((32, 2048, 4096), (4, 1024, 8192), (16, 520, 2048))  # GEMM with K split, 8-row K split, smaller GEMM
+    ws = [torch.from_numpy(random_weight(Q4_K, n, k, seed=21 + i)).cuda() for i, (m, n, k) in enumerate(shapes)]
+    xs = [torch.empty(m, k, device="cuda") for m, n, k in shapes]
+    got = [torch.full((m, n), float("nan"), device="cuda") for m, n, k in shapes]
+    want = [torch.full((m, n), float("nan"), device="cuda") for m, n, k in shapes]
+    eager_first = HipBackend(0)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    print("noalloc: first call of a fresh context, eager", flush=True)
+    for (m, n, k), w, x, y in zip(shapes, ws, xs, got):
+        x.fill_(1.0)
+        eager_first.quantized_matmul_noalloc(w, x, y, Q4_K, m, n, k)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the first calls of a new context changed the device's free memory"
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    print("noalloc: first call of a fresh context under capture", flush=True)
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        for (m, n, k), w, x, y in zip(shapes, ws, xs, got):
+            fresh.quantized_matmul_noalloc(w, x, y, Q4_K, m, n, k)
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for i, ((m, n, k), x) in enumerate(zip(shapes, xs)):
+            x.copy_(torch.from_numpy(random_activations(m, k, seed=100 * rep + i)).cuda())
+        for y in got:
+            y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for (m, n, k), w, x, y, z in zip(shapes, ws, xs, got, want):
+            ref.quantized_matmul(w, x, z, Q4_K, m, n, k)
+        torch.cuda.synchronize()
+        for (m, n, k), y, z in zip(shapes, got, want):
+            assert not bool(torch.isnan(z).any())
+            assert torch.equal(y.view(torch.int32), z.view(torch.int32)), f"replay {rep} m={m} n={n} k={k}"
+    # eager calls afterwards: still nothing allocated by the entry point
+    free_mid = torch.cuda.mem_get_info()[0]
+    for (m, n, k), w, x, y in zip(shapes, ws, xs, got):
+        fresh.quantized_matmul_noalloc(w, x, y, Q4_K, m, n, k)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_mid
