@@ -168,9 +168,13 @@ def cpu_time(fn, budget_s=8.0, max_reps=200):
 
 
 def run_other(args):
+    print(json.dumps(workload_result(args, args.workload, not args.no_cpu)), flush=True)
+
+
+def workload_result(args, name, want_cpu):
     """The baseline configurations other than the headline one, and the ops on either side of the
     matmul.  Same timing method; weights (or outputs, for the write-dominated ops) rotate over
-    enough copies to exceed the 256 MB Infinity Cache."""
+    enough copies to exceed the 256 MB Infinity Cache.  Returns the JSON line's dict."""
     import numpy as np
     import torch
 
@@ -183,7 +187,6 @@ def run_other(args):
     g = torch.Generator(device="cuda")
     g.manual_seed(0)
     threads = max(1, min(os.cpu_count() or 1, 16))
-    name = args.workload
     steps = args.steps
     sec = sample = None
     extra = {}
@@ -232,7 +235,7 @@ def run_other(args):
         flops = sum(2 * m * n * k for dt, n, k, m in ops)
         desc = " + ".join(f"{TAGS[dt]} M={m} K={k} N={n}" for dt, n, k, m in ops)
         t = measure(torch, region, steps, args.warmup)
-        if not args.no_cpu:
+        if want_cpu:
             # CPU: the oracle's reference-style path on the same shapes (bounded sample)
             host = [(random_weight(dt, n, k, seed=i), random_activations(m, k, seed=i), dt, m, n, k)
                     for i, (dt, n, k, m) in enumerate(ops)]
@@ -269,7 +272,7 @@ def run_other(args):
         flops = 128 * 2 * (2 * F * H + H * F)
         desc = (f"MoE expert matvec: {E} experts, top-{KK}, {T} tokens, gate/up Q4_K [{2 * F}x{H}], down Q6_K [{H}x{F}], "
                 f"{e_act:.1f} distinct experts hit per call on average, no capacity drop")
-        if not args.no_cpu:
+        if want_cpu:
             # CPU: 8 experts' worth of the same shapes (a sixteenth of the weights), 16 tokens top-2
             Ec = 8
             gu_h, dn_h = random_weight(12, Ec * 2 * F, H, seed=1), random_weight(14, Ec * H, F, seed=2)
@@ -303,7 +306,7 @@ def run_other(args):
         flops = 2 * n * k
         desc = (f"lm_head {TAGS[dtype]} 1x{k}->{n} + greedy token, " +
                 ("one call, logits not written" if fused else "matmul then argmax") + f", rotating over {copies} matrices")
-        if not args.no_cpu:
+        if want_cpu:
             host_w, host_x = random_weight(dtype, n // 8, k, seed=0), random_activations(1, k, seed=0)
             sec, creps, cdt = cpu_time(lambda: cref.argmax_token(
                 cref.quantized_matmul(host_w, host_x, dtype, 1, n // 8, k, acc=cref.ACC_F32, threads=threads)[0]))
@@ -323,7 +326,7 @@ def run_other(args):
         byts = n * row_bytes(dtype, k) + n * k * 4
         flops = 0
         desc = f"Backend::dequantize {TAGS[dtype]} {n} x {k} (block bytes in, f32 out), rotating over {copies} matrices"
-        if not args.no_cpu:
+        if want_cpu:
             host_w = random_weight(dtype, n // 8, k, seed=0)
             sec, creps, cdt = cpu_time(lambda: cref.dequantize(host_w, dtype))
             sec *= 8.0
@@ -350,7 +353,7 @@ def run_other(args):
         byts = 2 * F * row_bytes(12, H) + H * row_bytes(14, F) + 2 * mm * H * 4
         flops = 2 * mm * (2 * F * H + H * F)
         desc = f"dense FFN M={mm}: gate/up Q4_K {H}->{F}, SwiGLU, down Q6_K {F}->{H}, rotating over {copies} weight sets"
-        if not args.no_cpu:
+        if want_cpu:
             Fc = F // 8  # an eighth of the intermediate size: an eighth of every matrix
             hg, hu = random_weight(12, Fc, H, seed=1), random_weight(12, Fc, H, seed=2)
             hd = random_weight(14, H, Fc, seed=3)
@@ -376,7 +379,7 @@ def run_other(args):
         flops = 0
         desc = (f"Op::QuantGather {TAGS[dtype]}: {count} ids into a {vocab} x {hidden} table (row blocks in, f32 rows out), "
                 f"rotating over {copies} id sets and outputs")
-        if not args.no_cpu:
+        if want_cpu:
             host_t = random_weight(dtype, 1024, hidden, seed=0)
             host_ids = np.random.default_rng(0).integers(0, 1024, count // 8).astype(np.uint32)
             sec, creps, cdt = cpu_time(lambda: cref.quant_gather(host_t, dtype, 1024, hidden, host_ids))
@@ -402,9 +405,54 @@ def run_other(args):
     if sec is not None:
         result["cpu_baseline"] = {"value": round(byts / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
                                   "us_per_call": round(sec * 1e6, 1), "sample": sample}
+    result["config"]["kernel"] = hip.last_kernel_name()
     log(f"{name}: {us:.2f} us/call (p10 {t['p10_us']:.2f}, p90 {t['p90_us']:.2f}, {t['regions']} regions of {steps}), "
         f"{gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS * 100:.1f}% of 8 TB/s)")
-    print(json.dumps(result), flush=True)
+    return result
+
+
+# The baseline's configurations beside the headline one: timed in the default run as well (GPU legs
+# only), so that every figure quoted for them is one a plain `python bench.py` prints.
+CONTEXT_CONFIGS = (("cfg1_gemv_q4k_4096", "gemv_q4k_4096"), ("cfg2_gemv_q6k", "gemv_q6k"), ("cfg3_layer_mix", "layer_mix"),
+                   ("cfg4_gemm_m16", "gemm_m16"), ("cfg4_gemm_m32", "gemm_m32"), ("cfg4_gemm_m64", "gemm_m64"), ("cfg5_moe", "moe"))
+
+
+def context_configs(args, torch):
+    out = {}
+    for key, name in CONTEXT_CONFIGS:
+        r = workload_result(args, name, False)
+        out[key] = {"workload": name, "us_per_call": r["us_per_call"], "p10_us": r["p10_us"], "p90_us": r["p90_us"],
+                    "gbs": r["value"], "frac": r["roofline"]["frac"], "tflops": r["tflops"],
+                    "bytes_per_call": r["config"]["bytes_per_call"], "kernel": r["config"]["kernel"], "what": r["config"]["workload"]}
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
+def launch_cadence_us(torch, kernels: int = 500):
+    """Time per kernel of a captured sequence of empty-handed kernels on one stream (each adds 1 to
+    one float): what the device needs from one dependent launch to the next, whatever the kernel."""
+    t = torch.zeros(1, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            t.add_(1.0)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(kernels):
+                t.add_(1.0)
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(12)]
+        graph.replay()
+        side.synchronize()
+        for i in range(11):
+            e[i].record(side)
+            graph.replay()
+        e[11].record(side)
+        side.synchronize()
+    per = sorted(e[i].elapsed_time(e[i + 1]) * 1e3 / kernels for i in range(11))
+    return round(per[len(per) // 2], 3)
 
 
 def cpu_baseline(budget_s: float = 12.0, simd_budget_s: float = 5.0):
@@ -462,6 +510,7 @@ def main():
                          "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="kernel-family option of the library for this run (repeatable), e.g. mm8s=0")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other baseline configurations in the headline run's context")
     ap.add_argument("--copies", type=int, default=COPIES,
                     help="weight copies the headline workload rotates over (default 16 = 504 MiB, past every cache; fewer "
                          "shows what the caches give: 2 copies fit the memory-side cache but no L2)")
@@ -541,7 +590,8 @@ def main():
         xs = [torch.randn(M, K_DIM, device="cuda", generator=g) for _ in range(COPIES)]
         own = hip.make_batch([(ws[i % COPIES], xs[i % COPIES], ys[i % COPIES], DTYPE, M, N, K_DIM) for i in range(steps + COPIES)])
         t3 = measure(torch, lambda r: hip.run_batch(own, (r * steps) % COPIES, steps), steps, args.warmup)
-        context = {"cache_resident_us_per_call": round(t1["us"], 3),
+        context = {"launch_cadence_us": launch_cadence_us(torch),
+                   "cache_resident_us_per_call": round(t1["us"], 3),
                    "device_copy_gbs_read_plus_write": round(2 * nb / tc["us"] / 1e3, 1),
                    "independent_entries": {"us_per_call": round(t2["us"], 3), "p10_us": round(t2["p10_us"], 3),
                                            "p90_us": round(t2["p90_us"], 3),
@@ -560,6 +610,7 @@ def main():
             f"{ie['gbs']:.0f} GB/s ({ie['frac'] * 100:.1f}% of 8 TB/s); with an activation row of its own per entry "
             f"{ie['own_row_per_entry_us_per_call']:.2f} us/call ({ie['own_row_per_entry_frac'] * 100:.1f}%)")
         log(f"  plain device-to-device copy of the same 33 MB buffers: {context['device_copy_gbs_read_plus_write']:.0f} GB/s read+write")
+        log(f"  one dependent launch to the next, whatever the kernel (graph of one-float kernels): {context['launch_cadence_us']:.2f} us")
 
     result = {
         "metric": "Q4_K GEMV 1x4096x14336: achieved HBM GB/s",
@@ -587,6 +638,11 @@ def main():
                              "the event time includes the gap between back-to-back launches"},
     }
     if context:
+        del ws, ys, rotating, resident, free, own, xs, dsts
+        gc.collect()
+        torch.cuda.empty_cache()
+        if not args.no_configs:
+            context["configs"] = context_configs(args, torch)
         result["context"] = context
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
