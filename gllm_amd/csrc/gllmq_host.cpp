@@ -204,6 +204,9 @@ struct gllmq_ctx {
     hipFunction_t moe_mm8_glu_fn[3][2] = {};    // gated gate/up kernels [Mm8Kind (Q4_K and Q5_K only)][passes per tile - 1]
     hipFunction_t mmf_q4k[4][2][2] = {};        // f16 matrix-core GEMM [0 = Q4_K, 1 = Q5_K, 2 = Q6_K, 3 = Q8_0][32-row activation tiles - 1][bf16 mode]
     hipFunction_t mmfs[2][2] = {};              // its streamed form [0 = Q4_K, 1 = Q5_K][bf16 mode]
+    hipFunction_t mmfr[2] = {};                 // the streamed form whose waves prepare their own activations (f32, 9 to 16 rows) [0 = Q4_K, 1 = Q5_K]
+    bool use_mmfr = true;                       // "mmfr" = 0: never
+    uint32_t mmfr_min_rows = 8;                 // "mmfr_min_rows": fewest weight rows per CU that take it
     hipFunction_t mm8c[3][2] = {};              // chains of streamed matmuls in one launch [0 = Q4_K, 1 = Q5_K, 2 = Q8_0][some entry in pairs of blocks]
     bool chain_dependent = false;               // "chain_dependent" = 1: an entry that reads the output of the one before it stays in the chained launch (measured slower than a launch of its own)
     uint32_t chain_epoch = 1;                   // epochs handed to chained entries so far (see Mm8ChainParams::box)
@@ -1098,6 +1101,76 @@ int run_mmfs(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, cons
     return GLLMQ_OK;
 }
 
+// Q4_K and Q5_K, 9 to 16 rows of f32 activations, from `mmfr_min_rows` weight rows per CU up: the
+// streamed GEMM whose arithmetic waves prepare their own activations (mmfr.hip.inc), one launch and
+// nothing else.  A workgroup multiplies a slice of K of eight blocks (a block per arithmetic wave);
+// the slices of a row range meet through the scratch.  Returns -1 for what it does not take.
+int run_mmfr(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m, size_t n,
+             size_t k, bool act_bf16, void *stream, size_t min_m = 9)
+{
+    const int fmt = f.dtype == T_Q5_K ? 1 : f.dtype == T_Q4_K ? 0 : -1;
+    // (17 rows and more: two ways of sharing a block between two waves were built and timed slower than the three-launch form)
+    if (!ctx->use_mmf || !ctx->use_mmfr || fmt < 0 || m < min_m || m > 16 || n == 0) return -1;
+    if (act_bf16 || ctx->call_elem || ctx->call_glu) return -1; // plain f32 activations and outputs
+    const uint32_t ldx = row_stride_x(ctx, k);
+    if (!aligned(x, 16) || k % 4 != 0 || ldx % 4 != 0) return -1; // activation rows are loaded as aligned float4
+    const uint32_t cus = static_cast<uint32_t>(ctx->num_cus);
+    if (n < static_cast<size_t>(ctx->mmfr_min_rows) * cus) return -1;
+    const uint32_t groups = static_cast<uint32_t>((k + 255) / 256);
+    const uint32_t pieces = fmt == 1 ? gq::Mm8sFormat<1>::PIECES : gq::Mm8sFormat<0>::PIECES;
+    const uint32_t sb = gq::MMFR_CWAVES; // blocks of a slice
+    const uint32_t ksplit = (groups + sb - 1u) / sb;
+    const uint32_t ranges = std::max(1u, cus / ksplit);
+    const uint32_t rows_per_wg = static_cast<uint32_t>((n + ranges - 1) / ranges);
+    const uint32_t grid = static_cast<uint32_t>((n + rows_per_wg - 1) / rows_per_wg);
+    // the loader's 32-bit offsets stay inside a workgroup's rows
+    if (static_cast<size_t>(rows_per_wg) * gllmq_row_bytes(f.dtype, k) > 0xFFFFFFFFull) return -1;
+    const uint32_t wg_tiles = (rows_per_wg + 31u) / 32u;
+    const uint32_t tile_rows = (rows_per_wg + wg_tiles - 1u) / wg_tiles; // equal heights, <= 32
+    if (ksplit > 1 && grid > kScratchArriveBytes / 4u) return -1;       // one arrival counter per row range
+    const uint32_t item_bytes = tile_rows * pieces * 16u;
+    const uint32_t lds_ring = (static_cast<uint32_t>(sizeof(gq::Mm8sCtrl)) + gq::MMFR_RED_BUFS * gq::MMFR_CWAVES * gq::MMFR_RED_WAVE + 1023u) & ~1023u;
+    const uint32_t items = wg_tiles * sb;
+    uint32_t slots = std::min(items, (160u * 1024u - lds_ring) / item_bytes);
+    if (slots < items) slots -= slots % gq::MMFR_LOADERS; // a reused ring is a whole number of rounds of the loaders
+    uint32_t depth = ctx->mm8s_depth ? std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth) : 1u;
+    while (depth > 2u && slots < items && slots < gq::mm8s_min_slots(depth)) --depth;
+    // (the waves of a tile's blocks run side by side: a ring shorter than two tiles' items would let a loader wait for a wave that waits for it)
+    if (slots < items && (slots < gq::mm8s_min_slots(depth) || slots < 2u * sb)) return -1;
+    const size_t part_bytes = ksplit > 1 ? static_cast<size_t>(ksplit) * grid * wg_tiles * 2048u : 0u;
+    if (part_bytes) {
+        int grc = grow_scratch(ctx, S, &S.mmf, &S.mmf_bytes, part_bytes, stream, "quantized_matmul (GEMM)");
+        if (grc != GLLMQ_OK) return grc;
+    }
+    Mm8Params P{};
+    P.w = w;
+    P.x = x;
+    P.y = y;
+    P.n = static_cast<uint32_t>(n);
+    P.k = static_cast<uint32_t>(k);
+    P.groups = groups;
+    P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
+    P.m = static_cast<uint32_t>(m);
+    P.ldx = ldx;
+    P.ldy = static_cast<uint32_t>(n);
+    P.grid = grid;
+    P.ksplit = ksplit;
+    P.kslice_groups = sb;
+    P.part = static_cast<float *>(S.mmf);
+    P.arrive = S.mm8_arrive;
+    P.rows_per_wg = rows_per_wg;
+    P.tile_rows = tile_rows;
+    P.ring_slots = slots;
+    P.wg_tiles = wg_tiles;
+    P.last_wg_rows = P.n - (grid - 1u) * rows_per_wg;
+    P.last_wg_tiles = (P.last_wg_rows + tile_rows - 1u) / tile_rows;
+    P.lds_ctrl = 0;
+    P.lds_ring = lds_ring;
+    P.depth = depth;
+    return launch(ctx, ctx->mmfr[fmt], grid * ksplit, (gq::MMFR_CWAVES + gq::MMFR_LOADERS) * 64, lds_ring + slots * item_bytes, stream, &P,
+                  sizeof P, ksplit > 1);
+}
+
 // A chain of batch entries for one launch of mm8c.hip.inc: consecutive matmuls of one format
 // (Q4_K or Q5_K), one K <= 4096 and one activation row count <= 2 that the streamed kernels
 // would take one by one.  chain_length() says how many entries from `descs` on form one (0 or 1:
@@ -1275,7 +1348,9 @@ int run_gemv(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
 int dispatch_matmul(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const float *x, float *y, size_t m,
                     size_t n, size_t k, bool bf16, void *stream)
 {
-    int rc = run_mmfs(ctx, S, f, w, x, y, m, n, k, bf16, stream);
+    int rc = run_mmfr(ctx, S, f, w, x, y, m, n, k, bf16, stream);
+    if (rc >= 0) return rc;
+    rc = run_mmfs(ctx, S, f, w, x, y, m, n, k, bf16, stream);
     if (rc >= 0 || rc == kNeedPlainActivations) return rc;
     rc = run_mmf(ctx, S, f, w, x, y, m, n, k, bf16, stream);
     if (rc >= 0 || rc == kNeedPlainActivations) return rc;
@@ -1434,6 +1509,8 @@ int gllmq_init(gllmq_ctx **out, int device)
             snprintf(name, sizeof name, "gq_mmfs_%s%s", q ? "q5k" : "q4k", b ? "_bf16" : "");
             rc = get_function(ctx, &ctx->mmfs[q][b], name);
         }
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmfr[0], "gq_mmfr_q4k");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mmfr[1], "gq_mmfr_q5k");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_plan, "gq_moe_plan");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_act, "gq_moe_act");
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->moe_combine, "gq_moe_combine");
@@ -1610,6 +1687,8 @@ int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value)
     else if (n == "mmf") ctx->use_mmf = value != 0;
     else if (n == "mm8s") ctx->use_mm8s = value != 0;
     else if (n == "mmfs") ctx->use_mmfs = value != 0;
+    else if (n == "mmfr") ctx->use_mmfr = value != 0;
+    else if (n == "mmfr_min_rows") ctx->mmfr_min_rows = std::max(1u, u);
     else if (n == "chain") ctx->use_chain = value != 0;
     else if (n == "chain_dependent") ctx->chain_dependent = value != 0;
     else if (n == "chain_spin_limit") ctx->chain_spin_limit = u;

@@ -361,6 +361,12 @@ constexpr int MMFS_LOADERS = 4; // loader waves (MM8S_LOADERS: the loader is the
 constexpr int MMFS_RED_BUFS = 3; // tiles whose block sums can be waiting in LDS
 static_assert(MMFS_LOADERS == MM8S_LOADERS, "mm8s_min_slots() is worked out for that many loaders");
 
+// The streamed GEMM whose waves prepare their own activations (mmfr.hip.inc).
+constexpr int MMFR_CWAVES = 8;   // arithmetic waves
+constexpr int MMFR_LOADERS = 4;  // loader waves (MM8S_LOADERS: the loader is the same code)
+constexpr int MMFR_RED_BUFS = 3; // tiles whose block sums can be waiting in LDS
+constexpr uint32_t MMFR_RED_WAVE = 2u * 64u * 16u; // bytes of a tile's sums in LDS per wave: [column tile][lane] float4
+
 struct MmfPrepParams {
     const float *x;
     uint8_t *ximg;

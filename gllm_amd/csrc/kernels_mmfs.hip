@@ -16,3 +16,4 @@
 #undef GQ_TEMPLATES_ONLY
 
 #include "mmfs.hip.inc"
+#include "mmfr.hip.inc"

@@ -88,7 +88,8 @@ const char *gllmq_version(void);
  * int8 kernels), "mm8s_min_rows" (fewest weight rows per CU that take it), "mm8s_all" (1: that form wherever the
  * shape fits it, also where another kernel was timed faster), "mm8s_depth" (items a loader wave
  * keeps in flight; 0: by item size), "mmfs" / "mmfs_all" / "mmfs_min_rows" (the same three for the loader-wave
- * form of the f16 GEMM), "chain" (0: every entry of a batch is a launch of its own), "chain_dependent" (1: an entry
+ * form of the f16 GEMM), "mmfr" / "mmfr_min_rows" (0: no one-launch GEMM for 9 to 16 rows of f32 activations, whose
+ * waves prepare their own operands; fewest weight rows per CU that take it), "chain" (0: every entry of a batch is a launch of its own), "chain_dependent" (1: an entry
  * whose activations are the output of the entry before it stays inside a chained launch and takes them from a mailbox
  * in device memory as they are stored), "chain_spin_limit" (looks at that mailbox before a wave gives up and the next
  * batch call reports it), "prefetch" (1: a launch on a stream of the context's own pulls the weights of each

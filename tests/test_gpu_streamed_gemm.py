@@ -19,7 +19,8 @@ Q4_K, Q5_K = 12, 13
 def hip():
     # "mmfs_all": the streamed form wherever the shape fits, not only where it was timed fastest
     from gllm_amd.backend import HipBackend
-    return HipBackend(0, options={"mmfs_all": 1})
+    # ("mmfr" = 0: not its successor, which prepares its own activations and would take these shapes)
+    return HipBackend(0, options={"mmfs_all": 1, "mmfr": 0})
 
 
 @pytest.fixture(scope="module")
@@ -70,7 +71,7 @@ def test_streamed_gemm_bf16_mode_and_repeats(hip, torch, oracle):
 def test_streamed_gemm_against_the_three_launch_form(hip, torch):
     """Also the default choice between the two: the streamed form up to 40 M weights."""
     from gllm_amd.backend import HipBackend
-    plain, default = HipBackend(0, options={"mmfs": 0}), HipBackend(0)
+    plain, default = HipBackend(0, options={"mmfs": 0, "mmfr": 0}), HipBackend(0, options={"mmfr": 0})
     c = cus(torch)
     x, w = random_activations(16, 1024, seed=1), random_weight(Q4_K, 16 * c, 1024, seed=2)
     gpu_matmul(default, torch, w, x, Q4_K, 16, 16 * c, 1024)
