@@ -113,6 +113,8 @@ def load_library() -> C.CDLL:
     L.gllmq_reserve_moe.argtypes = [vp, sz, sz, sz, sz, vp]
     L.gllmq_weights_forget.restype = None
     L.gllmq_weights_forget.argtypes = [vp, vp]
+    L.gllmq_chain_status.restype = C.c_int
+    L.gllmq_chain_status.argtypes = [vp]
     L.gllmq_weight_uploads.restype = C.c_uint64
     L.gllmq_weight_uploads.argtypes = [vp]
     L.gllmq_quant_gather.restype = C.c_int
@@ -141,7 +143,7 @@ EXPORTED_SYMBOLS = [
     "gllmq_init", "gllmq_destroy", "gllmq_last_error", "gllmq_status_string", "gllmq_version",
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
-    "gllmq_quantized_matmul_noalloc",
+    "gllmq_quantized_matmul_noalloc", "gllmq_chain_status",
     "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_lm_head_argmax", "gllmq_quantized_matmul_elem", "gllmq_reserve_matmul_elem", "gllmq_quant_gather", "gllmq_moe_route", "gllmq_set_option", "gllmq_last_kernel_name",
     "gllmq_reserve_matmul", "gllmq_reserve_ffn", "gllmq_reserve_moe", "gllmq_weights_forget", "gllmq_weight_uploads",
     "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
@@ -355,6 +357,11 @@ class HipBackend:
         rc = self._lib.gllmq_quantized_matmul_batch(self._ctx, first, count, self._stream())
         if rc != OK:
             self._raise(rc, "quantized_matmul_batch")
+
+    def chain_status(self) -> bool:
+        """After a synchronisation: whether a chained launch of a batch since the last look gave up
+        waiting for the entry before it (``gllmq_chain_status``; the look sets the flag back)."""
+        return bool(self._lib.gllmq_chain_status(self._ctx))
 
     def quantized_matmul_batch(self, descs) -> None:
         """descs: iterable of (w, x, y, quant_type, m, n, k) device tensors; one C call."""

@@ -80,6 +80,10 @@ struct gllmq_gguf {
     std::map<std::string, Value> meta;
     std::vector<Tensor> tensors;
     std::map<std::string, size_t> index;
+    // layer -> (projection -> tensor index) over the per-layer weights "blk.{layer}.{projection}.weight",
+    // built once when the file is opened; layers at or beyond `layer_limit` are not in it
+    std::map<size_t, std::map<std::string, size_t>> layers;
+    size_t layer_limit = 0;
 };
 
 namespace {
@@ -327,10 +331,13 @@ bool parse(gllmq_gguf *g, Error *err)
     return true;
 }
 
+void build_layer_table(gllmq_gguf *g);
+
 int finish_open(gllmq_gguf *g, gllmq_gguf **out, char *err_buf, size_t err_len)
 {
     Error e;
     if (parse(g, &e)) {
+        build_layer_table(g);
         *out = g;
         return GLLMQ_GGUF_OK;
     }
@@ -358,16 +365,37 @@ bool layer_weight_name(const std::string &name, size_t *layer, std::string *proj
     return true;
 }
 
-// layer -> (projection -> tensor index), over the per-layer weights of the file
-std::map<size_t, std::map<std::string, size_t>> layer_table(const gllmq_gguf *g)
+// The per-layer weights of the file.  Layer numbers come from tensor names, that is from the
+// file: the table holds layers below the model's declared layer count ("{architecture}.block_count",
+// when the file says so as an unsigned or non-negative number) and never more layers than the
+// file has tensors, so a stray "blk.99999999999999.x.weight" costs nothing.  The reference groups
+// layers below the model's num_layers and ignores stray higher indices the same way
+// (build_graph.inc.rs:416-428).
+void build_layer_table(gllmq_gguf *g)
 {
-    std::map<size_t, std::map<std::string, size_t>> table;
+    size_t limit = g->tensors.size();
+    const auto arch = g->meta.find("general.architecture");
+    if (arch != g->meta.end() && arch->second.type == 8 && arch->second.str) { // 8: string
+        const auto count = g->meta.find(std::string(arch->second.str, static_cast<size_t>(arch->second.len)) + ".block_count");
+        if (count != g->meta.end()) {
+            const Value &v = count->second;
+            const bool is_unsigned = v.type == 0 || v.type == 2 || v.type == 4 || v.type == 10; // u8, u16, u32, u64
+            const bool is_signed = v.type == 1 || v.type == 3 || v.type == 5 || v.type == 11;   // i8, i16, i32, i64
+            uint64_t n = v.bits;
+            bool ok = is_unsigned;
+            if (is_signed) {
+                const int bits = v.type == 1 ? 8 : v.type == 3 ? 16 : v.type == 5 ? 32 : 64;
+                ok = bits == 64 ? static_cast<int64_t>(n) >= 0 : ((n >> (bits - 1)) & 1u) == 0u;
+            }
+            if (ok && n < limit) limit = static_cast<size_t>(n);
+        }
+    }
+    g->layer_limit = limit;
     for (size_t i = 0; i < g->tensors.size(); ++i) {
         size_t layer;
         std::string proj;
-        if (layer_weight_name(g->tensors[i].name, &layer, &proj)) table[layer][proj] = i;
+        if (layer_weight_name(g->tensors[i].name, &layer, &proj) && layer < limit) g->layers[layer][proj] = i;
     }
-    return table;
 }
 
 const Value *find_meta(const gllmq_gguf *g, const char *key)
@@ -464,14 +492,13 @@ const void *gllmq_gguf_tensor_data(const gllmq_gguf *g, size_t index)
 size_t gllmq_gguf_layer_count(const gllmq_gguf *g)
 {
     if (!g) return 0;
-    const auto table = layer_table(g);
-    return table.empty() ? 0 : table.rbegin()->first + 1;
+    return g->layers.empty() ? 0 : g->layers.rbegin()->first + 1;
 }
 
 size_t gllmq_gguf_layer_tensors(const gllmq_gguf *g, size_t layer, size_t *indices, size_t capacity)
 {
     if (!g) return 0;
-    const auto table = layer_table(g);
+    const auto &table = g->layers;
     const auto it = table.find(layer);
     if (it == table.end()) return 0;
     size_t n = 0;
@@ -485,13 +512,16 @@ size_t gllmq_gguf_layer_tensors(const gllmq_gguf *g, size_t layer, size_t *indic
 long gllmq_gguf_layer_tensor(const gllmq_gguf *g, size_t layer, const char *projection)
 {
     if (!g || !projection) return -1;
-    return gllmq_gguf_find_tensor(g, ("blk." + std::to_string(layer) + "." + projection + ".weight").c_str());
+    const auto it = g->layers.find(layer);
+    if (it == g->layers.end()) return -1;
+    const auto pt = it->second.find(projection);
+    return pt == it->second.end() ? -1 : static_cast<long>(pt->second);
 }
 
 size_t gllmq_gguf_mixed_quant_groups(const gllmq_gguf *g, uint32_t *group_of, size_t capacity)
 {
     if (!g) return 0;
-    const auto table = layer_table(g);
+    const auto &table = g->layers;
     // a layer's signature: its (projection, dtype) pairs in projection order
     typedef std::vector<std::pair<std::string, uint32_t>> Signature;
     std::map<Signature, std::vector<size_t>> by_signature;

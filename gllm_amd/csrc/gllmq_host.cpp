@@ -476,7 +476,9 @@ int launch2d(gllmq_ctx *ctx, hipFunction_t f, uint32_t grid_x, uint32_t grid_y, 
     void *config[] = { HIP_LAUNCH_PARAM_BUFFER_POINTER, params, HIP_LAUNCH_PARAM_BUFFER_SIZE,
                        &params_size, HIP_LAUNCH_PARAM_END };
     gllmq_ctx::Overlap &ov = ctx->overlap;
-    const bool unordered = ov.on && ov.entry_first && ov.group_open && !(uses_scratch && ov.group_uses_scratch);
+    // (the launch without order takes the launch's size in threads as 32-bit numbers)
+    const bool unordered = ov.on && ov.entry_first && ov.group_open && !(uses_scratch && ov.group_uses_scratch) &&
+                           static_cast<uint64_t>(grid_x) * block <= 0xFFFFFFFFull;
     if (unordered) {
         GLLMQ_HIP(ctx, hipExtModuleLaunchKernel(f, grid_x * block, grid_y, 1, block, 1, 1, lds, static_cast<hipStream_t>(stream),
                                                 nullptr, config, nullptr, nullptr, hipExtAnyOrderLaunch));
@@ -2158,8 +2160,13 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
     Scratch *S = nullptr;
     int rc = acquire_scratch(ctx, stream, &S);
     if (rc != GLLMQ_OK) return rc;
+    // (a stream that is being captured gets ordinary launches throughout: what a capture makes of a
+    // launch without order is not something to rely on; the graph's replays then run the batch's
+    // kernels one after the other)
+    const bool capturing = stream_is_capturing(stream);
+    const bool overlap_on = ctx->batch_overlap && !capturing;
     ctx->overlap = gllmq_ctx::Overlap{};
-    ctx->overlap.on = ctx->batch_overlap;
+    ctx->overlap.on = overlap_on;
     if (*ctx->chain_error) { // a chain launched earlier gave up waiting for a counter: its results are not to be trusted
         *ctx->chain_error = 0u;
         return fail(ctx, GLLMQ_ERR_HIP, "quantized_matmul_batch: an earlier chained launch timed out waiting for the entry before "
@@ -2169,7 +2176,7 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
     // part of the caller's stream).
     std::vector<BatchUnit> units;
     std::vector<gq::TouchEntry> touch;
-    if (ctx->prefetch && count >= 2 && !stream_is_capturing(stream)) plan_prefetch(ctx, *S, descs, count, stream, units, touch);
+    if (ctx->prefetch && count >= 2 && !capturing) plan_prefetch(ctx, *S, descs, count, stream, units, touch);
     if (!touch.empty()) {
         rc = launch_prefetch(ctx, touch);
         if (rc != GLLMQ_OK) return rc;
@@ -2187,7 +2194,7 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
             if (crc >= 0) {
                 rc = crc;
                 ctx->overlap = gllmq_ctx::Overlap{};
-                ctx->overlap.on = ctx->batch_overlap;
+                ctx->overlap.on = overlap_on;
                 i += chain - 1;
                 continue;
             }
@@ -2212,6 +2219,15 @@ int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs,
         if (e != hipSuccess && rc == GLLMQ_OK) rc = fail(ctx, GLLMQ_ERR_HIP, "prefetch: %s", hipGetErrorString(e));
     }
     return rc;
+}
+
+int gllmq_chain_status(gllmq_ctx *ctx)
+{
+    if (!ctx || !ctx->chain_error) return 0;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    const uint32_t raised = *static_cast<volatile uint32_t *>(ctx->chain_error);
+    *ctx->chain_error = 0u;
+    return raised ? 1 : 0;
 }
 
 int gllmq_moe_route(gllmq_ctx *ctx, const float *logits, size_t tokens, size_t experts, size_t top_k,

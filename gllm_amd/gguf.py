@@ -180,6 +180,11 @@ class GgufFile:
         v = C.c_uint64()
         return v.value if self._lib.gllmq_gguf_meta_u64(self._h, key.encode(), C.byref(v)) else None
 
+    def layer_count(self) -> int:
+        """Highest layer with a per-layer weight, plus one, among the layers below the model's declared
+        layer count (gllmq_gguf_layer_count)."""
+        return int(self._lib.gllmq_gguf_layer_count(self._h))
+
     def layer_table(self) -> dict:
         """``{layer: {projection: TensorInfo}}`` over the per-layer weights ``blk.{layer}.{projection}.weight``
         (attn_q, attn_k, attn_v, attn_output, ffn_gate, ffn_up, ffn_down, ...): the (layer, projection) ->

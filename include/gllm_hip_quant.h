@@ -283,6 +283,17 @@ typedef struct gllmq_matmul_desc {
 int gllmq_quantized_matmul_batch(gllmq_ctx *ctx, const gllmq_matmul_desc *descs, size_t count,
                                  void *stream);
 
+/* With option "chain_dependent" an entry whose activations are the output of the entry before it
+ * stays inside the chained launch and waits there for those outputs, a bounded number of looks
+ * (option "chain_spin_limit"); a wave whose wait runs out goes on with what it has, so the launch
+ * always ends, and raises a word in host-visible memory.  That word is looked at by the NEXT
+ * gllmq_quantized_matmul_batch call on the context, which fails with GLLMQ_ERR_HIP once (the
+ * outputs of the launch that timed out are invalid), and by this function: after the caller has
+ * waited for the stream, 1 if a chained launch since the last look timed out (and the word is set
+ * back, so the next batch call reports nothing), 0 if none did.  No counterpart in the reference,
+ * whose decode step has no waits of its own. */
+int gllmq_chain_status(gllmq_ctx *ctx);
+
 /* ---- MoE router: gate logits -> route table ------------------------------------------
  * Replaces the graph ops MoEGate + TopK (src/arch/auto_graph_fragments/build_graph.inc.rs:2064-2071)
  * and their host mirror ExpertRouteTable::from_gate_logits (src/moe/routing.rs:100-160) over

@@ -54,6 +54,7 @@ extern "C" {
                                      act_mode: c_int, stream: *mut c_void) -> c_int;
     pub fn gllmq_quantized_matmul_batch(ctx: *mut gllmq_ctx, descs: *const gllmq_matmul_desc, count: usize,
                                         stream: *mut c_void) -> c_int;
+    pub fn gllmq_chain_status(ctx: *mut gllmq_ctx) -> c_int;
     pub fn gllmq_moe_route(ctx: *mut gllmq_ctx, logits_dev: *const f32, tokens: usize, experts: usize, top_k: usize,
                            capacity_factor: f32, route_expert_dev: *mut u32, route_weight_dev: *mut f32,
                            route_len_dev: *mut u32, route_pos_dev: *mut u32, expert_counts_dev: *mut u32,

@@ -219,3 +219,22 @@ def test_layer_table_with_gaps_and_other_names():
     groups = g.mixed_quant_groups()
     # signatures in order: (ffn_down Q4_K), (ffn_down Q4_K, ffn_up Q4_K), (ffn_down Q6_K)
     assert [layers for _, layers in groups] == [[0], [5], [2]]
+
+
+def test_stray_layer_indices_cost_nothing():
+    """Layer numbers come from tensor names: a file with a tensor named blk.99999999999999.x.weight
+    must not make the table (or anything sized by the layer count) that large.  Layers at or beyond
+    the declared `{architecture}.block_count` are ignored, as the reference ignores layers beyond
+    num_layers (build_graph.inc.rs:416-428); without the key nothing beyond the tensor count is."""
+    w = lambda name, dt: (name, [256, 4], dt, np.asarray(random_weight(dt, 4, 256, seed=1)).tobytes())
+    tensors = [w("blk.0.ffn_down.weight", Q4_K), w("blk.1.ffn_down.weight", Q6_K), w("blk.99999999999999.ffn_down.weight", Q4_K),
+               w("blk.7.ffn_down.weight", Q4_K)]
+    declared = GgufFile(image=W.build([("general.architecture", W.STR, "llama"), ("llama.block_count", W.U32, 2)], tensors))
+    assert declared.layer_count() == 2 and list(declared.layer_table()) == [0, 1]
+    assert declared.layer_tensor(7, "ffn_down") is None and declared.layer_tensor(99999999999999, "ffn_down") is None
+    assert [layers for _, layers in declared.mixed_quant_groups()] == [[0], [1]]
+    undeclared = GgufFile(image=W.build([("general.architecture", W.STR, "llama")], tensors))
+    assert undeclared.layer_count() == 2 and list(undeclared.layer_table()) == [0, 1]  # four tensors: layers 0..3 at most
+    signed = GgufFile(image=W.build([("general.architecture", W.STR, "llama"), ("llama.block_count", W.I32, -1)], tensors))
+    assert signed.layer_count() == 2  # a negative count reads as absent
+    assert declared.tensor("blk.7.ffn_down.weight").ggml_dtype == Q4_K  # still a tensor of the file

@@ -200,3 +200,75 @@ def test_a_wait_that_runs_out_is_reported_and_the_launch_still_ends(torch):
     hip.set_option("chain_spin_limit", 1 << 20)
     run_batch(hip, torch, entries, after_previous=lambda i: i > 0)  # the error was reported once; this one runs
     run_batch(hip, torch, entries, after_previous=lambda i: i > 0)
+
+
+def test_a_wait_that_runs_out_can_be_asked_for(torch):
+    """gllmq_chain_status after a synchronisation: set once by the launch whose wait ran out, set back
+    by the look, so that the next batch call has nothing to report."""
+    from gllm_amd.backend import HipBackend
+    hip = HipBackend(0, options={"chain_spin_limit": 0, "chain_dependent": 1})
+    c, k = cus(torch), 4096
+    n = 56 * c
+    wd = dev_weight(torch, random_weight(Q4_K, n, k, seed=1))
+    x = torch.from_numpy(random_activations(1, k, seed=2)).cuda()
+    ys = [torch.empty(1, n, device="cuda") for _ in range(6)]
+    entries = [(wd, x if i == 0 else ys[i - 1], ys[i], Q4_K, 1, n, k) for i in range(6)]
+    assert not hip.chain_status()
+    print("chain: status after a wait that ran out", flush=True)
+    run_batch(hip, torch, entries, after_previous=lambda i: i > 0)
+    assert hip.chain_status() and not hip.chain_status()
+    hip.set_option("chain_spin_limit", 1 << 20)
+    run_batch(hip, torch, entries, after_previous=lambda i: i > 0)  # nothing left to report
+    assert not hip.chain_status()
+
+
+def test_a_captured_batch_replays_like_the_eager_one(torch, oracle):
+    """A batch with a chained launch (Q, K, V on one x), an entry that waits for it, independent entries
+    of other kinds and an entry of sixteen rows, captured into a graph: every replay gives the bits
+    of the eager call on the same inputs (a captured batch runs its kernels as ordinary launches)."""
+    from gllm_amd.backend import HipBackend
+    hip = HipBackend(0)
+    c, k = cus(torch), 2048
+    ns = [16 * c, 4 * c, 4 * c, 12 * c, 9 * c, 8 * c]
+    dts = [Q4_K, Q4_K, Q4_K, Q4_K, 14, Q5_K]
+    ms = [1, 1, 1, 1, 1, 16]
+    ws = [dev_weight(torch, random_weight(dt, n, k, seed=70 + i)) for i, (dt, n) in enumerate(zip(dts, ns))]
+    x1, x16 = torch.empty(1, k, device="cuda"), torch.empty(16, k, device="cuda")
+    def outputs():
+        return [torch.full((m, n), float("nan"), device="cuda") for m, n in zip(ms, ns)]
+    got, want = outputs(), outputs()
+    def entries(ys):
+        return [(w, x16 if m == 16 else x1, y, dt, m, n, k) for w, y, dt, m, n in zip(ws, ys, dts, ms, ns)]
+    flags = lambda i: i == 3  # the fourth entry starts after the chain of the first three
+    eager = hip.make_batch(entries(want), after_previous=flags)
+    captured = hip.make_batch(entries(got), after_previous=flags)
+    x1.copy_(torch.from_numpy(random_activations(1, k, seed=1)).cuda())
+    x16.copy_(torch.from_numpy(random_activations(16, k, seed=2)).cuda())
+    hip.run_batch(captured, 0, len(ns))  # once eagerly: the stream's scratch exists before the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    print("chain: a batch inside a graph", flush=True)
+    with torch.cuda.stream(side):
+        hip.run_batch(captured, 0, len(ns))
+        side.synchronize()
+        graph.capture_begin()
+        hip.run_batch(captured, 0, len(ns))
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for rep in range(3):
+        x1.copy_(torch.from_numpy(random_activations(1, k, seed=10 + rep)).cuda())
+        x16.copy_(torch.from_numpy(random_activations(16, k, seed=20 + rep)).cuda())
+        for y in got:
+            y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        hip.run_batch(eager, 0, len(ns))
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert not bool(torch.isnan(b).any())
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32)), f"replay {rep}, entry {i}"
+    x = x1.cpu().numpy()
+    check_close(got[0].cpu().numpy(), oracle.quantized_matmul(random_weight(Q4_K, ns[0], k, seed=70), x, Q4_K, 1, ns[0], k,
+                                                               acc=oracle.ACC_F64, threads=16), "entry 0 of the last replay")
