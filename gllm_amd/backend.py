@@ -30,6 +30,7 @@ DESC_ELEM_F16, DESC_ELEM_BF16 = 0x100, 0x200  # gllmq_matmul_desc.flags: element
 
 
 ELEM_F32, ELEM_F16, ELEM_BF16 = 0, 1, 2  # gllmq_quantized_matmul_elem: element type of activations and outputs
+OUT_ACCUMULATE = 1  # flags of gllmq_ffn_swiglu_elem / gllmq_moe_matvec_elem: add to the output instead of replacing it
 ARGMAX_NONE = 0xFFFFFFFF  # gllmq_argmax: the row has no entry that is not NaN
 
 
@@ -121,6 +122,13 @@ def load_library() -> C.CDLL:
     L.gllmq_quant_gather.argtypes = [vp, vp, sz, u32, sz, sz, vp, sz, C.c_float, vp, vp]
     L.gllmq_ffn_swiglu.restype = C.c_int
     L.gllmq_ffn_swiglu.argtypes = [vp, vp, vp, sz, u32, vp, sz, u32, vp, vp, sz, sz, sz, C.c_int, vp]
+    L.gllmq_ffn_swiglu_elem.restype = C.c_int
+    L.gllmq_ffn_swiglu_elem.argtypes = [vp, vp, vp, sz, u32, vp, sz, u32, vp, vp, sz, sz, sz, C.c_int, C.c_int, C.c_int, vp]
+    L.gllmq_moe_matvec_elem.restype = C.c_int
+    L.gllmq_moe_matvec_elem.argtypes = [vp, vp, sz, sz, vp, sz, sz, u32, vp, sz, sz, u32, vp, vp, sz, sz, sz, sz, sz, vp, vp, vp,
+                                        C.c_int, C.c_int, C.c_int, vp]
+    L.gllmq_quant_gather_elem.restype = C.c_int
+    L.gllmq_quant_gather_elem.argtypes = [vp, vp, sz, u32, sz, sz, vp, sz, C.c_float, vp, C.c_int, vp]
     L.gllmq_argmax.restype = C.c_int
     L.gllmq_argmax.argtypes = [vp, vp, sz, sz, sz, vp, vp, vp]
     L.gllmq_quantized_matmul_elem.restype = C.c_int
@@ -143,7 +151,7 @@ EXPORTED_SYMBOLS = [
     "gllmq_init", "gllmq_destroy", "gllmq_last_error", "gllmq_status_string", "gllmq_version",
     "gllmq_block_size", "gllmq_block_bytes", "gllmq_row_bytes", "gllmq_dequantize",
     "gllmq_quantized_matmul", "gllmq_quantized_matmul_ex", "gllmq_quantized_matmul_batch",
-    "gllmq_quantized_matmul_noalloc", "gllmq_chain_status",
+    "gllmq_quantized_matmul_noalloc", "gllmq_chain_status", "gllmq_ffn_swiglu_elem", "gllmq_moe_matvec_elem", "gllmq_quant_gather_elem",
     "gllmq_moe_matvec", "gllmq_ffn_swiglu", "gllmq_argmax", "gllmq_lm_head_argmax", "gllmq_quantized_matmul_elem", "gllmq_reserve_matmul_elem", "gllmq_quant_gather", "gllmq_moe_route", "gllmq_set_option", "gllmq_last_kernel_name",
     "gllmq_reserve_matmul", "gllmq_reserve_ffn", "gllmq_reserve_moe", "gllmq_weights_forget", "gllmq_weight_uploads",
     "gllmq_dequantize_host", "gllmq_quant_gather_host", "gllmq_quantized_matmul_host",
@@ -377,34 +385,49 @@ class HipBackend:
         dt = _dtype_id(quant_type)
         if not (_is_torch(table) and table.is_cuda and token_ids.is_cuda and output.is_cuda):
             raise OtherError("quant_gather: tensors must live on the GPU")
-        if token_ids.element_size() != 4 or token_ids.is_floating_point() or output.dtype != self._torch.float32:
-            raise OtherError("quant_gather: token ids must be 32-bit integers, output f32")
+        elem = self._elem_of(output.dtype)
+        if token_ids.element_size() != 4 or token_ids.is_floating_point() or elem is None:
+            raise OtherError("quant_gather: token ids must be 32-bit integers, output f32, f16 or bf16")
         count = token_ids.numel()
         if output.numel() < count * hidden_dim:
             raise OtherError("quant_gather: output shorter than len(ids) * hidden_dim")
-        rc = self._lib.gllmq_quant_gather(self._ctx, table.data_ptr(), table.numel() * table.element_size(), dt,
-                                          vocab_size, hidden_dim, token_ids.data_ptr(), count,
-                                          1.0 if scale is None else float(scale), output.data_ptr(), self._stream())
+        if elem == ELEM_F32:
+            rc = self._lib.gllmq_quant_gather(self._ctx, table.data_ptr(), table.numel() * table.element_size(), dt,
+                                              vocab_size, hidden_dim, token_ids.data_ptr(), count,
+                                              1.0 if scale is None else float(scale), output.data_ptr(), self._stream())
+        else:
+            rc = self._lib.gllmq_quant_gather_elem(self._ctx, table.data_ptr(), table.numel() * table.element_size(), dt,
+                                                   vocab_size, hidden_dim, token_ids.data_ptr(), count,
+                                                   1.0 if scale is None else float(scale), output.data_ptr(), elem, self._stream())
         if rc != OK:
             self._raise(rc, "quant_gather")
 
     def ffn_swiglu(self, gate, up, dtype_gate_up, down, dtype_down, x, out, m: int, hidden: int, ffn: int,
-                   relu_gate: bool = False) -> None:
+                   relu_gate: bool = False, accumulate: bool = False) -> None:
         """Dense feed-forward block on device tensors: ``out = (silu(x gate^T) * (x up^T)) down^T``;
         ``gate`` and ``up`` are ``[ffn x hidden]`` blocks of ``dtype_gate_up`` (``up`` may be the second
-        half of one stacked tensor), ``down`` is ``[hidden x ffn]`` of ``dtype_down``."""
+        half of one stacked tensor), ``down`` is ``[hidden x ffn]`` of ``dtype_down``; ``x`` and ``out``
+        f32, f16 or bf16 (both of one type); ``accumulate``: ``out += ...`` (the shared-expert and
+        residual adds behind the block)."""
         for t in (gate, up, down, x, out):
             if not (_is_torch(t) and t.is_cuda):
                 raise OtherError("ffn_swiglu: tensors must live on the GPU")
-        if x.dtype != self._torch.float32 or out.dtype != self._torch.float32:
-            raise OtherError("ffn_swiglu: x and out must be f32")
+        elem = self._elem_of(x.dtype)
+        if elem is None or out.dtype != x.dtype:
+            raise OtherError("ffn_swiglu: x and out must be f32, f16 or bf16, both of one type")
         if x.numel() < m * hidden or out.numel() < m * hidden:
             raise OtherError("ffn_swiglu: x/out shorter than m * hidden")
         gb, ub = gate.numel() * gate.element_size(), up.numel() * up.element_size()
-        rc = self._lib.gllmq_ffn_swiglu(self._ctx, gate.data_ptr(), up.data_ptr(), min(gb, ub), _dtype_id(dtype_gate_up),
-                                        down.data_ptr(), down.numel() * down.element_size(), _dtype_id(dtype_down),
-                                        x.data_ptr(), out.data_ptr(), m, hidden, ffn, 1 if relu_gate else 0,
-                                        self._stream())
+        if elem == ELEM_F32 and not accumulate:
+            rc = self._lib.gllmq_ffn_swiglu(self._ctx, gate.data_ptr(), up.data_ptr(), min(gb, ub), _dtype_id(dtype_gate_up),
+                                            down.data_ptr(), down.numel() * down.element_size(), _dtype_id(dtype_down),
+                                            x.data_ptr(), out.data_ptr(), m, hidden, ffn, 1 if relu_gate else 0,
+                                            self._stream())
+        else:
+            rc = self._lib.gllmq_ffn_swiglu_elem(self._ctx, gate.data_ptr(), up.data_ptr(), min(gb, ub), _dtype_id(dtype_gate_up),
+                                                 down.data_ptr(), down.numel() * down.element_size(), _dtype_id(dtype_down),
+                                                 x.data_ptr(), out.data_ptr(), m, hidden, ffn, 1 if relu_gate else 0,
+                                                 elem, OUT_ACCUMULATE if accumulate else 0, self._stream())
         if rc != OK:
             self._raise(rc, "ffn_swiglu")
 
@@ -468,12 +491,16 @@ class HipBackend:
 
     def moe_matvec(self, gate_up, dtype_gate_up, down, dtype_down, x, out, hidden: int, ffn: int,
                    experts: int, route_expert, route_weight, route_len, relu_gate: bool = False,
-                   up=None) -> None:
+                   up=None, accumulate: bool = False) -> None:
         """Expert matvec over a route table.  ``gate_up``: per expert ``ffn`` gate rows followed by
         ``ffn`` up rows (one stacked tensor), or, with ``up`` given, the gate rows of all experts
         (``[experts, ffn, hidden]``) with ``up`` holding the up rows the same way (GGUF's layout);
-        ``down``: ``[experts, hidden, ffn]``."""
+        ``down``: ``[experts, hidden, ffn]``; ``x`` and ``out`` f32, f16 or bf16 (both of one type);
+        ``accumulate``: ``out += ...``."""
         tokens, top_k = route_expert.shape
+        elem = self._elem_of(x.dtype)
+        if elem is None or out.dtype != x.dtype:
+            raise OtherError("moe_matvec: x and out must be f32, f16 or bf16, both of one type")
         dgu, ddn = _dtype_id(dtype_gate_up), _dtype_id(dtype_down)
         each = ffn * self._lib.gllmq_row_bytes(dgu, hidden)  # 0 for a dtype the library does not cover
         gbytes = gate_up.numel() * gate_up.element_size()
@@ -483,11 +510,14 @@ class HipBackend:
         else:
             gate_ptr, gate_b, gate_st = gate_up.data_ptr(), gbytes, each
             up_ptr, up_b, up_st = up.data_ptr(), up.numel() * up.element_size(), each
-        rc = self._lib.gllmq_moe_matvec(
-            self._ctx, gate_ptr, gate_b, gate_st, up_ptr, up_b, up_st, dgu,
-            down.data_ptr(), down.numel() * down.element_size(), hidden * self._lib.gllmq_row_bytes(ddn, ffn), ddn,
-            x.data_ptr(), out.data_ptr(), tokens, hidden, ffn, experts, top_k, route_expert.data_ptr(),
-            route_weight.data_ptr(), route_len.data_ptr(), int(relu_gate), self._stream())
+        args = (self._ctx, gate_ptr, gate_b, gate_st, up_ptr, up_b, up_st, dgu,
+                down.data_ptr(), down.numel() * down.element_size(), hidden * self._lib.gllmq_row_bytes(ddn, ffn), ddn,
+                x.data_ptr(), out.data_ptr(), tokens, hidden, ffn, experts, top_k, route_expert.data_ptr(),
+                route_weight.data_ptr(), route_len.data_ptr(), int(relu_gate))
+        if elem == ELEM_F32 and not accumulate:
+            rc = self._lib.gllmq_moe_matvec(*args, self._stream())
+        else:
+            rc = self._lib.gllmq_moe_matvec_elem(*args, elem, OUT_ACCUMULATE if accumulate else 0, self._stream())
         if rc != OK:
             self._raise(rc, "moe_matvec")
 

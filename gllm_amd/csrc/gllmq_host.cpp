@@ -171,6 +171,8 @@ struct gllmq_ctx {
     hipModule_t modules[9] = {}; // one per embedded code object
     hipFunction_t dequant[kNumFormats][2] = {}; // [format][0 = scalar stores, 1 = float4 stores]
     hipFunction_t gather[kNumFormats][2] = {};  // quantized embedding lookup [format][0 = scalar stores, 1 = float4 stores]
+    hipFunction_t gather_e16[kNumFormats][2] = {}; // the same into rows of a 16-bit element type [format][0 = scalar stores, 1 = 8-byte stores]
+    hipFunction_t finish_elem = nullptr;        // f32 result in scratch -> output of any element type, plain or added to it
     // gated form of the int8 kernels (gate and up rows in one launch, act(gate) * up out):
     // [0 = Q4_K, 1 = Q5_K][pairs 1,2,4][early steps 1,2,4] and the register-operand variants
     hipFunction_t mm8_glu[2][3][3] = {};
@@ -1474,6 +1476,12 @@ int gllmq_init(gllmq_ctx **out, int device)
         if (rc != GLLMQ_OK) break;
         snprintf(name, sizeof name, "gq_gather_%s_v4", kFormats[i].tag);
         rc = get_function(ctx, &ctx->gather[i][1], name);
+        if (rc != GLLMQ_OK) break;
+        snprintf(name, sizeof name, "gq_gather_%s_e16_v1", kFormats[i].tag);
+        rc = get_function(ctx, &ctx->gather_e16[i][0], name);
+        if (rc != GLLMQ_OK) break;
+        snprintf(name, sizeof name, "gq_gather_%s_e16_v4", kFormats[i].tag);
+        rc = get_function(ctx, &ctx->gather_e16[i][1], name);
         for (int m = 1; m <= 2 && rc == GLLMQ_OK; ++m) {
             snprintf(name, sizeof name, "gq_gemv_%s_m%d", kFormats[i].tag, m);
             rc = get_function(ctx, &ctx->gemv[i][m - 1], name);
@@ -1552,6 +1560,7 @@ int gllmq_init(gllmq_ctx **out, int device)
         else rc = fail(ctx, GLLMQ_ERR_HIP, "error word: %s", hipGetErrorString(he));
     }
     if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->touch, "gq_touch");
+    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->finish_elem, "gq_finish_elem");
     if (rc == GLLMQ_OK) {
         hipError_t he = hipMalloc(reinterpret_cast<void **>(&ctx->progress), 256);
         if (he == hipSuccess) he = hipMemset(ctx->progress, 0, 256);
@@ -1769,7 +1778,16 @@ int gllmq_dequantize(gllmq_ctx *ctx, const void *blocks, size_t n_bytes, float *
 int gllmq_quant_gather(gllmq_ctx *ctx, const void *table, size_t table_bytes, uint32_t dtype, size_t vocab,
                        size_t hidden, const uint32_t *ids, size_t count, float scale, float *out, void *stream)
 {
+    return gllmq_quant_gather_elem(ctx, table, table_bytes, dtype, vocab, hidden, ids, count, scale, out, GLLMQ_ELEM_F32, stream);
+}
+
+int gllmq_quant_gather_elem(gllmq_ctx *ctx, const void *table, size_t table_bytes, uint32_t dtype, size_t vocab,
+                            size_t hidden, const uint32_t *ids, size_t count, float scale, void *out, int elem, void *stream)
+{
     if (!ctx) return GLLMQ_ERR_INVALID;
+    if (elem != GLLMQ_ELEM_F32 && elem != GLLMQ_ELEM_F16 && elem != GLLMQ_ELEM_BF16)
+        return fail(ctx, GLLMQ_ERR_INVALID, "quant_gather: unknown element type %d", elem);
+    const bool e16 = elem != GLLMQ_ELEM_F32;
     std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
     const Format *f = find_format(dtype);
     if (!f)
@@ -1784,21 +1802,22 @@ int gllmq_quant_gather(gllmq_ctx *ctx, const void *table, size_t table_bytes, ui
     if (table_bytes < vocab * rb)
         return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "quant_gather: table has %zu bytes, %zu rows of %zu elements need %zu",
                     table_bytes, vocab, hidden, vocab * rb);
-    if (!aligned(ids, 4) || !aligned(out, 4))
-        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "quant_gather: ids and output must be 4-byte aligned");
+    if (!aligned(ids, 4) || !aligned(out, e16 ? 2 : 4))
+        return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "quant_gather: ids must be 4-byte aligned, the output aligned to its element");
     GatherParams P{};
     P.table = static_cast<const uint8_t *>(table);
     P.ids = ids;
-    P.out = out;
+    P.out = static_cast<float *>(out);
     P.vocab = static_cast<uint32_t>(vocab);
     P.hidden = static_cast<uint32_t>(hidden);
     P.row_bytes = static_cast<uint32_t>(rb);
     P.quads_per_row = static_cast<uint32_t>(hidden / 4);
     P.count = static_cast<uint32_t>(count);
     P.scale = scale;
-    const int vec = aligned(out, 16) ? 1 : 0; // hidden is a multiple of 4, so every row then is
+    P.elem = static_cast<uint32_t>(elem);
+    const int vec = aligned(out, e16 ? 8 : 16) ? 1 : 0; // hidden is a multiple of 4, so every row then is
     // (a one-block-per-wave form as in gq_dequant_q4k_wave measured the same: 15.9 against 16.0 us)
-    return launch2d(ctx, ctx->gather[format_index(dtype)][vec], (P.quads_per_row + 255u) / 256u,
+    return launch2d(ctx, (e16 ? ctx->gather_e16 : ctx->gather)[format_index(dtype)][vec], (P.quads_per_row + 255u) / 256u,
                     static_cast<uint32_t>(std::min<size_t>(count, 65535)), 256, 0, stream, &P, sizeof P);
 }
 
@@ -2068,6 +2087,93 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_
         if (rc != GLLMQ_OK) return rc;
     }
     return dispatch_matmul(ctx, S, *fd, static_cast<const uint8_t *>(down_w), h, out, m, hidden, ffn, false, stream);
+}
+
+namespace {
+
+// What the element-type forms of the feed-forward block and of the expert matvec have in common:
+// activations of a 16-bit type are widened into the stream's scratch (exact), the f32 entry point
+// runs on them, and unless the result can go straight to `out` (f32, nothing to add) it goes to
+// scratch too and one small launch writes out = round(result) or out = round(out + result).
+struct ElemStage {
+    const float *x = nullptr; // what the f32 entry point reads
+    float *result = nullptr;  // where it writes
+    bool finish = false;
+};
+
+int elem_stage_begin(gllmq_ctx *ctx, const void *x, void *out, size_t count, int elem, int flags, void *stream, const char *what,
+                     ElemStage *st)
+{
+    if (elem != GLLMQ_ELEM_F32 && elem != GLLMQ_ELEM_F16 && elem != GLLMQ_ELEM_BF16)
+        return fail(ctx, GLLMQ_ERR_INVALID, "%s: unknown element type %d", what, elem);
+    if (flags & ~GLLMQ_OUT_ACCUMULATE) return fail(ctx, GLLMQ_ERR_INVALID, "%s: unknown flag bits 0x%x", what, flags);
+    st->x = static_cast<const float *>(x);
+    st->result = static_cast<float *>(out);
+    st->finish = elem != GLLMQ_ELEM_F32 || (flags & GLLMQ_OUT_ACCUMULATE);
+    if (!st->finish || count == 0) return GLLMQ_OK;
+    if (!x || !out) return fail(ctx, GLLMQ_ERR_INVALID, "%s: NULL device pointer", what);
+    if (!aligned(x, 2) || !aligned(out, 2)) return fail(ctx, GLLMQ_ERR_BAD_ALIGNMENT, "%s: x and out must be aligned to their element", what);
+    Scratch *S = nullptr;
+    int rc = acquire_scratch(ctx, stream, &S);
+    if (rc != GLLMQ_OK) return rc;
+    const size_t each = (count * 4 + 255) & ~size_t(255);
+    rc = grow_scratch(ctx, *S, &S->elem, &S->elem_bytes, 2 * each, stream, what);
+    if (rc != GLLMQ_OK) return rc;
+    st->result = reinterpret_cast<float *>(static_cast<uint8_t *>(S->elem) + each);
+    if (elem != GLLMQ_ELEM_F32) {
+        float *xf = static_cast<float *>(S->elem);
+        rc = convert_elems(ctx, x, xf, count, static_cast<uint32_t>(elem), true, stream);
+        st->x = xf;
+    }
+    return rc;
+}
+
+int elem_stage_end(gllmq_ctx *ctx, const ElemStage &st, void *out, size_t count, int elem, int flags, void *stream)
+{
+    if (!st.finish || count == 0) return GLLMQ_OK;
+    gq::ConvertParams C{};
+    C.src = st.result;
+    C.dst = out;
+    C.count = count;
+    C.elem = static_cast<uint32_t>(elem);
+    C.accumulate = (flags & GLLMQ_OUT_ACCUMULATE) ? 1u : 0u;
+    const uint32_t grid = static_cast<uint32_t>(std::min<size_t>((count + 255) / 256, 4096));
+    return launch(ctx, ctx->finish_elem, std::max(1u, grid), 256, 0, stream, &C, sizeof C, true);
+}
+
+} // namespace
+
+int gllmq_ffn_swiglu_elem(gllmq_ctx *ctx, const void *gate_w, const void *up_w, size_t gate_up_bytes_each, uint32_t dtype_gate_up,
+                          const void *down_w, size_t down_bytes, uint32_t dtype_down, const void *x, void *out, size_t m,
+                          size_t hidden, size_t ffn, int relu_gate, int elem, int flags, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    ElemStage st;
+    int rc = elem_stage_begin(ctx, x, out, m * hidden, elem, flags, stream, "ffn_swiglu", &st);
+    if (rc != GLLMQ_OK) return rc;
+    rc = gllmq_ffn_swiglu(ctx, gate_w, up_w, gate_up_bytes_each, dtype_gate_up, down_w, down_bytes, dtype_down, st.x, st.result, m,
+                          hidden, ffn, relu_gate, stream);
+    if (rc != GLLMQ_OK) return rc;
+    return elem_stage_end(ctx, st, out, m * hidden, elem, flags, stream);
+}
+
+int gllmq_moe_matvec_elem(gllmq_ctx *ctx, const void *gate, size_t gate_bytes, size_t gate_expert_stride, const void *up,
+                          size_t up_bytes, size_t up_expert_stride, uint32_t dtype_gu, const void *down, size_t down_bytes,
+                          size_t down_expert_stride, uint32_t dtype_dn, const void *x, void *out, size_t tokens, size_t hidden,
+                          size_t ffn, size_t experts, size_t top_k, const uint32_t *route_expert, const float *route_weight,
+                          const uint32_t *route_len, int relu_gate, int elem, int flags, void *stream)
+{
+    if (!ctx) return GLLMQ_ERR_INVALID;
+    std::lock_guard<std::recursive_mutex> call(ctx->call_mutex);
+    ElemStage st;
+    int rc = elem_stage_begin(ctx, x, out, tokens * hidden, elem, flags, stream, "moe_matvec", &st);
+    if (rc != GLLMQ_OK) return rc;
+    rc = gllmq_moe_matvec(ctx, gate, gate_bytes, gate_expert_stride, up, up_bytes, up_expert_stride, dtype_gu, down, down_bytes,
+                          down_expert_stride, dtype_dn, st.x, st.result, tokens, hidden, ffn, experts, top_k, route_expert,
+                          route_weight, route_len, relu_gate, stream);
+    if (rc != GLLMQ_OK) return rc;
+    return elem_stage_end(ctx, st, out, tokens * hidden, elem, flags, stream);
 }
 
 int gllmq_quantized_matmul(gllmq_ctx *ctx, const void *w, size_t w_bytes, const float *x, float *y,

@@ -390,6 +390,7 @@ struct GatherParams {
     uint32_t quads_per_row; // hidden / 4
     uint32_t count;
     float scale;            // 1.0f when the lookup is not scaled
+    uint32_t elem;          // the 16-bit kernels: element type of out (ELEM_F16 / ELEM_BF16)
 };
 
 struct GluActParams {
@@ -403,8 +404,9 @@ struct ConvertParams {
     const void *src;
     void *dst;
     uint64_t count;  // elements
-    uint32_t elem;   // the 16-bit type (ELEM_F16 / ELEM_BF16)
+    uint32_t elem;   // the 16-bit type (ELEM_F16 / ELEM_BF16); gq_finish_elem: any element type
     uint32_t widen;  // 1: 16-bit -> f32, 0: f32 -> 16-bit
+    uint32_t accumulate, pad; // gq_finish_elem: dst = round(dst + src) instead of round(src)
 };
 
 struct ArgmaxParams {

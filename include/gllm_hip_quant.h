@@ -143,6 +143,14 @@ int gllmq_quant_gather(gllmq_ctx *ctx, const void *table_dev, size_t table_bytes
                        size_t vocab, size_t hidden, const uint32_t *ids_dev, size_t count, float scale,
                        float *out_dev, void *stream);
 
+/* The same with rows of another element type on the way out (Backend<E>, src/compat/mod.rs:376-378:
+ * the lookup is the graph's first op and feeds activations of the model's element type): out_dev
+ * holds `elem` (GLLMQ_ELEM_F32 / _F16 / _BF16) elements, each the f32 value of gllmq_quant_gather
+ * rounded to nearest, ties to even; 16-bit rows are written by the lookup's own stores. */
+int gllmq_quant_gather_elem(gllmq_ctx *ctx, const void *table_dev, size_t table_bytes, uint32_t ggml_dtype,
+                            size_t vocab, size_t hidden, const uint32_t *ids_dev, size_t count, float scale,
+                            void *out_dev, int elem, void *stream);
+
 /* ---- Dense feed-forward block: gate/up projections, SwiGLU, down projection -------------
  * Replaces the op sequence the reference emits per layer (QuantGemm gate_proj, QuantGemm
  * up_proj, Op::SwiGlu, QuantGemm down_proj: src/arch/auto_graph_fragments/
@@ -159,6 +167,20 @@ int gllmq_ffn_swiglu(gllmq_ctx *ctx, const void *gate_dev, const void *up_dev, s
                      uint32_t dtype_gate_up, const void *down_dev, size_t down_bytes, uint32_t dtype_down,
                      const float *x_dev, float *out_dev, size_t m, size_t hidden, size_t ffn, int relu_gate,
                      void *stream);
+
+/* The same over activations and outputs of element type `elem` (Backend<E>, src/compat/mod.rs:376-378),
+ * and, with GLLMQ_OUT_ACCUMULATE in `flags`, added to what out_dev holds instead of replacing it:
+ * the Op::Add that puts a shared expert's feed-forward block on top of the routed experts' sum, and
+ * the residual add behind the block (build_graph.inc.rs:2132-2170).  16-bit activations widen
+ * exactly; the block runs in f32 as gllmq_ffn_swiglu does; out = round(result) or
+ * out = round(widen(out) + result), one rounding to nearest, ties to even (f32: none beyond the
+ * addition's).  Bit for bit: the result of gllmq_ffn_swiglu on the widened activations, added and
+ * rounded.  The conversions are small launches of their own around the block's kernels. */
+#define GLLMQ_OUT_ACCUMULATE 1
+int gllmq_ffn_swiglu_elem(gllmq_ctx *ctx, const void *gate_dev, const void *up_dev, size_t gate_up_bytes_each,
+                          uint32_t dtype_gate_up, const void *down_dev, size_t down_bytes, uint32_t dtype_down,
+                          const void *x_dev, void *out_dev, size_t m, size_t hidden, size_t ffn, int relu_gate,
+                          int elem, int flags, void *stream);
 
 /* ---- Op::Argmax: greedy token choice behind the lm_head matmul -----------------------
  * Replaces the graph op of src/arch/auto_graph_fragments/build_graph.inc.rs:2661 with the
@@ -344,6 +366,15 @@ int gllmq_moe_matvec(gllmq_ctx *ctx, const void *gate_dev, size_t gate_bytes, si
                      const float *x_dev, float *out_dev, size_t tokens, size_t hidden, size_t ffn, size_t experts,
                      size_t top_k, const uint32_t *route_expert_dev, const float *route_weight_dev,
                      const uint32_t *route_len_dev, int relu_gate, void *stream);
+
+/* gllmq_moe_matvec over activations and outputs of element type `elem`, and with
+ * GLLMQ_OUT_ACCUMULATE added to out_dev (see gllmq_ffn_swiglu_elem: same rules, same rounding). */
+int gllmq_moe_matvec_elem(gllmq_ctx *ctx, const void *gate_dev, size_t gate_bytes, size_t gate_expert_stride,
+                          const void *up_dev, size_t up_bytes, size_t up_expert_stride, uint32_t dtype_gate_up,
+                          const void *down_dev, size_t down_bytes, size_t down_expert_stride, uint32_t dtype_down,
+                          const void *x_dev, void *out_dev, size_t tokens, size_t hidden, size_t ffn, size_t experts,
+                          size_t top_k, const uint32_t *route_expert_dev, const float *route_weight_dev,
+                          const uint32_t *route_len_dev, int relu_gate, int elem, int flags, void *stream);
 
 /* ---- GGUF reader and tensor upload ---------------------------------------------------
  * The file side of the path: what the reference's loader accepts and rejects

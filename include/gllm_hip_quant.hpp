@@ -134,6 +134,18 @@ public:
                     "quant_gather");
     }
 
+    // Op::QuantGather into rows of element type `elem` (GLLMQ_ELEM_*): the f32 lookup's values,
+    // rounded to nearest even by the lookup's own stores.
+    BackendError quant_gather_elem_device(const void *table_dev, size_t table_bytes, QuantType quant_type,
+                                          size_t vocab_size, size_t hidden_dim, const uint32_t *token_ids_dev, size_t count,
+                                          const float *scale, void *out_dev, int elem, void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_quant_gather_elem(ctx_, table_dev, table_bytes, static_cast<uint32_t>(quant_type), vocab_size,
+                                            hidden_dim, token_ids_dev, count, scale ? *scale : 1.0f, out_dev, elem, stream),
+                    "quant_gather");
+    }
+
     // Dense feed-forward block over device buffers: gate_proj, up_proj, Op::SwiGlu, down_proj
     // (src/arch/auto_graph_fragments/build_graph.inc.rs:1957-1995).
     BackendError ffn_swiglu_device(const void *gate_dev, const void *up_dev, size_t gate_up_bytes_each, QuantType t_gate_up,
@@ -145,6 +157,21 @@ public:
         return make(gllmq_ffn_swiglu(ctx_, gate_dev, up_dev, gate_up_bytes_each, static_cast<uint32_t>(t_gate_up), down_dev,
                                      down_bytes, static_cast<uint32_t>(t_down), x_dev, out_dev, m, hidden, ffn,
                                      relu_gate ? 1 : 0, stream),
+                    "ffn_swiglu");
+    }
+
+    // The same for E = f32 / f16 / bf16 activations and outputs (`elem`: GLLMQ_ELEM_*), replacing
+    // out_dev or, with accumulate, added to it (Op::Add of a shared expert's block and the
+    // residual, build_graph.inc.rs:2132-2170); one rounding to nearest even.
+    BackendError ffn_swiglu_elem_device(const void *gate_dev, const void *up_dev, size_t gate_up_bytes_each,
+                                        QuantType t_gate_up, const void *down_dev, size_t down_bytes, QuantType t_down,
+                                        const void *x_dev, void *out_dev, size_t m, size_t hidden, size_t ffn, int elem,
+                                        bool accumulate = false, bool relu_gate = false, void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_ffn_swiglu_elem(ctx_, gate_dev, up_dev, gate_up_bytes_each, static_cast<uint32_t>(t_gate_up),
+                                          down_dev, down_bytes, static_cast<uint32_t>(t_down), x_dev, out_dev, m, hidden, ffn,
+                                          relu_gate ? 1 : 0, elem, accumulate ? GLLMQ_OUT_ACCUMULATE : 0, stream),
                     "ffn_swiglu");
     }
 
@@ -214,6 +241,26 @@ public:
                                      route_expert_dev, route_weight_dev, route_len_dev, relu_gate ? 1 : 0, stream),
                     "moe_matvec");
     }
+
+    // The same for E = f32 / f16 / bf16 activations and outputs, replacing out_dev or added to it.
+    BackendError moe_matvec_elem_device(ExpertWeights gate, ExpertWeights up, QuantType t_gate_up, ExpertWeights down,
+                                        QuantType t_down, const void *x_dev, void *out_dev, size_t tokens, size_t hidden,
+                                        size_t ffn, size_t experts, size_t top_k, const uint32_t *route_expert_dev,
+                                        const float *route_weight_dev, const uint32_t *route_len_dev, int elem,
+                                        bool accumulate = false, bool relu_gate = false, void *stream = nullptr) const
+    {
+        if (!ctx_) return init_error_;
+        return make(gllmq_moe_matvec_elem(ctx_, gate.dev, gate.bytes, gate.expert_stride, up.dev, up.bytes, up.expert_stride,
+                                          static_cast<uint32_t>(t_gate_up), down.dev, down.bytes, down.expert_stride,
+                                          static_cast<uint32_t>(t_down), x_dev, out_dev, tokens, hidden, ffn, experts, top_k,
+                                          route_expert_dev, route_weight_dev, route_len_dev, relu_gate ? 1 : 0, elem,
+                                          accumulate ? GLLMQ_OUT_ACCUMULATE : 0, stream),
+                    "moe_matvec");
+    }
+
+    // 1 if a chained launch since the last look ran out of its bounded wait (option
+    // "chain_dependent"), 0 if none did; call after waiting for the stream.
+    int chain_status() const { return ctx_ ? gllmq_chain_status(ctx_) : 0; }
 
     gllmq_ctx *raw() const { return ctx_; }
 

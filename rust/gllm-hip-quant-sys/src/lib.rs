@@ -55,6 +55,20 @@ extern "C" {
     pub fn gllmq_quantized_matmul_batch(ctx: *mut gllmq_ctx, descs: *const gllmq_matmul_desc, count: usize,
                                         stream: *mut c_void) -> c_int;
     pub fn gllmq_chain_status(ctx: *mut gllmq_ctx) -> c_int;
+    pub fn gllmq_quant_gather_elem(ctx: *mut gllmq_ctx, table_dev: *const c_void, table_bytes: usize, ggml_dtype: u32,
+                                   vocab: usize, hidden: usize, ids_dev: *const u32, count: usize, scale: f32,
+                                   out_dev: *mut c_void, elem: c_int, stream: *mut c_void) -> c_int;
+    pub fn gllmq_ffn_swiglu_elem(ctx: *mut gllmq_ctx, gate_dev: *const c_void, up_dev: *const c_void,
+                                 gate_up_bytes_each: usize, dtype_gate_up: u32, down_dev: *const c_void, down_bytes: usize,
+                                 dtype_down: u32, x_dev: *const c_void, out_dev: *mut c_void, m: usize, hidden: usize,
+                                 ffn: usize, relu_gate: c_int, elem: c_int, flags: c_int, stream: *mut c_void) -> c_int;
+    pub fn gllmq_moe_matvec_elem(ctx: *mut gllmq_ctx, gate_dev: *const c_void, gate_bytes: usize, gate_expert_stride: usize,
+                                 up_dev: *const c_void, up_bytes: usize, up_expert_stride: usize, dtype_gate_up: u32,
+                                 down_dev: *const c_void, down_bytes: usize, down_expert_stride: usize, dtype_down: u32,
+                                 x_dev: *const c_void, out_dev: *mut c_void, tokens: usize, hidden: usize, ffn: usize,
+                                 experts: usize, top_k: usize, route_expert_dev: *const u32, route_weight_dev: *const f32,
+                                 route_len_dev: *const u32, relu_gate: c_int, elem: c_int, flags: c_int,
+                                 stream: *mut c_void) -> c_int;
     pub fn gllmq_moe_route(ctx: *mut gllmq_ctx, logits_dev: *const f32, tokens: usize, experts: usize, top_k: usize,
                            capacity_factor: f32, route_expert_dev: *mut u32, route_weight_dev: *mut f32,
                            route_len_dev: *mut u32, route_pos_dev: *mut u32, expert_counts_dev: *mut u32,
