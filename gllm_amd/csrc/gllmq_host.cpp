@@ -209,7 +209,7 @@ struct gllmq_ctx {
     hipFunction_t mmfr[2] = {};                 // the streamed form whose waves prepare their own activations (f32, 9 to 16 rows) [0 = Q4_K, 1 = Q5_K]
     bool use_mmfr = true;                       // "mmfr" = 0: never
     uint32_t mmfr_min_rows = 8;                 // "mmfr_min_rows": fewest weight rows per CU that take it
-    hipFunction_t mm8c[3][2] = {};              // chains of streamed matmuls in one launch [0 = Q4_K, 1 = Q5_K, 2 = Q8_0][some entry in pairs of blocks]
+    hipFunction_t mm8c[3][2][2] = {};           // chains of streamed matmuls in one launch [0 = Q4_K, 1 = Q5_K, 2 = Q8_0][some entry in pairs of blocks][some entry waits for the one before it]
     bool chain_dependent = false;               // "chain_dependent" = 1: an entry that reads the output of the one before it stays in the chained launch (measured slower than a launch of its own)
     uint32_t chain_epoch = 1;                   // epochs handed to chained entries so far (see Mm8ChainParams::box)
     bool use_chain = true;                      // "chain" = 0: every entry of a batch is a launch of its own
@@ -1322,7 +1322,7 @@ int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t
         ctx->chain_epoch += static_cast<uint32_t>(len);
     }
     P.launched = launched;
-    return launch(ctx, ctx->mm8c[fmt][folds ? 1 : 0], launched, (gq::MM8C_CWAVES + gq::MM8C_LOADERS) * 64, P.lds_ring + slots * P.slot_bytes,
+    return launch(ctx, ctx->mm8c[fmt][folds ? 1 : 0][waits ? 1 : 0], launched, (gq::MM8C_CWAVES + gq::MM8C_LOADERS) * 64, P.lds_ring + slots * P.slot_bytes,
                   stream, &P, sizeof P, true);
 }
 
@@ -1512,8 +1512,12 @@ int gllmq_init(gllmq_ctx **out, int device)
                 rc = get_function(ctx, &ctx->mmf_q4k[q][t][b], name);
             }
     static const char *const kMm8c[3][2] = { { "gq_mm8c_q4k", "gq_mm8c_q4k_f" }, { "gq_mm8c_q5k", "gq_mm8c_q5k_f" }, { "gq_mm8c_q8_0", "gq_mm8c_q8_0_f" } };
-    for (int q = 0; q < 3; ++q)
-        for (int v = 0; v < 2 && rc == GLLMQ_OK; ++v) rc = get_function(ctx, &ctx->mm8c[q][v], kMm8c[q][v]);
+    for (int q = 0; q < 3 && rc == GLLMQ_OK; ++q)
+        for (int v = 0; v < 2 && rc == GLLMQ_OK; ++v)
+            for (int d = 0; d < 2 && rc == GLLMQ_OK; ++d) {
+                snprintf(name, sizeof name, "%s%s", kMm8c[q][v], d ? "_d" : "");
+                rc = get_function(ctx, &ctx->mm8c[q][v][d], name);
+            }
     for (int q = 0; q < 2 && rc == GLLMQ_OK; ++q)
         for (int b = 0; b < 2 && rc == GLLMQ_OK; ++b) {
             snprintf(name, sizeof name, "gq_mmfs_%s%s", q ? "q5k" : "q4k", b ? "_bf16" : "");
@@ -1638,7 +1642,7 @@ int gllmq_init(gllmq_ctx **out, int device)
         for (auto &q : ctx->mm8s_glu) for (hipFunction_t f : q) add(f);
         for (auto &q : ctx->mm8s_fold) for (hipFunction_t f : q) add(f);
         for (auto &q : ctx->mm8s_split) for (auto &r : q) for (hipFunction_t f : r) add(f);
-        for (auto &q : ctx->mm8c) for (hipFunction_t f : q) add(f);
+        for (auto &q : ctx->mm8c) for (auto &v : q) for (hipFunction_t f : v) add(f);
     }
     // the scratch array of the entry point that allocates nothing: found (and thereby placed on
     // this device) now, while allocating is allowed

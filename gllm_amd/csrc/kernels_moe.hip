@@ -13,6 +13,7 @@
 #include "gemv_i8.hip.inc"
 #include "mm8.hip.inc"
 #include "mm8_q6k.hip.inc"
+#define GQ_Q6K_STEPWISE AREG // (115 -> 166 registers of 168, no scratch; the Q6_K down launch of 128 experts 93.1 -> 91.4 us)
 #include "mm8s.hip.inc"
 #undef GQ_TEMPLATES_ONLY
 
