@@ -176,6 +176,7 @@ struct gllmq_ctx {
     // gated form of the int8 kernels (gate and up rows in one launch, act(gate) * up out):
     // [0 = Q4_K, 1 = Q5_K][pairs 1,2,4][early steps 1,2,4] and the register-operand variants
     hipFunction_t mm8_glu[2][3][3] = {};
+    hipFunction_t mm8_gated_p4[MM8_KINDS] = {}; // five to eight rows of gated activations (a down projection's), by Mm8Kind
     hipFunction_t mm8_glu_areg[2][2][3][2] = {};
     hipFunction_t glu_act = nullptr;            // act(gate) * up as a kernel of its own
     hipFunction_t argmax_part = nullptr, argmax_final = nullptr;
@@ -278,7 +279,7 @@ struct gllmq_ctx {
     hipFunction_t mm8s_gated[2][6] = {};        // streamed gate/up kernels with act(g) * u at the end of a tile pair [Q4_K, Q5_K][p1_e1_a, p1_e2_a, p2_e4_a, p1_e2, p2_e4, p1_e4]
     bool ffn_streamed = true;                   // "ffn_streamed" = 0: gllmq_ffn_swiglu never uses them
     hipFunction_t mm8s_e16[4][6] = {};          // streamed kernels over 16-bit activations and outputs [format][p1_e1_a, p1_e2_a, p2_e4_a, p1_e2, p2_e4, p1_e4]
-    hipFunction_t mm8s_glu[4][3] = {};          // streamed kernels that take gated activations [format][p1_e2, p2_e4, p1_e4]
+    hipFunction_t mm8s_glu[4][4] = {};          // streamed kernels that take gated activations [format][p1_e2, p2_e4, p1_e4, p4_e4]
     // streamed kernels whose items are pairs of blocks of a tile of at most 16 weight rows (one
     // activation row) [format][p1_e1_a, p1_e2_a, p1_e2, p1_e4, p1_e2 and p1_e4 over gated activations,
     // the first four over a 16-bit element type]
@@ -753,7 +754,7 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
         if (gv < 0) return -1;
         fn = ctx->mm8s_gated[sfmt][gv];
     } else if (ctx->call_glu) {
-        const int gv = variant == 3 ? 0 : variant == 4 ? 1 : variant == 6 ? 2 : -1;
+        const int gv = variant == 3 ? 0 : variant == 4 ? 1 : variant == 6 ? 2 : variant == 5 ? 3 : -1; // (the rest keep their planes in registers: rows of at most 4096 elements, not a down projection's)
         if (gv < 0 || !glu_vector_ok(ctx)) return kNeedPlainActivations;
         fn = ctx->mm8s_glu[sfmt][gv];
     } else if (ctx->call_elem) {
@@ -877,7 +878,12 @@ int run_mm8(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         --rows_per_pass;
     if (rows_per_pass == 0) return -1;
     if (one_pass_only && rows_per_pass < m) return -1;
-    if (ctx->call_glu || ctx->call_elem) return kNeedPlainActivations; // these kernels read and write f32
+    if (ctx->call_elem) return kNeedPlainActivations; // these kernels read and write f32
+    // gated activations (a feed-forward block's down projection): passes of five to eight rows have a kernel for them
+    if (ctx->call_glu) {
+        const size_t last_pass = m - ((m - 1) / rows_per_pass) * rows_per_pass;
+        if (glu || rows_per_pass < 5 || last_pass < 5 || !glu_vector_ok(ctx) || !ctx->mm8_gated_p4[kind]) return kNeedPlainActivations;
+    }
     for (size_t m0 = 0; m0 < m; m0 += rows_per_pass) {
         const uint32_t mm = static_cast<uint32_t>(std::min<size_t>(rows_per_pass, m - m0));
         const int pi = mm <= 2 ? 0 : (mm <= 4 ? 1 : 2);
@@ -890,15 +896,17 @@ int run_mm8(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         P.arrive = S.mm8_arrive;
         P.w2 = w2;
         P.glu_relu = glu_relu ? 1u : 0u;
+        P.glu = ctx->call_glu;
+        P.glu_off = ctx->call_glu_off;
         P.w = w;
-        P.x = x + m0 * k;
+        P.x = x + m0 * row_stride_x(ctx, k);
         P.y = y + m0 * n;
         P.n = static_cast<uint32_t>(n);
         P.k = static_cast<uint32_t>(k);
         P.groups = groups;
         P.row_bytes = static_cast<uint32_t>(gllmq_row_bytes(f.dtype, k));
         P.m = mm;
-        P.ldx = static_cast<uint32_t>(k);
+        P.ldx = row_stride_x(ctx, k);
         P.ldy = static_cast<uint32_t>(n);
         P.tiles = (P.n + 31u) / 32u;
         P.act_bf16 = act_bf16 ? 1u : 0u;
@@ -918,6 +926,7 @@ int run_mm8(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *w, const
         const bool even_slices = ksplit == 1 || ppt_row % slice_passes == 0;
         if (pi <= 1 && ppt <= 2 && even_slices)
             fn = glu ? ctx->mm8_glu_areg[gi][pi][ei][ppt - 1] : ctx->mm8_areg[kind][pi][ei][ppt - 1];
+        if (ctx->call_glu) fn = ctx->mm8_gated_p4[kind]; // (pi == 2: checked above)
         int rc = launch(ctx, fn, grid * ksplit, 512, lds, stream, &P, sizeof P, ksplit > 1);
         if (rc != GLLMQ_OK) return rc;
     }
@@ -1585,6 +1594,10 @@ int gllmq_init(gllmq_ctx **out, int device)
                     snprintf(name, sizeof name, "gq_mm8_%s_%s_a%d", kMm8Format[q], k.tag, a);
                     rc = get_function(ctx, &ctx->mm8_areg[q][k.pi][k.ei][a - 1], name);
                 }
+                if (k.pi == 2) {
+                    snprintf(name, sizeof name, "gq_mm8_%s_%s_g", kMm8Format[q], k.tag);
+                    if (rc == GLLMQ_OK) rc = get_function(ctx, &ctx->mm8_gated_p4[q], name);
+                }
                 if (q != MM8_Q4K && q != MM8_Q5K) continue;
                 const int gi = q == MM8_Q5K ? 1 : 0;
                 snprintf(name, sizeof name, "gq_mm8_glu_%s_%s", kMm8Format[q], k.tag);
@@ -1626,9 +1639,9 @@ int gllmq_init(gllmq_ctx **out, int device)
                 snprintf(name, sizeof name, "gq_mm8s_%s_p%d_e4%s_s", kMm8sFormat[q], 1 + (v & 1), (v & 2) ? "_g" : "");
                 rc = get_function(ctx, &ctx->mm8s_split[q][v & 1][v >> 1], name);
             }
-        static const char *const kMm8sGlu[3] = { "p1_e2_g", "p2_e4_g", "p1_e4_g" };
+        static const char *const kMm8sGlu[4] = { "p1_e2_g", "p2_e4_g", "p1_e4_g", "p4_e4_g" };
         for (int q = 0; q < 4; ++q)
-            for (int v = 0; v < 3 && rc == GLLMQ_OK; ++v) {
+            for (int v = 0; v < 4 && rc == GLLMQ_OK; ++v) {
                 snprintf(name, sizeof name, "gq_mm8s_%s_%s", kMm8sFormat[q], kMm8sGlu[v]);
                 rc = get_function(ctx, &ctx->mm8s_glu[q][v], name);
             }

@@ -122,6 +122,11 @@ def test_ffn_three_step_form(torch, oracle):
     (Q4_K, Q5_K, 2048, 5120, (16, 40)),        # GEMM: the preparation launch of the down projection applies the gate
     (Q6_K, Q6_K, 512, 776, (1, 9)),            # ragged ffn
     (Q8_0, Q8_0, 256, 200, (1, 2, 70)),        # ffn not a multiple of 64: the GEMV's scalar loads
+    (Q6_K, Q6_K, 2048, 4096, (5, 8)),          # five to eight rows: kernels of four row pairs that read the gated product
+    (Q4_K, Q8_0, 2048, 4352, (6, 7)),
+    (Q5_K, Q4_K, 4096, 3072, (5, 8)),
+    (Q4_K, Q5_K, 1024, 2560, (7,)),
+    (Q4_K, Q6_K, 4096, 14336, (6,)),           # rows of 14336 elements: a K split, or passes of fewer rows than the call has
 ])
 def test_down_projection_reads_the_gated_product(torch, oracle, t_gu, t_dn, hidden, ffn, ms):
     """Where the gate/up products are not gated in their kernel's epilogue, the down projection's
@@ -141,6 +146,8 @@ def test_down_projection_reads_the_gated_product(torch, oracle, t_gu, t_dn, hidd
             x = random_activations(m, hidden, seed=m)
             got = run_ffn(fused, torch, gate, up, t_gu, down, t_dn, x, m, hidden, ffn, relu=relu, stacked=stacked)
             ref = run_ffn(plain, torch, gate, up, t_gu, down, t_dn, x, m, hidden, ffn, relu=relu, stacked=stacked)
+            if 5 <= m <= 8:  # (the streamed kernel of four row pairs, or the fetch-and-compute one, with gated loads)
+                assert fused.last_kernel_name().endswith("_p4_e4_g"), fused.last_kernel_name()
             assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), "differs from the activation as its own launch"
             want = oracle.ffn_swiglu(gate, up, t_gu, down, t_dn, x, m, hidden, ffn, relu_gate=relu, acc=oracle.ACC_F64, threads=8)
             check(got, want, f"gated loads m={m}")
