@@ -441,7 +441,7 @@ int acquire_scratch(gllmq_ctx *ctx, void *stream, Scratch **out)
 // stream is being captured, and never happens for a set of fixed size.
 int grow_scratch(gllmq_ctx *ctx, const Scratch &S, void **buf, size_t *have, size_t need, void *stream, const char *what)
 {
-    if (*have >= need) return GLLMQ_OK;
+    if (*have >= need || ctx->probe) return GLLMQ_OK; // (a dry run of the dispatch allocates nothing)
     if (S.fixed)
         return fail(ctx, GLLMQ_ERR_BAD_SHAPE, "%s needs %zu bytes of scratch, the fixed scratch of this entry point has %zu",
                     what, need, *have);
@@ -1384,6 +1384,28 @@ int dispatch_matmul(gllmq_ctx *ctx, Scratch &S, const Format &f, const uint8_t *
 size_t ffn_h_bytes(size_t m, size_t ffn) { return ((m * ffn * sizeof(float)) + 255) & ~size_t(255); }
 size_t ffn_scratch_bytes(size_t m, size_t ffn) { return ffn_h_bytes(m, ffn) + m * 2 * ffn * sizeof(float); }
 
+// Which kernel the dispatch gives a matmul: the dispatch itself, run with launches and allocations
+// switched off (ctx->probe), so that the answer cannot drift from what a call does.  `fn` is the
+// kernel when the call is exactly one launch, else null; `launches` counts them.
+struct DispatchChoice {
+    hipFunction_t fn = nullptr;
+    uint32_t launches = 0;
+};
+
+template <class Call>
+DispatchChoice dispatch_choice(gllmq_ctx *ctx, Call &&call)
+{
+    ctx->probe = true;
+    ctx->probe_launches = 0;
+    ctx->probe_fn = nullptr;
+    const int rc = call();
+    ctx->probe = false;
+    DispatchChoice c;
+    c.launches = rc == GLLMQ_OK ? ctx->probe_launches : 0u;
+    c.fn = c.launches == 1u ? ctx->probe_fn : nullptr;
+    return c;
+}
+
 // One validated quantized matmul with the scratch of `S` (call_mutex held).
 int matmul_on_scratch(gllmq_ctx *ctx, Scratch &S, const void *w, size_t w_bytes, const float *x, float *y, uint32_t dtype,
                       size_t m, size_t n, size_t k, int act_mode, void *stream)
@@ -1889,18 +1911,16 @@ int gllmq_lm_head_argmax(gllmq_ctx *ctx, const void *w, size_t w_bytes, const fl
     // The matvec whose workgroups leave their best candidate behind: the one-row GEMV of Q6_K and
     // Q8_0 (the types of GGUF output matrices) where one launch covers K; the workgroup that
     // finishes last picks among the candidates.  With a logits buffer it runs where the GEMV is
-    // the kernel gllmq_quantized_matmul gives the shape anyway (asked by a dry run of the
-    // dispatch), so that the logits are that call's bit for bit; without one, always.
+    // the kernel gllmq_quantized_matmul gives the shape anyway (dispatch_choice() asks the dispatch
+    // itself), so that the logits are that call's bit for bit; without one, always.
     const size_t rb = gllmq_row_bytes(dtype, k);
     const bool gemv_type = dtype == 14u || dtype == 8u;
     bool gemv_anyway = true;
     if (ctx->lm_head_fused && gemv_type && !ctx->gemv_f32 && k <= 16384 && logits) {
-        ctx->probe = true;
-        ctx->probe_launches = 0;
-        ctx->probe_fn = nullptr;
-        const int prc = dispatch_matmul(ctx, *S, *f, static_cast<const uint8_t *>(w), x, logits, 1, n, k, false, stream);
-        ctx->probe = false;
-        gemv_anyway = prc == GLLMQ_OK && ctx->probe_launches == 1 && ctx->probe_fn == ctx->gemv_i8[format_index(dtype)][0];
+        const DispatchChoice c = dispatch_choice(ctx, [&] {
+            return dispatch_matmul(ctx, *S, *f, static_cast<const uint8_t *>(w), x, logits, 1, n, k, false, stream);
+        });
+        gemv_anyway = c.fn != nullptr && c.fn == ctx->gemv_i8[format_index(dtype)][0];
     }
     if (ctx->lm_head_fused && gemv_type && !ctx->gemv_f32 && k <= 16384 && gemv_anyway) {
         GemvPlan L = plan_gemv(ctx, 1, static_cast<uint32_t>(n), static_cast<uint32_t>(k), rb, ctx->gemv_waves);
@@ -2234,12 +2254,8 @@ void plan_prefetch(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, s
             u.announces = true;
         } else if (!(descs[i].flags & ~kKnown)) {
             u.ordered = (descs[i].flags & GLLMQ_DESC_AFTER_PREVIOUS) != 0 || i == 0 || !ctx->batch_overlap;
-            ctx->probe = true;
-            ctx->probe_launches = 0;
-            ctx->probe_fn = nullptr;
-            const int rc = batch_entry(ctx, S, descs[i], stream);
-            ctx->probe = false;
-            u.announces = rc == GLLMQ_OK && ctx->probe_launches == 1 && ctx->announces.count(ctx->probe_fn) != 0;
+            const DispatchChoice c = dispatch_choice(ctx, [&] { return batch_entry(ctx, S, descs[i], stream); });
+            u.announces = c.fn != nullptr && ctx->announces.count(c.fn) != 0;
         }
         u.seq = ++ctx->launch_seq;
         units.push_back(u);

@@ -81,27 +81,36 @@ const char *gllmq_last_error(const gllmq_ctx *ctx);
 const char *gllmq_status_string(int status);
 const char *gllmq_version(void);
 
-/* Kernel-family choices of a context; no counterpart in the reference.  The defaults are the
- * measured best and nothing needs setting; the test-suite uses this to reach every kernel family
- * through the public entry points.  Names: "gemv_f32" (1: f32 multiply-add GEMV instead of the
- * integer-dot one), "mm8" / "mmf" (0: no int8 / f16 matrix-core kernels), "mm8s" (0: no loader-wave form of the
- * int8 kernels), "mm8s_min_rows" (fewest weight rows per CU that take it), "mm8s_all" (1: that form wherever the
- * shape fits it, also where another kernel was timed faster), "mm8s_depth" (items a loader wave
- * keeps in flight; 0: by item size), "mmfs" / "mmfs_all" / "mmfs_min_rows" (the same three for the loader-wave
- * form of the f16 GEMM), "mmfr" / "mmfr_min_rows" (0: no one-launch GEMM for 9 to 16 rows of f32 activations, whose
- * waves prepare their own operands; fewest weight rows per CU that take it), "chain" (0: every entry of a batch is a launch of its own), "chain_dependent" (1: an entry
- * whose activations are the output of the entry before it stays inside a chained launch and takes them from a mailbox
- * in device memory as they are stored), "chain_spin_limit" (looks at that mailbox before a wave gives up and the next
- * batch call reports it), "prefetch" (1: a launch on a stream of the context's own pulls the weights of each
- * dependent launch of a batch into the memory-side cache while the launch before it runs; measured slower), "batch_overlap" (0: the kernels of a
- * batch run strictly one after the other), "ffn_fused" (0: the
- * feed-forward block in three steps), "mm8_q5k_min_m" / "mm8_q6k_min_m" / "mm8_q8_0_min_m"
- * (fewest rows that take the int8 matrix-core kernel; 0 = never), "mmf_small_min_m" (fewest rows
- * of long rows that take the GEMM; 0 = never), "mm8_ksplit" (most K slices; 0 = never split),
- * "moe_mm8" / "moe_mm8_q6k" / "moe_mm8_rows" / "moe_glu" (0: expert rows off the matrix cores /
- * Q6_K ones / no wave-per-tile kernel / activation as its own launch), "weights_cache_mib" (bytes
- * of uploaded weights the host-slice calls keep, in MiB).  Unknown names return
- * GLLMQ_ERR_INVALID.  Not to be changed while calls are in flight on other threads. */
+/* Options of a context; no counterpart in the reference.  Nothing needs setting: the defaults are
+ * the measured best.  Unknown names return GLLMQ_ERR_INVALID.  Not to be changed while calls are in
+ * flight on other threads.
+ *
+ * Supported (kept stable):
+ *   "weights_cache_mib"  MiB of uploaded weights the host-slice calls keep (default 65536)
+ *   "chain"              0: every entry of a batch is a launch of its own (default 1)
+ *   "batch_overlap"      0: the kernels of a batch run strictly one after the other (default 1)
+ *   "ffn_fused"          0: the feed-forward block as separate products (default 1)
+ *   "chain_dependent"    1: an entry whose activations are the output of the entry before it stays
+ *                        inside a chained launch and takes them from a mailbox in device memory as
+ *                        they are stored (default 0: measured slower than a launch each, 9.0
+ *                        against 8.5 us per 33 MB entry); "chain_spin_limit": looks at that mailbox
+ *                        before a wave gives up (see gllmq_chain_status)
+ *   "prefetch"           1: a launch on a stream of the context's own pulls the weights of each
+ *                        dependent launch of a batch into the memory-side cache while the launch
+ *                        before it runs (default 0: measured slower, 12.3 against 8.5 us)
+ *
+ * Development switches (UNSTABLE: they exist so that the test-suite and the measurements can reach
+ * every kernel family through the public entry points; names and meaning may change with any
+ * version, and a production caller should set none of them):
+ *   kernel families on/off: "gemv_f32", "mm8", "mmf", "mm8s", "mm8s_q8_0", "mmfs", "mmfr",
+ *     "moe_mm8", "moe_mm8_q6k", "moe_mm8_rows", "moe_glu", "moe_streamed", "lm_head_fused",
+ *     "elem_fused", "ffn_glu_load", "ffn_streamed", "mm8s_areg", "mm8s_fold", "mm8s_split",
+ *     "mm8_small_to_gemv"
+ *   shape thresholds: "mm8s_min_rows", "mmfs_min_rows", "mmfr_min_rows", "chain_min_rows",
+ *     "mm8_q5k_min_m", "mm8_q6k_min_m", "mm8_q8_0_min_m", "mmf_small_min_m", "mm8_ksplit",
+ *     "mm8s_all", "mmfs_all" (1: that form wherever the shape fits it, also where another was timed faster)
+ *   launch parameters: "mm8s_depth", "moe_depth", "moe_slices", "prefetch_wgs", "prefetch_threads",
+ *     "prefetch_timeout_us", "prefetch_flags", "prefetch_announce", "prefetch_min_kib" */
 int gllmq_set_option(gllmq_ctx *ctx, const char *name, long value);
 /* Name of the kernel the context launched last ("" before the first launch): lets a profile be
  * matched to a call.  No counterpart in the reference. */
