@@ -35,6 +35,9 @@ pub const GLLMQ_ERR_INVALID: c_int = 5;
 pub const GLLMQ_ACT_F32_SPLIT: c_int = 0;
 pub const GLLMQ_ACT_BF16: c_int = 1;
 
+/// `flags` of the `_elem` block entry points: add to the output instead of replacing it.
+pub const GLLMQ_OUT_ACCUMULATE: c_int = 1;
+
 extern "C" {
     pub fn gllmq_init(out_ctx: *mut *mut gllmq_ctx, device: c_int) -> c_int;
     pub fn gllmq_destroy(ctx: *mut gllmq_ctx);
@@ -304,6 +307,63 @@ impl HipQuant {
                                                stream: *mut c_void) -> Result<(), QuantError> {
         self.check(gllmq_quantized_matmul_elem(self.ctx, w, w_bytes, x, y, ggml_dtype, m, n, k, elem, stream),
                    "quantized_matmul")
+    }
+
+    /// `Op::QuantGather` into rows of element type `elem` (0 f32, 1 f16, 2 bf16): the f32 lookup's
+    /// values rounded to the nearest element, ties to even.  `scale`: `None` for none.
+    ///
+    /// # Safety
+    /// `table` must hold `table_bytes` bytes, `ids` `count` u32, `out` `count * hidden` elements of
+    /// the type, all on this device.
+    #[allow(clippy::too_many_arguments)]
+    pub unsafe fn quant_gather_elem_device(&self, table: *const c_void, table_bytes: usize, ggml_dtype: u32,
+                                           vocab_size: usize, hidden_dim: usize, ids: *const u32, count: usize,
+                                           scale: Option<f32>, out: *mut c_void, elem: c_int,
+                                           stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_quant_gather_elem(self.ctx, table, table_bytes, ggml_dtype, vocab_size, hidden_dim, ids, count,
+                                           scale.unwrap_or(1.0), out, elem, stream), "quant_gather")
+    }
+
+    /// The dense feed-forward block over activations and outputs of element type `elem`; with
+    /// `accumulate` it is added to `out` instead of replacing it (the `Op::Add` of a shared expert's
+    /// block and of the residual, build_graph.inc.rs:2132-2170), one rounding to nearest even.
+    ///
+    /// # Safety
+    /// As `ffn_swiglu_device`, with `x` and `out` holding `m * hidden` elements of the type.
+    #[allow(clippy::too_many_arguments)]
+    pub unsafe fn ffn_swiglu_elem_device(&self, gate: *const c_void, up: *const c_void, gate_up_bytes_each: usize,
+                                         dtype_gate_up: u32, down: *const c_void, down_bytes: usize, dtype_down: u32,
+                                         x: *const c_void, out: *mut c_void, m: usize, hidden: usize, ffn: usize,
+                                         elem: c_int, accumulate: bool, relu_gate: bool,
+                                         stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_ffn_swiglu_elem(self.ctx, gate, up, gate_up_bytes_each, dtype_gate_up, down, down_bytes,
+                                         dtype_down, x, out, m, hidden, ffn, relu_gate as c_int, elem,
+                                         if accumulate { GLLMQ_OUT_ACCUMULATE } else { 0 }, stream), "ffn_swiglu")
+    }
+
+    /// The routed experts' blocks over activations and outputs of element type `elem`, replacing
+    /// `out` or added to it.
+    ///
+    /// # Safety
+    /// As `moe_matvec_device`, with `x` and `out` holding `tokens * hidden` elements of the type.
+    #[allow(clippy::too_many_arguments)]
+    pub unsafe fn moe_matvec_elem_device(&self, gate: *const c_void, gate_bytes: usize, gate_stride: usize,
+                                         up: *const c_void, up_bytes: usize, up_stride: usize, dtype_gate_up: u32,
+                                         down: *const c_void, down_bytes: usize, down_stride: usize, dtype_down: u32,
+                                         x: *const c_void, out: *mut c_void, tokens: usize, hidden: usize, ffn: usize,
+                                         experts: usize, top_k: usize, route_expert: *const u32,
+                                         route_weight: *const f32, route_len: *const u32, elem: c_int, accumulate: bool,
+                                         relu_gate: bool, stream: *mut c_void) -> Result<(), QuantError> {
+        self.check(gllmq_moe_matvec_elem(self.ctx, gate, gate_bytes, gate_stride, up, up_bytes, up_stride, dtype_gate_up,
+                                         down, down_bytes, down_stride, dtype_down, x, out, tokens, hidden, ffn, experts,
+                                         top_k, route_expert, route_weight, route_len, relu_gate as c_int, elem,
+                                         if accumulate { GLLMQ_OUT_ACCUMULATE } else { 0 }, stream), "moe_matvec")
+    }
+
+    /// Whether a chained launch since the last look ran out of its bounded wait (option
+    /// "chain_dependent"); call after waiting for the stream.
+    pub fn chain_status(&self) -> bool {
+        unsafe { gllmq_chain_status(self.ctx) != 0 }
     }
 
     /// The lm_head matvec of one activation row and `Op::Argmax` behind it as one call.  `logits`

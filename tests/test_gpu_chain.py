@@ -272,3 +272,38 @@ def test_a_captured_batch_replays_like_the_eager_one(torch, oracle):
     x = x1.cpu().numpy()
     check_close(got[0].cpu().numpy(), oracle.quantized_matmul(random_weight(Q4_K, ns[0], k, seed=70), x, Q4_K, 1, ns[0], k,
                                                                acc=oracle.ACC_F64, threads=16), "entry 0 of the last replay")
+
+
+def test_the_weight_prefetch_beside_dependent_launches_changes_no_bit(torch):
+    """Option "prefetch": a launch on a stream of the context's own reads the weights of each
+    dependent entry into the memory-side cache while the entry before it runs (it waits for that
+    launch's announcement, bounded by a time-out, and writes nothing).  Same outputs bit for bit as
+    without it, over a sequence in which every matmul reads the output of the one before; large and
+    small matrices (entries under the size threshold are left out of the prefetch), twice, and
+    ordinary calls on the stream afterwards."""
+    from gllm_amd.backend import HipBackend
+    with_it, without = HipBackend(0, options={"prefetch": 1}), HipBackend(0)
+    k = 4096
+    ns = [4096, 4096, 14336]
+    ws = [random_weight(Q4_K, ns[0], k, seed=70), random_weight(Q4_K, ns[1], k, seed=71), random_weight(Q4_K, ns[2], k, seed=72)]
+    wd = [dev_weight(torch, w) for w in ws]
+    for attempt in range(2):
+        x0 = (random_activations(1, k, seed=80 + attempt) * 0.5).astype(np.float32)
+        outs = []
+        for backend in (with_it, without):
+            bufs = [torch.from_numpy(x0).cuda(), torch.full((1, ns[0]), float("nan"), device="cuda"),
+                    torch.full((1, ns[1]), float("nan"), device="cuda"), torch.full((1, ns[2]), float("nan"), device="cuda")]
+            entries = [(wd[i], bufs[i], bufs[i + 1], Q4_K, 1, ns[i], k) for i in range(3)]
+            print(f"prefetch: attempt {attempt} prefetch={backend is with_it}", flush=True)
+            run_batch(backend, torch, entries, after_previous=lambda i: i > 0)
+            outs.append([b.cpu().numpy() for b in bufs[1:]])
+        for a, b in zip(*outs):
+            assert np.isfinite(a).all()
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    # an ordinary call behind the batches on the same stream
+    x = torch.from_numpy(random_activations(1, k, seed=90)).cuda()
+    ya, yb = torch.empty(1, ns[2], device="cuda"), torch.empty(1, ns[2], device="cuda")
+    with_it.quantized_matmul(wd[2], x, ya, Q4_K, 1, ns[2], k)
+    without.quantized_matmul(wd[2], x, yb, Q4_K, 1, ns[2], k)
+    torch.cuda.synchronize()
+    assert torch.equal(ya.view(torch.int32), yb.view(torch.int32))
