@@ -1277,11 +1277,11 @@ int run_chain(gllmq_ctx *ctx, Scratch &S, const gllmq_matmul_desc *descs, size_t
     P.lds_ctrl = (prep.red + 15u) & ~15u;
     const uint32_t red = P.lds_ctrl + static_cast<uint32_t>(sizeof(gq::Mm8sCtrl)) + gq::MM8C_MAX_SLOTS * 4u;
     P.lds_ring = (red + gq::MM8C_RED_BUFS * gq::MM8C_CWAVES * 64u * 4u + 1023u) & ~1023u;
-    P.depth = ctx->mm8s_depth ? std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth) : 1u; // as for the single launches of one or two rows
+    P.depth = ctx->mm8s_depth ? std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth) : 0u; // 0: by the entry's items, see the loader
     if (P.lds_ring >= 160u * 1024u) return -1;
     uint32_t slots = std::min(gq::MM8C_MAX_SLOTS, (160u * 1024u - P.lds_ring) / P.slot_bytes);
     slots -= slots % gq::MM8C_LOADERS;
-    if (slots < gq::mm8s_min_slots(P.depth)) return -1;
+    if (slots < gq::mm8s_min_slots(std::max(2u, P.depth))) return -1;
     P.ring_slots = slots;
     P.spin_limit = ctx->chain_spin_limit;
     P.epoch0 = ctx->chain_epoch;
