@@ -52,7 +52,7 @@ MAX_TIMED_STEPS = 400_000
 # under rocprofv3 (FETCH_SIZE, then WRITE_SIZE, per dispatch), each scaled by what the same
 # counter reads for a plain copy of known size; the summary sits in profiles/ beside the
 # kernel trace.
-TRAFFIC_BYTES_PER_LAUNCH = 33_357_200
+TRAFFIC_BYTES_PER_LAUNCH = 33_374_000
 TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a plain copy (profiles/)"
 
 
