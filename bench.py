@@ -200,7 +200,7 @@ def workload_result(args, name, want_cpu):
         return region
 
     if name in ("gemv_q4k_4096", "gemv_q6k", "gemm_m16", "gemm_m32", "gemm_m64", "layer_mix", "layer_mix_m4", "layer_mix_m32",
-                "lm_head_q6k", "down_q6k", "down_q4k", "down_q6k_m2", "down_q4k_m4", "gemv_q8_0", "gemv_q5k"):
+                "lm_head_q6k", "down_q6k", "down_q4k", "down_q6k_m2", "down_q4k_m4", "gemv_q8_0", "gemv_q5k", "qkv_q4k", "down_q5k"):
         if name.startswith("layer_mix"):
             mm = int(name.split("_m")[2]) if name.count("_m") == 2 else 1  # decode, or batched decode of 4 / 32 sequences
             ops = [(12, 6144, 4096, mm), (12, 4096, 4096, mm), (12, 2 * 14336, 4096, mm), (14, 4096, 14336, mm)]
@@ -211,7 +211,9 @@ def workload_result(args, name, want_cpu):
                               "gemm_m16": (12, 14336, 4096, 16), "gemm_m32": (12, 14336, 4096, 32),
                               "gemm_m64": (12, 14336, 4096, 64),
                               # the down projection of the layer: few weight rows (16 per CU), long rows
-                              "down_q6k": (14, 4096, 14336, 1), "down_q4k": (12, 4096, 14336, 1),
+                              "down_q6k": (14, 4096, 14336, 1), "down_q4k": (12, 4096, 14336, 1), "down_q5k": (13, 4096, 14336, 1),
+                              # the fused Q, K and V projection of the layer: 24 weight rows per CU
+                              "qkv_q4k": (12, 6144, 4096, 1),
                               "down_q6k_m2": (14, 4096, 14336, 2), "down_q4k_m4": (12, 4096, 14336, 4),
                               # the output projection of a 128256-token vocabulary: Q6_K even in Q4 files
                               "lm_head_q6k": (14, 128256, 4096, 1)}[name]
@@ -506,7 +508,7 @@ def main():
     ap.add_argument("--no-context", action="store_true",
                     help="skip the cache-resident and copy-rate context runs (profiling: only the timed kernel launches)")
     ap.add_argument("--workload", default="gemv_q4k",
-                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q5k, gemv_q6k, gemv_q8_0, layer_mix, layer_mix_m4, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, down_q6k, down_q4k, down_q6k_m2, down_q4k_m4, lm_head_q6k, lm_head_argmax_q6k, lm_head_then_argmax_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
+                    help="gemv_q4k (headline, default), gemv_q4k_4096, gemv_q5k, gemv_q6k, gemv_q8_0, layer_mix, layer_mix_m4, layer_mix_m32, gemm_m16, gemm_m32, gemm_m64, qkv_q4k, down_q6k, down_q4k, down_q5k, down_q6k_m2, down_q4k_m4, lm_head_q6k, lm_head_argmax_q6k, lm_head_then_argmax_q6k, ffn_m1, ffn_m4, ffn_m32, moe, "
                          "dequant_q4k, dequant_q5k, dequant_q6k, dequant_q8_0, gather_q4k, gather_q6k, gather_q8_0")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="kernel-family option of the library for this run (repeatable), e.g. mm8s=0")

@@ -692,10 +692,11 @@ int run_mm8s(gllmq_ctx *ctx, const Format &f, const uint8_t *w, const float *x, 
     // against 55.4, two rows of Q6_K 4096 -> 14336 12.7 against 13.4).  Three and four rows, whose
     // arithmetic per item is longer, keep about MM8S_DEPTH_BYTES worth of items on their way
     // (three rows 4096 -> 6144: 6.6 against 6.9 us with one), fewer when a reused ring is too short.
-    // Pairs of Q4_K blocks of a long row (4.5 KiB an item, its 32 pieces of 144 bytes a whole row or
-    // eight blocks apart) come in late enough for two: 14336 -> 4096 9.1 against 10.1 us (Q6_K
-    // pairs, 6.6 KiB: 13.6 against 13.3).
-    uint32_t depth = pi == 0 ? ((fold && item_bytes <= 5120u) ? 2u : 1u)
+    // Pairs of Q4_K or Q5_K blocks of a long row (4.5 and 5.5 KiB an item, its 32 pieces a whole row
+    // or eight blocks apart) come in late enough for two: 14336 -> 4096 Q4_K 9.1 against 10.1 us,
+    // Q5_K 11.0 against 11.5 (Q6_K pairs, 6.6 KiB: 13.6 against 13.3; whole blocks of 24 rows,
+    // 4096 -> 6144: 5.46 against 5.41).
+    uint32_t depth = pi == 0 ? ((fold && item_bytes < 6144u) ? 2u : 1u)
                              : std::min(gq::MM8S_MAX_DEPTH, std::max(2u, (gq::MM8S_DEPTH_BYTES + item_bytes / 2u) / item_bytes));
     if (ctx->mm8s_depth) depth = std::min(gq::MM8S_MAX_DEPTH, ctx->mm8s_depth);
     while (depth > (split ? 1u : 2u) && slots < items && slots < gq::mm8s_min_slots(depth)) --depth;
