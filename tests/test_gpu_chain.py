@@ -307,3 +307,29 @@ def test_the_weight_prefetch_beside_dependent_launches_changes_no_bit(torch):
     without.quantized_matmul(wd[2], x, yb, Q4_K, 1, ns[2], k)
     torch.cuda.synchronize()
     assert torch.equal(ya.view(torch.int32), yb.view(torch.int32))
+
+
+@pytest.mark.parametrize("dtype,m", [(Q4_K, 1), (Q5_K, 2), (Q8_0, 1)])
+def test_open_requests_per_loader_change_no_bit(torch, dtype, m):
+    """By default a loader of the chained launch keeps one item open on entries of full tiles and
+    two on entries of low tiles or paired blocks; whatever number it is told to keep, and however
+    often it stands before a taken slot and counts its open requests in there, the results are
+    the same bits."""
+    from gllm_amd.backend import HipBackend
+    c, k = cus(torch), 4096
+    ns = [24 * c, 16 * c, 112 * c + 5, 8 * c, 56 * c + 31, 16 * c, 24 * c + 3]
+    host = [(random_weight(dtype, n, k, seed=40 + i), random_activations(m, k, seed=50 + i)) for i, n in enumerate(ns)]
+    outs = []
+    for depth in (0, 1, 2, 3, 4):
+        backend = HipBackend(0, options={"mm8s_depth": depth})
+        entries = [(dev_weight(torch, w), torch.from_numpy(x).cuda(), torch.full((m, n), float("nan"), device="cuda"), dtype, m, n, k)
+                   for (w, x), n in zip(host, ns)]
+        print(f"chain: open requests dtype={dtype} m={m} depth={depth}", flush=True)
+        run_batch(backend, torch, entries, after_previous=None)
+        # (a ring too short for the number asked for sends the entries to single launches: the same bits)
+        if depth <= 2:
+            assert backend.last_kernel_name().startswith("gq_mm8c_"), backend.last_kernel_name()
+        outs.append([e[2].cpu().numpy() for e in entries])
+    for depth, out in enumerate(outs[1:], 1):
+        for i in range(len(ns)):
+            assert np.array_equal(out[i].view(np.uint32), outs[0][i].view(np.uint32)), f"entry {i}, depth {depth}"

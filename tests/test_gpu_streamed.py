@@ -199,3 +199,26 @@ def test_default_choice_of_form(torch):
         a = gpu_matmul(default, torch, w, x, dtype, m, n, k)
         assert default.last_kernel_name().startswith("gq_mm8s_") == streamed, default.last_kernel_name()
         check_close(a, gpu_matmul(plain, torch, w, x, dtype, m, n, k), f"default form dtype={dtype} m={m} n={n} k={k}")
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q5_K, Q6_K])
+def test_more_open_requests_per_loader_change_no_bit(hip, torch, dtype):
+    """A loader wave keeps one or two items open by default (two for pairs of Q4_K / Q5_K blocks of
+    a long row).  With up to four, on long rows whose ring is short beside them, a loader stands
+    before taken slots most of the time and counts its open requests in there: every item must
+    still be seen by its arithmetic wave, complete, whatever the depth."""
+    from gllm_amd.backend import HipBackend
+    c = cus(torch)
+    for m, n, k in ((1, 16 * c, 14336), (1, 16 * c + 5, 8192 + 256), (2, 32 * c, 8192), (1, 56 * c, 4096), (4, 40 * c, 2048)):
+        if dtype == Q6_K and m > 2:
+            continue
+        w, x = random_weight(dtype, n, k, seed=n + k), random_activations(m, k, seed=m)
+        base = gpu_matmul(hip, torch, w, x, dtype, m, n, k)
+        name = hip.last_kernel_name()
+        assert name.startswith("gq_mm8s_"), name
+        for depth in (1, 2, 3, 4):
+            print(f"open requests dtype={dtype} m={m} n={n} k={k} depth={depth}", flush=True)
+            deep = HipBackend(0, options={"mm8s_all": 1, "mm8s_split": 0, "mm8s_depth": depth})
+            got = gpu_matmul(deep, torch, w, x, dtype, m, n, k)
+            assert deep.last_kernel_name() == name
+            assert np.array_equal(got.view(np.uint32), base.view(np.uint32)), (dtype, m, n, k, depth)
