@@ -282,3 +282,28 @@ def test_moe_error_behaviour(hip, torch):
     zw = torch.zeros(8, dtype=torch.float32, device="cuda").reshape(4, 2)
     with pytest.raises(Unimplemented):
         hip.moe_matvec(z, 2, z, Q6_K, z, z, 256, 256, 4, zi, zw, zl)  # Q4_0 gate/up: not covered
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_moe_shapes_from_a_seeded_generator(hip, torch, oracle, seed):
+    """Experts, tokens, routes per token, capacity, widths and formats drawn from a seeded
+    generator: jobs of one to many tokens, experts nobody is routed to, dropped routes, rows of
+    one to eight blocks, expert matrices too low for the grouped matrix-core kernels."""
+    rng = np.random.default_rng(seed)
+    for i in range(12):
+        experts = int(rng.choice([2, 4, 8, 16, 24, 40]))
+        tokens = int(rng.choice([1, 2, 5, 9, 16, 33]))
+        top_k = int(rng.integers(1, min(4, experts) + 1))
+        hidden = 256 * int(rng.choice([1, 2, 3, 4, 8]))
+        ffn = 256 * int(rng.choice([1, 2, 3, 6]))
+        dt_gu, dt_dn = int(rng.choice([Q4_K, Q5_K, Q6_K, Q8_0])), int(rng.choice([Q4_K, Q5_K, Q6_K, Q8_0]))
+        capacity = float(rng.choice([0.5, 1.25, float(experts)]))
+        relu = bool(rng.integers(0, 2))
+        print(f"moe seeded {seed}/{i}: experts={experts} tokens={tokens} top_k={top_k} hidden={hidden} ffn={ffn} "
+              f"gu={dt_gu} dn={dt_dn} capacity={capacity} relu={relu}", flush=True)
+        gu, dn = expert_weights(dt_gu, dt_dn, experts, hidden, ffn, seed=seed * 100 + i)
+        x = random_activations(tokens, hidden, seed=seed * 300 + i)
+        dev, r = route_gpu(hip, torch, oracle, random_gate_logits(tokens, experts, seed=seed * 500 + i), top_k, capacity)
+        want = oracle.moe_ffn(gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, r["expert"], r["weight"], r["len"], relu_gate=relu)
+        got = run_gpu(hip, torch, gu, dt_gu, dn, dt_dn, x, hidden, ffn, experts, *dev, relu_gate=relu, split=bool(i & 1))
+        check_close(got, want, f"moe seeded {seed}/{i}")
