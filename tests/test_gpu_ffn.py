@@ -166,3 +166,29 @@ def test_ffn_argument_errors(hip, torch):
     hip.ffn_swiglu(w, w, Q4_K, w, Q4_K, x, out, 0, 256, 64)       # no rows: nothing written
     torch.cuda.synchronize()
     assert bool(torch.all(out == 7.0))
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_ffn_shapes_from_a_seeded_generator(hip, torch, oracle, seed):
+    """Rows, widths, formats, the ReLU gate and stacked or separate gate/up tensors drawn from a
+    seeded generator: every path of the block (gated kernels, gated activation loads of the down
+    projection for one to eight rows, the activation launch, the GEMMs) at sizes nobody chose."""
+    rng = np.random.default_rng(seed)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    seen = set()
+    for i in range(14):
+        t_gu, t_dn = int(rng.choice(ALL)), int(rng.choice(ALL))
+        m = int(rng.choice([1, 1, 2, 3, 4, 6, 8, 9, 16, 20]))
+        hidden = 256 * int(rng.choice([2, 4, 8, 16]))
+        ffn = 256 * int(rng.choice([1, 3, 6, 11, 14])) if rng.integers(0, 2) else int(rng.choice([8, 16, 33])) * cus
+        ffn = max(256, (ffn // 256) * 256)  # the down projection's rows are whole blocks here
+        relu = bool(rng.integers(0, 2))
+        print(f"ffn seeded {seed}/{i}: gu={t_gu} dn={t_dn} m={m} hidden={hidden} ffn={ffn} relu={relu}", flush=True)
+        gate, up = random_weight(t_gu, ffn, hidden, seed=seed * 10 + i), random_weight(t_gu, ffn, hidden, seed=seed * 20 + i)
+        down = random_weight(t_dn, hidden, ffn, seed=seed * 30 + i)
+        x = random_activations(m, hidden, seed=seed * 40 + i)
+        want = oracle.ffn_swiglu(gate, up, t_gu, down, t_dn, x, m, hidden, ffn, relu_gate=relu, acc=oracle.ACC_F64, threads=16)
+        got = run_ffn(hip, torch, gate, up, t_gu, down, t_dn, x, m, hidden, ffn, relu=relu, stacked=bool(i & 1))
+        check(got, want, f"ffn seeded {seed}/{i} kernel={hip.last_kernel_name()}")
+        seen.add(hip.last_kernel_name())
+    print("last kernels met:", sorted(seen), flush=True)
